@@ -1,0 +1,337 @@
+/*
+ * thgpu.h -- C ABI of libthgpu, the MI355X (gfx950) implementation of the
+ * gputorch/gpunn convolution hot path: THGPUStorage / THGPUTensor on hipMalloc
+ * memory, THGPUBlas_gemm on fp32 MFMA, batched im2col / col2im,
+ * nn.SpatialConvolutionMM, nn.SpatialMaxPooling and nn.Threshold forward and
+ * backward.
+ *
+ * Plain C: pointers, sizes and the two TH structs whose layout LuaJIT FFI code
+ * reads directly (gputorch/FFI.lua:5-29).  Every declaration cites the
+ * reference interface it replaces (paths relative to the reference tree).
+ *
+ * Conventions
+ *  - `data` of a THGPUStorage is a DEVICE pointer (hipMalloc); `allocator` and
+ *    `allocatorContext` are unused and NULL.
+ *  - All device work is enqueued on one library-owned HIP stream.  Functions
+ *    that hand data to the host (get, copies to host, thgpu_synchronize)
+ *    block until the stream has drained; everything else returns as soon as
+ *    the work is enqueued.  Not thread-safe, like the reference.
+ *  - TH-named functions return void/values as in the reference and report
+ *    errors through the installable handler (THGPUSetErrorHandler), which
+ *    mirrors THSetErrorHandler / THSetArgErrorHandler (TH/THGeneral.c:7-65).
+ *    thgpu_* functions return 0 on success or a non-zero status and leave a
+ *    message in thgpu_last_error(); they never call the handler.
+ */
+#ifndef THGPU_H
+#define THGPU_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- struct layouts (ABI) ------------------------------------------------ */
+
+typedef struct THAllocator THAllocator; /* opaque, never dereferenced here */
+
+#define TH_STORAGE_REFCOUNTED 1 /* TH/generic/THStorage.h:19-21 */
+#define TH_STORAGE_RESIZABLE 2
+#define TH_STORAGE_FREEMEM 4
+#define TH_TENSOR_REFCOUNTED 1 /* gputorch/lib/THC/THCTensor.h:16 */
+
+/* TH/generic/THStorage.h:23-31 instantiated with real=float, Real=GPU by
+ * gputorch/lib/THC/THCStorage.h:10-20; FFI view gputorch/FFI.lua:6-14. */
+typedef struct THGPUStorage {
+    float *data; /* device pointer */
+    long size;
+    int refcount;
+    char flag;
+    THAllocator *allocator;
+    void *allocatorContext;
+} THGPUStorage;
+
+/* gputorch/lib/THC/THCTensor.h:18-50 (data members only); FFI view
+ * gputorch/FFI.lua:16-28. */
+typedef struct THGPUTensor {
+    long *size;
+    long *stride;
+    int nDimension;
+    THGPUStorage *storage;
+    long storageOffset;
+    int refcount;
+    char flag;
+} THGPUTensor;
+
+/* Host-side TH types that appear in the copy signatures.  Same layouts
+ * (TH/generic/THStorage.h:23-31, TH/generic/THTensor.h), host pointers. */
+#define THGPU_DECLARE_HOST_TYPES(Name, ctype)                                              \
+    typedef struct TH##Name##Storage {                                                     \
+        ctype *data;                                                                       \
+        long size;                                                                         \
+        int refcount;                                                                      \
+        char flag;                                                                         \
+        THAllocator *allocator;                                                            \
+        void *allocatorContext;                                                            \
+    } TH##Name##Storage;                                                                   \
+    typedef struct TH##Name##Tensor {                                                      \
+        long *size;                                                                        \
+        long *stride;                                                                      \
+        int nDimension;                                                                    \
+        TH##Name##Storage *storage;                                                        \
+        long storageOffset;                                                                \
+        int refcount;                                                                      \
+        char flag;                                                                         \
+    } TH##Name##Tensor;
+THGPU_DECLARE_HOST_TYPES(Byte, unsigned char)
+THGPU_DECLARE_HOST_TYPES(Char, char)
+THGPU_DECLARE_HOST_TYPES(Short, short)
+THGPU_DECLARE_HOST_TYPES(Int, int)
+THGPU_DECLARE_HOST_TYPES(Long, long)
+THGPU_DECLARE_HOST_TYPES(Float, float)
+THGPU_DECLARE_HOST_TYPES(Double, double)
+
+/* ---- runtime --------------------------------------------------------------- */
+
+/* Error handler, replacing THSetErrorHandler/THSetArgErrorHandler
+ * (TH/THGeneral.c:16-65) and __THGPUCheck (gputorch/lib/THC/THCGeneral.cpp:
+ * 17-24).  The default handler prints the message and exits, as TH's default
+ * does (TH/THGeneral.c:7-11,40-47).  A handler that returns makes the failing
+ * TH-named function return early without touching its arguments. */
+typedef void (*THGPUErrorHandler)(const char *msg, void *data);
+void THGPUSetErrorHandler(THGPUErrorHandler handler, void *data);
+
+/* Message of the most recent failure (empty string if none). */
+const char *thgpu_last_error(void);
+
+/* Selects device 0, creates the library stream.  Called lazily by everything
+ * else; explicit call returns non-zero if no usable GPU is present. */
+int thgpu_init(void);
+
+/* Real stream synchronisation, replacing the no-op gputorch.synchronize
+ * (gputorch/init.cpp:10-14). */
+int thgpu_synchronize(void);
+
+/* Device name / compute-unit count / total memory, replacing the stubbed
+ * getDeviceProperties (gputorch/init.cpp:40-66). */
+int thgpu_device_info(char *name, long name_cap, int *compute_units, long *total_mem_bytes);
+
+/* Timing on the library stream (the reference brackets ops with torch.Timer
+ * around the no-op synchronize, gpunn/test/test.lua:2823-2831).  Events are
+ * small integer handles. */
+int thgpu_event_create(void);
+int thgpu_event_record(int ev);
+int thgpu_event_elapsed_ms(int ev_start, int ev_stop, float *ms); /* synchronises on ev_stop */
+
+/* Per-kernel timing: while enabled every kernel launch of the library is
+ * bracketed by HIP events on the library stream.  The report is a JSON object
+ * {"kernel name": {"calls": n, "ms": total, "flops": total, "bytes": total}}
+ * with the algorithmic flops/bytes the launch sites declare. */
+int thgpu_prof_enable(int on);
+int thgpu_prof_reset(void);
+long thgpu_prof_report(char *buf, long cap); /* returns the length needed */
+
+/* Host-only self check of the index arithmetic the kernels rely on (magic-number
+ * division against the C operators over a sweep of divisors and dividends).
+ * Needs no GPU.  Returns the number of mismatches. */
+long thgpu_selftest_index_math(void);
+
+/* ---- THGPUStorage: TH/generic/THStorage.h:33-65 instantiated for GPU,
+ *      implementation replaced: gputorch/lib/THC/THCStorage.cpp:7-198 -------- */
+float *THGPUStorage_data(const THGPUStorage *self);
+long THGPUStorage_size(const THGPUStorage *self);
+void THGPUStorage_set(THGPUStorage *self, long index, float value);  /* THCStorage.cpp:7-12, blocking */
+float THGPUStorage_get(const THGPUStorage *self, long index);        /* THCStorage.cpp:14-21, blocking */
+THGPUStorage *THGPUStorage_new(void);                                 /* THCStorage.cpp:23-34 */
+THGPUStorage *THGPUStorage_newWithSize(long size);                    /* THCStorage.cpp:36-57 */
+THGPUStorage *THGPUStorage_newWithSize1(float);                       /* THCStorage.cpp:59-64 */
+THGPUStorage *THGPUStorage_newWithSize2(float, float);                /* THCStorage.cpp:66-72 */
+THGPUStorage *THGPUStorage_newWithSize3(float, float, float);         /* THCStorage.cpp:74-81 */
+THGPUStorage *THGPUStorage_newWithSize4(float, float, float, float);  /* THCStorage.cpp:83-91 */
+THGPUStorage *THGPUStorage_newWithMapping(const char *filename, long size, int shared); /* error, THCStorage.cpp:93-97 */
+/* `data` is a HOST pointer (THCStorage.cpp:99-110); its contents are uploaded. */
+THGPUStorage *THGPUStorage_newWithData(float *data, long size);
+void THGPUStorage_setFlag(THGPUStorage *self, const char flag);
+void THGPUStorage_clearFlag(THGPUStorage *self, const char flag);
+void THGPUStorage_retain(THGPUStorage *self);                         /* THCStorage.cpp:112-116 */
+void THGPUStorage_free(THGPUStorage *self);                           /* THCStorage.cpp:118-140 */
+void THGPUStorage_resize(THGPUStorage *self, long size);              /* THCStorage.cpp:154-198: new buffer, D2D copy of min(old,new) */
+void THGPUStorage_fill(THGPUStorage *self, float value);              /* THCStorage.cpp:142-152 */
+
+/* gputorch/lib/THC/THCStorageCopy.h:9-26, THCStorageCopy.cpp:5-75 */
+void THGPUStorage_rawCopy(THGPUStorage *self, float *src); /* src is a DEVICE pointer (THCStorageCopy.cpp:56-62) */
+void THGPUStorage_copy(THGPUStorage *self, THGPUStorage *src);
+void THGPUStorage_copyGPU(THGPUStorage *self, THGPUStorage *src);
+void THGPUStorage_copyByte(THGPUStorage *self, struct THByteStorage *src);
+void THGPUStorage_copyChar(THGPUStorage *self, struct THCharStorage *src);
+void THGPUStorage_copyShort(THGPUStorage *self, struct THShortStorage *src);
+void THGPUStorage_copyInt(THGPUStorage *self, struct THIntStorage *src);
+void THGPUStorage_copyLong(THGPUStorage *self, struct THLongStorage *src);
+void THGPUStorage_copyFloat(THGPUStorage *self, struct THFloatStorage *src);
+void THGPUStorage_copyDouble(THGPUStorage *self, struct THDoubleStorage *src);
+void THByteStorage_copyGPU(THByteStorage *self, struct THGPUStorage *src);
+void THCharStorage_copyGPU(THCharStorage *self, struct THGPUStorage *src);
+void THShortStorage_copyGPU(THShortStorage *self, struct THGPUStorage *src);
+void THIntStorage_copyGPU(THIntStorage *self, struct THGPUStorage *src);
+void THLongStorage_copyGPU(THLongStorage *self, struct THGPUStorage *src);
+void THFloatStorage_copyGPU(THFloatStorage *self, struct THGPUStorage *src);
+void THDoubleStorage_copyGPU(THDoubleStorage *self, struct THGPUStorage *src);
+
+/* ---- THGPUTensor: gputorch/lib/THC/THCTensor.h:53-152,
+ *      implementation replaced: gputorch/lib/THC/THCTensor.cpp ---------------- */
+THGPUStorage *THGPUTensor_storage(const THGPUTensor *self);
+long THGPUTensor_storageOffset(const THGPUTensor *self);
+int THGPUTensor_nDimension(const THGPUTensor *self);
+long THGPUTensor_size(const THGPUTensor *self, int dim);
+long THGPUTensor_stride(const THGPUTensor *self, int dim);
+THLongStorage *THGPUTensor_newSizeOf(THGPUTensor *self);
+THLongStorage *THGPUTensor_newStrideOf(THGPUTensor *self);
+float *THGPUTensor_data(const THGPUTensor *self); /* device pointer incl. storageOffset */
+void THGPUTensor_setFlag(THGPUTensor *self, const char flag);
+void THGPUTensor_clearFlag(THGPUTensor *self, const char flag);
+
+THGPUTensor *THGPUTensor_new(void);
+THGPUTensor *THGPUTensor_newWithTensor(THGPUTensor *tensor);
+THGPUTensor *THGPUTensor_newWithStorage(THGPUStorage *storage, long storageOffset, THLongStorage *size,
+                                        THLongStorage *stride); /* stride may be NULL */
+THGPUTensor *THGPUTensor_newWithStorage1d(THGPUStorage *storage, long storageOffset, long size0, long stride0);
+THGPUTensor *THGPUTensor_newWithStorage2d(THGPUStorage *storage, long storageOffset, long size0, long stride0,
+                                          long size1, long stride1);
+THGPUTensor *THGPUTensor_newWithStorage3d(THGPUStorage *storage, long storageOffset, long size0, long stride0,
+                                          long size1, long stride1, long size2, long stride2);
+THGPUTensor *THGPUTensor_newWithStorage4d(THGPUStorage *storage, long storageOffset, long size0, long stride0,
+                                          long size1, long stride1, long size2, long stride2, long size3,
+                                          long stride3);
+THGPUTensor *THGPUTensor_newWithSize(THLongStorage *size, THLongStorage *stride);
+THGPUTensor *THGPUTensor_newWithSize1d(long size0);
+THGPUTensor *THGPUTensor_newWithSize2d(long size0, long size1);
+THGPUTensor *THGPUTensor_newWithSize3d(long size0, long size1, long size2);
+THGPUTensor *THGPUTensor_newWithSize4d(long size0, long size1, long size2, long size3);
+THGPUTensor *THGPUTensor_newClone(THGPUTensor *self);                 /* THCTensor.cpp:178-184 */
+THGPUTensor *THGPUTensor_newContiguous(THGPUTensor *tensor);          /* THCTensor.cpp:186-195: self retained if contiguous */
+THGPUTensor *THGPUTensor_newSelect(THGPUTensor *tensor, int dimension, long sliceIndex);
+THGPUTensor *THGPUTensor_newNarrow(THGPUTensor *tensor, int dimension, long firstIndex, long size);
+THGPUTensor *THGPUTensor_newTranspose(THGPUTensor *tensor, int dimension1, int dimension2);
+
+void THGPUTensor_resize(THGPUTensor *tensor, THLongStorage *size, THLongStorage *stride);
+void THGPUTensor_resizeAs(THGPUTensor *tensor, THGPUTensor *src);
+void THGPUTensor_resize1d(THGPUTensor *tensor, long size0);
+void THGPUTensor_resize2d(THGPUTensor *tensor, long size0, long size1);
+void THGPUTensor_resize3d(THGPUTensor *tensor, long size0, long size1, long size2);
+void THGPUTensor_resize4d(THGPUTensor *tensor, long size0, long size1, long size2, long size3);
+void THGPUTensor_resize5d(THGPUTensor *tensor, long size0, long size1, long size2, long size3, long size4);
+
+void THGPUTensor_set(THGPUTensor *self, THGPUTensor *src);
+void THGPUTensor_setStorage(THGPUTensor *self, THGPUStorage *storage, long storageOffset, THLongStorage *size,
+                            THLongStorage *stride);
+void THGPUTensor_narrow(THGPUTensor *self, THGPUTensor *src, int dimension, long firstIndex, long size);
+void THGPUTensor_select(THGPUTensor *self, THGPUTensor *src, int dimension, long sliceIndex);
+void THGPUTensor_transpose(THGPUTensor *self, THGPUTensor *src, int dimension1, int dimension2);
+
+int THGPUTensor_isContiguous(const THGPUTensor *self);                /* THCTensor.cpp:510-525 */
+int THGPUTensor_isSameSizeAs(const THGPUTensor *self, const THGPUTensor *src);
+long THGPUTensor_nElement(const THGPUTensor *self);
+void THGPUTensor_retain(THGPUTensor *self);
+void THGPUTensor_free(THGPUTensor *self);
+void THGPUTensor_freeCopyTo(THGPUTensor *self, THGPUTensor *dst);
+
+void THGPUTensor_set1d(THGPUTensor *tensor, long x0, float value);
+void THGPUTensor_set2d(THGPUTensor *tensor, long x0, long x1, float value);
+void THGPUTensor_set3d(THGPUTensor *tensor, long x0, long x1, long x2, float value);
+void THGPUTensor_set4d(THGPUTensor *tensor, long x0, long x1, long x2, long x3, float value);
+float THGPUTensor_get1d(const THGPUTensor *tensor, long x0);
+float THGPUTensor_get2d(const THGPUTensor *tensor, long x0, long x1);
+float THGPUTensor_get3d(const THGPUTensor *tensor, long x0, long x1, long x2);
+float THGPUTensor_get4d(const THGPUTensor *tensor, long x0, long x1, long x2, long x3);
+
+/* gputorch/lib/THC/THCTensorMath.h:7-8, THCTensorMath.cpp:15-42 */
+void THGPUTensor_fill(THGPUTensor *self, float value);
+void THGPUTensor_zero(THGPUTensor *self);
+
+/* gputorch/lib/THC/THCTensorCopy.h:7-23.  copy handles any strides
+ * (THCTensorCopy.cpp:170-290); host<->device copies are blocking
+ * (THCTensorCopy.cpp:20-36,64-80). */
+void THGPUTensor_copy(THGPUTensor *self, THGPUTensor *src);
+void THGPUTensor_copyGPU(THGPUTensor *self, THGPUTensor *src);
+void THGPUTensor_copyByte(THGPUTensor *self, THByteTensor *src);
+void THGPUTensor_copyChar(THGPUTensor *self, THCharTensor *src);
+void THGPUTensor_copyShort(THGPUTensor *self, THShortTensor *src);
+void THGPUTensor_copyInt(THGPUTensor *self, THIntTensor *src);
+void THGPUTensor_copyLong(THGPUTensor *self, THLongTensor *src);
+void THGPUTensor_copyFloat(THGPUTensor *self, THFloatTensor *src);
+void THGPUTensor_copyDouble(THGPUTensor *self, THDoubleTensor *src);
+void THByteTensor_copyGPU(THByteTensor *self, THGPUTensor *src);
+void THCharTensor_copyGPU(THCharTensor *self, THGPUTensor *src);
+void THShortTensor_copyGPU(THShortTensor *self, THGPUTensor *src);
+void THIntTensor_copyGPU(THIntTensor *self, THGPUTensor *src);
+void THLongTensor_copyGPU(THLongTensor *self, THGPUTensor *src);
+void THFloatTensor_copyGPU(THFloatTensor *self, THGPUTensor *src);
+void THDoubleTensor_copyGPU(THDoubleTensor *self, THGPUTensor *src);
+
+/* ---- BLAS ------------------------------------------------------------------ */
+
+/* Column-major C = beta*C + alpha*op(A)*op(B) on DEVICE pointers: the generic
+ * THBlas signature (TH/generic/THBlas.h:17 instantiated by gputorch/lib/THC/
+ * THCBlas.h:6-14); replaces the array_view overload THCBlas.h:35-39 and its
+ * kernels THCBlas.cpp:10-288 (offsets fold into the pointers).  All four
+ * transpose variants honour lda/ldb/ldc.  Quick returns as THCBlas.cpp:257. */
+void THGPUBlas_gemm(char transa, char transb, long m, long n, long k, float alpha, float *a, long lda, float *b,
+                    long ldb, float beta, float *c, long ldc);
+
+/* ---- flat operator entry points -------------------------------------------- */
+
+/* Batched im2col: im [B,C,H,W] -> col [B, C*kH*kW, Ho*Wo] (device pointers).
+ * Replaces the per-image kernel gputorch/lib/THC/gpunn-impl/
+ * SpatialConvolutionMM.cpp:10-52; output layout and zero padding as the CPU
+ * nn_(unfolded_copy), mcw_nn/generic/SpatialConvolutionMM.c:52-96. */
+int thgpu_im2col(const float *im, long B, int C, int H, int W, int kH, int kW, int padH, int padW, int sH, int sW,
+                 float *col);
+
+/* Batched col2im gather: col [B, C*kH*kW, Ho*Wo] -> im [B,C,H,W], overwriting
+ * im.  Replaces gpunn-impl/SpatialConvolutionMM.cpp:54-108; every pixel is
+ * summed from 0 in kh-ascending, kw-ascending order, bit-matching the CPU
+ * nn_(unfolded_acc), mcw_nn/generic/SpatialConvolutionMM.c:6-50. */
+int thgpu_col2im(const float *col, long B, int C, int H, int W, int kH, int kW, int padH, int padW, int sH, int sW,
+                 float *im);
+
+/* nn.SpatialConvolutionMM.  Replace gpunn_SpatialConvolutionMM_updateOutput /
+ * _updateGradInput / _accGradParameters (gpunn-impl/SpatialConvolutionMM.cpp:
+ * 110-225, 227-311, 313-429); arguments are the module fields those read by
+ * name (:116-128) with the single `padding` split into padW/padH.  input is
+ * [C,H,W] or [B,C,H,W] contiguous and is never modified; weight is
+ * [M, C*kH*kW].  Buffer semantics follow the CPU module, the parity target
+ * (mcw_nn/generic/SpatialConvolutionMM.c:179,243,318): finput is resized to
+ * [B,K,N] and keeps the whole batch of columns, fgradInput likewise holds the
+ * column gradients, and accGradParameters reuses finput from the preceding
+ * updateOutput without recomputing it. */
+int thgpu_SpatialConvolutionMM_updateOutput(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias,
+                                            THGPUTensor *finput, THGPUTensor *fgradInput, THGPUTensor *output,
+                                            int kW, int kH, int dW, int dH, int padW, int padH);
+int thgpu_SpatialConvolutionMM_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *weight,
+                                               THGPUTensor *finput, THGPUTensor *fgradInput,
+                                               THGPUTensor *gradInput, int kW, int kH, int dW, int dH, int padW,
+                                               int padH);
+int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor *gradOutput,
+                                                 THGPUTensor *gradWeight, THGPUTensor *gradBias,
+                                                 THGPUTensor *finput, THGPUTensor *fgradInput, int kW, int kH,
+                                                 int dW, int dH, int padW, int padH, float scale);
+
+/* nn.SpatialMaxPooling.  Replace gpunn_SpatialMaxPooling_updateOutput /
+ * _updateGradInput (gpunn-impl/SpatialMaxPooling.cpp:205-281, 283-383).
+ * indices is resized to [2,(B,)C,Ho,Wo] floats, plane 0 = ky+1, plane 1 = kx+1
+ * (mcw_nn/generic/SpatialMaxPooling.c:51-52,133-134).  Backward accepts
+ * overlapping windows (the reference GPU code rejects dW!=kW, :293-294) and
+ * adds in the CPU order (mcw_nn/generic/SpatialMaxPooling.c:165-174). */
+int thgpu_SpatialMaxPooling_updateOutput(THGPUTensor *input, THGPUTensor *output, THGPUTensor *indices, int kW,
+                                         int kH, int dW, int dH);
+int thgpu_SpatialMaxPooling_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *gradInput,
+                                            THGPUTensor *indices, int kW, int kH, int dW, int dH);
+
+/* nn.Threshold / nn.ReLU.  Replace gpunn_Threshold_updateOutput /
+ * _updateGradInput (gpunn-impl/Threshold.cpp:16-38, 53-81). */
+int thgpu_Threshold_updateOutput(THGPUTensor *input, THGPUTensor *output, float threshold, float val);
+int thgpu_Threshold_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *gradInput,
+                                    float threshold);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* THGPU_H */

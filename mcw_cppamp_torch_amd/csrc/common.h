@@ -1,0 +1,106 @@
+// Internal helpers shared by the libthgpu sources: error plumbing, the library
+// stream, launch bracketing for per-kernel timing, magic-number division.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/thgpu.h"
+
+namespace thgpu {
+
+// ---- errors -----------------------------------------------------------------
+// Records a message for thgpu_last_error(); returns a non-zero status so that
+// `return fail(...)` reads naturally in the flat entry points.
+int fail(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+// Records the message and calls the installed TH-style handler.
+void raise(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+
+#define THGPU_HIP_TRY(expr)                                                                       \
+    do {                                                                                          \
+        hipError_t _e = (expr);                                                                   \
+        if (_e != hipSuccess)                                                                     \
+            return ::thgpu::fail("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, \
+                                 __LINE__);                                                       \
+    } while (0)
+
+// For TH-named functions (void or value returning): raise through the handler
+// and return `ret` if the handler comes back.
+#define THGPU_ARGCHECK(cond, argn, msg, ret)                         \
+    do {                                                             \
+        if (!(cond)) {                                               \
+            ::thgpu::raise("bad argument #%d: %s", (argn), (msg));   \
+            return ret;                                              \
+        }                                                            \
+    } while (0)
+
+#define THGPU_HIP_CHECK_RAISE(expr, ret)                                                           \
+    do {                                                                                           \
+        hipError_t _e = (expr);                                                                    \
+        if (_e != hipSuccess) {                                                                    \
+            ::thgpu::raise("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, __LINE__); \
+            return ret;                                                                            \
+        }                                                                                          \
+    } while (0)
+
+// ---- runtime ----------------------------------------------------------------
+// Library stream (created on first use).  nullptr means initialisation failed
+// and the error is recorded.
+hipStream_t stream();
+// Grow-only device scratch for split reductions; stream-ordered with the
+// kernels that use it because everything runs on the one library stream.
+float *workspace(size_t bytes);
+int num_cus();
+
+// Brackets one kernel launch with events when per-kernel timing is enabled.
+struct LaunchScope {
+    LaunchScope(const char *name, double flops, double bytes);
+    ~LaunchScope();
+    int slot;
+};
+
+// Checks the launch itself (bad configuration shows up here, not at sync).
+int check_launch(const char *name);
+
+// ---- raw device helpers (storage.hip) -----------------------------------------
+int fill_device(float *p, long n, float v);           // async on the library stream
+int copy_h2d(float *dst, const float *src, long n);   // blocking
+int copy_d2h(float *dst, const float *src, long n);   // blocking
+int copy_d2d(float *dst, const float *src, long n);   // async on the library stream
+
+// ---- unsigned division by a run-time constant ---------------------------------
+// q = n / d for 0 <= n < 2^31, 1 <= d < 2^31 via one mul-hi and a shift.
+struct FastDiv {
+    uint32_t d, mul, shr;
+    FastDiv() : d(1), mul(0), shr(0) {}
+    explicit FastDiv(uint32_t div) : d(div) {
+        if (div == 1) { mul = 0; shr = 0; return; }
+        uint32_t l = 0;
+        while ((1ull << l) < div) ++l;                      // ceil(log2 d), >= 1 here
+        // Round-up method: the 33-bit multiplier ceil(2^(32+l)/d) lies in
+        // [2^32, 2^33); its low 32 bits are kept and the implicit top bit is
+        // folded into the (n - t)/2 + t step of div().
+        uint64_t mm = ((1ull << (32 + l)) + div - 1) / div;
+        mul = (uint32_t)(mm - (1ull << 32));
+        shr = l;
+    }
+    __host__ __device__ inline uint32_t div(uint32_t n) const {
+        if (d == 1) return n;
+#if defined(__HIP_DEVICE_COMPILE__)
+        uint32_t t = __umulhi(n, mul);
+#else
+        uint32_t t = (uint32_t)(((uint64_t)n * mul) >> 32);
+#endif
+        // (n + t) may overflow 32 bits: use the standard overflow-free form
+        return (((n - t) >> 1) + t) >> (shr - 1);
+    }
+    __host__ __device__ inline void divmod(uint32_t n, uint32_t &q, uint32_t &r) const {
+        q = div(n);
+        r = n - q * d;
+    }
+};
+
+}  // namespace thgpu

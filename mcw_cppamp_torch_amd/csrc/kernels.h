@@ -1,0 +1,21 @@
+// Launchers of the hot-path kernels (all enqueue on the library stream and
+// return 0 or a recorded error).
+#pragma once
+
+#include "common.h"
+
+namespace thgpu {
+
+int im2col_launch(const float *im, long B, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW,
+                  float *col);
+int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW,
+                  float *im);
+int maxpool_fwd_launch(const float *in, long planes, int H, int W, int kH, int kW, int dH, int dW, float *out,
+                       float *indices);
+int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int H, int W, int Ho, int Wo, int kH,
+                       int kW, int dH, int dW, float *gin);
+int threshold_fwd_launch(const float *in, float *out, long n, float th, float val);
+int threshold_bwd_launch(const float *in, const float *gout, float *gin, long n, float th);
+int gradbias_launch(const float *gout, float *gbias, long B, int M, long N, float scale);
+
+}  // namespace thgpu

@@ -1,0 +1,321 @@
+// Operator entry points on THGPUTensor arguments: nn.SpatialConvolutionMM,
+// nn.SpatialMaxPooling, nn.Threshold.  These are what the luaT bindings of the
+// reference do after unpacking the module table
+// (gputorch/lib/THC/gpunn-impl/SpatialConvolutionMM.cpp:110-429,
+//  SpatialMaxPooling.cpp:205-383, Threshold.cpp:16-81): check shapes, resize
+// the module's buffers, launch.  One launch per kernel for the whole batch
+// instead of the reference's per-image loops.
+#include "gemm_mfma.h"
+#include "kernels.h"
+
+using namespace thgpu;
+
+namespace {
+
+struct ConvShape {
+    long B;
+    int C, H, W, M, K, Ho, Wo;
+    long N;
+    bool batched;
+};
+
+// Common argument checks.  Messages follow the reference's luaL_argcheck /
+// THArgCheck texts where it has one.
+int conv_shape(ConvShape &s, const THGPUTensor *input, const THGPUTensor *weight, int kW, int kH, int dW, int dH,
+               int padW, int padH) {
+    if (!input || !weight) return fail("SpatialConvolutionMM: null tensor");
+    if (!(input->nDimension == 3 || input->nDimension == 4)) return fail("3D or 4D (batch mode) tensor is expected");
+    if (kW <= 0 || kH <= 0 || dW <= 0 || dH <= 0 || padW < 0 || padH < 0)
+        return fail("SpatialConvolutionMM: invalid kernel/stride/padding");
+    if (weight->nDimension != 2) return fail("SpatialConvolutionMM: weight must be 2D [nOutputPlane, nInputPlane*kH*kW]");
+    s.batched = input->nDimension == 4;
+    const int o = s.batched ? 1 : 0;
+    s.B = s.batched ? input->size[0] : 1;
+    s.C = (int)input->size[o];
+    s.H = (int)input->size[o + 1];
+    s.W = (int)input->size[o + 2];
+    s.M = (int)weight->size[0];
+    s.K = s.C * kH * kW;
+    if (weight->size[1] != s.K) return fail("input channels and nInputPlane dont match");
+    if (s.H + 2 * padH < kH || s.W + 2 * padW < kW) return fail("SpatialConvolutionMM: input image smaller than kernel size");
+    s.Ho = (s.H + 2 * padH - kH) / dH + 1;
+    s.Wo = (s.W + 2 * padW - kW) / dW + 1;
+    s.N = (long)s.Ho * s.Wo;
+    if (s.B * s.N >= (1L << 31)) return fail("SpatialConvolutionMM: batch*outputHeight*outputWidth exceeds 2^31");
+    return 0;
+}
+
+int require_contiguous(const THGPUTensor *t, const char *what) {
+    if (!THGPUTensor_isContiguous(t)) return fail("SpatialConvolutionMM: %s must be contiguous", what);
+    return 0;
+}
+
+int check_grad_output(const ConvShape &s, const THGPUTensor *gradOutput) {
+    if (gradOutput->nDimension != (s.batched ? 4 : 3))
+        return fail("SpatialConvolutionMM: gradOutput must have as many dimensions as the output");
+    const int o = s.batched ? 1 : 0;
+    if (gradOutput->size[o] != s.M) return fail("Number of output features is not equal to nOutputPlane");
+    if ((s.batched && gradOutput->size[0] != s.B) || gradOutput->size[o + 1] != s.Ho || gradOutput->size[o + 2] != s.Wo)
+        return fail("SpatialConvolutionMM: gradOutput size does not match the output size");
+    return 0;
+}
+
+// Device pointer of element 0; tensors that reach a kernel are contiguous.
+inline float *dptr(const THGPUTensor *t) { return THGPUTensor_data(t); }
+
+}  // namespace
+
+extern "C" {
+
+int thgpu_SpatialConvolutionMM_updateOutput(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias,
+                                            THGPUTensor *finput, THGPUTensor *fgradInput, THGPUTensor *output,
+                                            int kW, int kH, int dW, int dH, int padW, int padH) {
+    (void)fgradInput;  // the reference uses it as a buffer of ones for the bias GEMM; the bias is fused here
+    ConvShape s;
+    if (conv_shape(s, input, weight, kW, kH, dW, dH, padW, padH)) return 1;
+    if (!bias || !finput || !output) return fail("SpatialConvolutionMM: null tensor");
+    if (THGPUTensor_nElement(bias) != s.M) return fail("SpatialConvolutionMM: bias must have nOutputPlane elements");
+    if (require_contiguous(weight, "weight") || require_contiguous(bias, "bias")) return 1;
+    THGPUTensor *in = THGPUTensor_newContiguous(input);
+    if (!in) return 1;
+
+    if (s.batched) {
+        THGPUTensor_resize3d(finput, s.B, s.K, s.N);
+        THGPUTensor_resize4d(output, s.B, s.M, s.Ho, s.Wo);
+    } else {
+        THGPUTensor_resize2d(finput, s.K, s.N);
+        THGPUTensor_resize3d(output, s.M, s.Ho, s.Wo);
+    }
+    int rc = 0;
+    if (!THGPUTensor_isContiguous(finput) || !THGPUTensor_isContiguous(output) ||
+        THGPUTensor_nElement(finput) != s.B * s.K * s.N || THGPUTensor_nElement(output) != s.B * s.M * s.N)
+        rc = fail("SpatialConvolutionMM: could not size finput/output");
+
+    if (!rc) rc = im2col_launch(dptr(in), s.B, s.C, s.H, s.W, kH, kW, padH, padW, dH, dW, dptr(finput));
+    if (!rc) {
+        // output[b][m][n] = bias[m] + sum_k weight[m][k] * finput[b][k][n]
+        GemmProblem p;
+        p.A = dptr(weight);
+        p.a_rc = true;
+        p.sA = s.K;
+        p.B = dptr(finput);
+        p.b_rc = false;
+        p.sB = s.N;
+        p.bsB = (long)s.K * s.N;
+        p.C = dptr(output);
+        p.sC = s.N;
+        p.bsC = (long)s.M * s.N;
+        p.bias = dptr(bias);
+        p.M = s.M;
+        p.J = (int)(s.B * s.N);
+        p.N = (int)s.N;
+        p.R = s.K;
+        p.tag = "gemm_conv_fwd";
+        rc = gemm_launch(p);
+    }
+    THGPUTensor_free(in);
+    return rc;
+}
+
+int thgpu_SpatialConvolutionMM_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *weight,
+                                               THGPUTensor *finput, THGPUTensor *fgradInput,
+                                               THGPUTensor *gradInput, int kW, int kH, int dW, int dH, int padW,
+                                               int padH) {
+    (void)finput;
+    ConvShape s;
+    if (conv_shape(s, input, weight, kW, kH, dW, dH, padW, padH)) return 1;
+    if (!gradOutput || !fgradInput || !gradInput) return fail("SpatialConvolutionMM: null tensor");
+    if (check_grad_output(s, gradOutput)) return 1;
+    if (require_contiguous(weight, "weight")) return 1;
+    THGPUTensor *go = THGPUTensor_newContiguous(gradOutput);
+    if (!go) return 1;
+
+    if (s.batched) {
+        THGPUTensor_resize4d(gradInput, s.B, s.C, s.H, s.W);
+        THGPUTensor_resize3d(fgradInput, s.B, s.K, s.N);
+    } else {
+        THGPUTensor_resize3d(gradInput, s.C, s.H, s.W);
+        THGPUTensor_resize2d(fgradInput, s.K, s.N);
+    }
+    int rc = 0;
+    if (!THGPUTensor_isContiguous(gradInput) || !THGPUTensor_isContiguous(fgradInput) ||
+        THGPUTensor_nElement(fgradInput) != s.B * s.K * s.N ||
+        THGPUTensor_nElement(gradInput) != s.B * (long)s.C * s.H * s.W)
+        rc = fail("SpatialConvolutionMM: could not size gradInput/fgradInput");
+
+    if (!rc) {
+        // fgradInput[b][k][n] = sum_m weight[m][k] * gradOutput[b][m][n]
+        GemmProblem p;
+        p.A = dptr(weight);
+        p.a_rc = false;  // A(i = k, r = m) = weight[m][k]: contiguous along i
+        p.sA = s.K;
+        p.B = dptr(go);
+        p.b_rc = false;
+        p.sB = s.N;
+        p.bsB = (long)s.M * s.N;
+        p.C = dptr(fgradInput);
+        p.sC = s.N;
+        p.bsC = (long)s.K * s.N;
+        p.M = s.K;
+        p.J = (int)(s.B * s.N);
+        p.N = (int)s.N;
+        p.R = s.M;
+        p.tag = "gemm_conv_gradinput";
+        rc = gemm_launch(p);
+    }
+    if (!rc) rc = col2im_launch(dptr(fgradInput), s.B, s.C, s.H, s.W, kH, kW, padH, padW, dH, dW, dptr(gradInput));
+    THGPUTensor_free(go);
+    return rc;
+}
+
+int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor *gradOutput,
+                                                 THGPUTensor *gradWeight, THGPUTensor *gradBias,
+                                                 THGPUTensor *finput, THGPUTensor *fgradInput, int kW, int kH,
+                                                 int dW, int dH, int padW, int padH, float scale) {
+    (void)fgradInput;
+    ConvShape s;
+    if (!gradWeight || !gradBias || !finput || !gradOutput) return fail("SpatialConvolutionMM: null tensor");
+    if (conv_shape(s, input, gradWeight, kW, kH, dW, dH, padW, padH)) return 1;
+    if (check_grad_output(s, gradOutput)) return 1;
+    if (THGPUTensor_nElement(gradBias) != s.M) return fail("SpatialConvolutionMM: gradBias must have nOutputPlane elements");
+    if (require_contiguous(gradWeight, "gradWeight") || require_contiguous(gradBias, "gradBias")) return 1;
+    THGPUTensor *go = THGPUTensor_newContiguous(gradOutput);
+    if (!go) return 1;
+    int rc = 0;
+    // The CPU module reuses the forward's columns (mcw_nn/generic/
+    // SpatialConvolutionMM.c:318,336).  If finput does not have the forward's
+    // shape (the module was never run forward on this input size) the columns
+    // are rebuilt from the input, as the reference GPU code always did
+    // (gpunn-impl/SpatialConvolutionMM.cpp:394-396).
+    if (THGPUTensor_nElement(finput) != s.B * s.K * s.N || !THGPUTensor_isContiguous(finput)) {
+        THGPUTensor *in = THGPUTensor_newContiguous(input);
+        if (s.batched)
+            THGPUTensor_resize3d(finput, s.B, s.K, s.N);
+        else
+            THGPUTensor_resize2d(finput, s.K, s.N);
+        if (THGPUTensor_nElement(finput) != s.B * s.K * s.N)
+            rc = fail("SpatialConvolutionMM: could not size finput");
+        if (!rc) rc = im2col_launch(dptr(in), s.B, s.C, s.H, s.W, kH, kW, padH, padW, dH, dW, dptr(finput));
+        THGPUTensor_free(in);
+    }
+    if (!rc) {
+        // gradWeight[m][k] += scale * sum_b sum_n gradOutput[b][m][n] * finput[b][k][n]
+        GemmProblem p;
+        p.A = dptr(go);
+        p.a_rc = true;
+        p.sA = s.N;
+        p.rbA = (long)s.M * s.N;
+        p.B = dptr(finput);
+        p.b_rc = true;
+        p.sB = s.N;
+        p.rbB = (long)s.K * s.N;
+        p.C = dptr(gradWeight);
+        p.sC = s.K;
+        p.M = s.M;
+        p.J = s.K;
+        p.N = s.K;
+        p.R = (int)s.N;
+        p.nb = (int)s.B;
+        p.alpha = scale;
+        p.beta = 1.0f;
+        p.tag = "gemm_conv_gradweight";
+        rc = gemm_launch(p);
+    }
+    if (!rc) rc = gradbias_launch(dptr(go), dptr(gradBias), s.B, s.M, s.N, scale);
+    THGPUTensor_free(go);
+    return rc;
+}
+
+int thgpu_SpatialMaxPooling_updateOutput(THGPUTensor *input, THGPUTensor *output, THGPUTensor *indices, int kW,
+                                         int kH, int dW, int dH) {
+    if (!input || !output || !indices) return fail("SpatialMaxPooling: null tensor");
+    if (!(input->nDimension == 3 || input->nDimension == 4)) return fail("3D or 4D (batch) tensor expected");
+    if (kW <= 0 || kH <= 0 || dW <= 0 || dH <= 0) return fail("SpatialMaxPooling: invalid kernel/stride");
+    const bool batched = input->nDimension == 4;
+    const int o = batched ? 1 : 0;
+    const long B = batched ? input->size[0] : 1;
+    const long C = input->size[o];
+    const int H = (int)input->size[o + 1], W = (int)input->size[o + 2];
+    if (!(W >= kW && H >= kH)) return fail("input image smaller than kernel size");
+    const int Ho = (H - kH) / dH + 1, Wo = (W - kW) / dW + 1;
+    THGPUTensor *in = THGPUTensor_newContiguous(input);
+    if (!in) return 1;
+    if (batched) {
+        THGPUTensor_resize4d(output, B, C, Ho, Wo);
+        THGPUTensor_resize5d(indices, 2, B, C, Ho, Wo);
+    } else {
+        THGPUTensor_resize3d(output, C, Ho, Wo);
+        THGPUTensor_resize4d(indices, 2, C, Ho, Wo);
+    }
+    int rc = 0;
+    if (!THGPUTensor_isContiguous(output) || !THGPUTensor_isContiguous(indices) ||
+        THGPUTensor_nElement(output) != B * C * Ho * Wo || THGPUTensor_nElement(indices) != 2 * B * C * Ho * Wo)
+        rc = fail("SpatialMaxPooling: could not size output/indices");
+    if (!rc) rc = maxpool_fwd_launch(dptr(in), B * C, H, W, kH, kW, dH, dW, dptr(output), dptr(indices));
+    THGPUTensor_free(in);
+    return rc;
+}
+
+int thgpu_SpatialMaxPooling_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *gradInput,
+                                            THGPUTensor *indices, int kW, int kH, int dW, int dH) {
+    if (!input || !gradOutput || !gradInput || !indices) return fail("SpatialMaxPooling: null tensor");
+    if (!(input->nDimension == 3 || input->nDimension == 4)) return fail("3D or 4D (batch) tensor expected");
+    if (kW <= 0 || kH <= 0 || dW <= 0 || dH <= 0) return fail("SpatialMaxPooling: invalid kernel/stride");
+    const bool batched = input->nDimension == 4;
+    const int o = batched ? 1 : 0;
+    const long B = batched ? input->size[0] : 1;
+    const long C = input->size[o];
+    const int H = (int)input->size[o + 1], W = (int)input->size[o + 2];
+    if (!(W >= kW && H >= kH)) return fail("input image smaller than kernel size");
+    const int Ho = (H - kH) / dH + 1, Wo = (W - kW) / dW + 1;
+    if (gradOutput->nDimension != input->nDimension || gradOutput->size[o] != C || gradOutput->size[o + 1] != Ho ||
+        gradOutput->size[o + 2] != Wo || (batched && gradOutput->size[0] != B))
+        return fail("SpatialMaxPooling: gradOutput size does not match the output size");
+    if (THGPUTensor_nElement(indices) != 2 * B * C * Ho * Wo || !THGPUTensor_isContiguous(indices))
+        return fail("SpatialMaxPooling: indices do not match (run updateOutput first)");
+    THGPUTensor *go = THGPUTensor_newContiguous(gradOutput);
+    if (!go) return 1;
+    THGPUTensor_resizeAs(gradInput, input);
+    int rc = 0;
+    if (!THGPUTensor_isContiguous(gradInput) || THGPUTensor_nElement(gradInput) != B * C * H * W)
+        rc = fail("SpatialMaxPooling: could not size gradInput");
+    if (!rc)
+        rc = maxpool_bwd_launch(dptr(go), dptr(indices), B * C, H, W, Ho, Wo, kH, kW, dH, dW, dptr(gradInput));
+    THGPUTensor_free(go);
+    return rc;
+}
+
+int thgpu_Threshold_updateOutput(THGPUTensor *input, THGPUTensor *output, float threshold, float val) {
+    if (!input || !output) return fail("Threshold: null tensor");
+    THGPUTensor *in = THGPUTensor_newContiguous(input);
+    if (!in) return 1;
+    THGPUTensor_resizeAs(output, in);
+    long n = THGPUTensor_nElement(in);
+    int rc = 0;
+    if (THGPUTensor_nElement(output) != n || !THGPUTensor_isContiguous(output))
+        rc = fail("Threshold: could not size output");
+    if (!rc) rc = threshold_fwd_launch(dptr(in), dptr(output), n, threshold, val);
+    THGPUTensor_free(in);
+    return rc;
+}
+
+int thgpu_Threshold_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *gradInput,
+                                    float threshold) {
+    if (!input || !gradOutput || !gradInput) return fail("Threshold: null tensor");
+    if (THGPUTensor_nElement(input) != THGPUTensor_nElement(gradOutput))
+        return fail("Threshold: input and gradOutput sizes do not match");
+    THGPUTensor *in = THGPUTensor_newContiguous(input);
+    THGPUTensor *go = THGPUTensor_newContiguous(gradOutput);
+    if (!in || !go) return 1;
+    THGPUTensor_resizeAs(gradInput, in);
+    long n = THGPUTensor_nElement(in);
+    int rc = 0;
+    if (THGPUTensor_nElement(gradInput) != n || !THGPUTensor_isContiguous(gradInput))
+        rc = fail("Threshold: could not size gradInput");
+    if (!rc) rc = threshold_bwd_launch(dptr(in), dptr(go), dptr(gradInput), n, threshold);
+    THGPUTensor_free(in);
+    THGPUTensor_free(go);
+    return rc;
+}
+
+}  // extern "C"

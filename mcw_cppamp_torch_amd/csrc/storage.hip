@@ -1,0 +1,260 @@
+// THGPUStorage on hipMalloc memory with hipMemcpyAsync copies on the library
+// stream.  Semantics follow gputorch/lib/THC/THCStorage.cpp and
+// THCStorageCopy.cpp; the device buffer replaces the array_view that the
+// reference kept in allocatorContext.
+#include "common.h"
+
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+using namespace thgpu;
+
+namespace thgpu {
+
+__global__ void fill_kernel(float *__restrict__ p, long n, float v) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    long stride = (long)gridDim.x * blockDim.x;
+    // 16-byte stores over the aligned body, scalar head/tail.
+    long head = ((16 - ((uintptr_t)p & 15)) & 15) / 4;
+    if (head > n) head = n;
+    if (i < head) p[i] = v;
+    float4 *p4 = reinterpret_cast<float4 *>(p + head);
+    long n4 = (n - head) / 4;
+    float4 v4 = make_float4(v, v, v, v);
+    for (long j = i; j < n4; j += stride) p4[j] = v4;
+    long tail = head + n4 * 4;
+    if (i < n - tail) p[tail + i] = v;
+}
+
+int fill_device(float *p, long n, float v) {
+    if (n <= 0) return 0;
+    hipStream_t s = stream();
+    if (!s) return 1;
+    long blocks = (n / 4 + 255) / 256;
+    if (blocks < 1) blocks = 1;
+    if (blocks > 8192) blocks = 8192;
+    {
+        LaunchScope scope("fill", 0.0, 4.0 * n);
+        hipLaunchKernelGGL(fill_kernel, dim3((unsigned)blocks), dim3(256), 0, s, p, n, v);
+    }
+    return check_launch("fill");
+}
+
+// Blocking host<->device copies: stage through the caller's pageable memory
+// with hipMemcpyAsync on the library stream, then drain the stream, which is
+// what a blocking clEnqueue{Read,Write}Buffer gave the reference's callers
+// (gputorch/lib/THC/copyHelpers.cpp:14-85).
+int copy_h2d(float *dst, const float *src, long n) {
+    if (n <= 0) return 0;
+    hipStream_t s = stream();
+    if (!s) return 1;
+    THGPU_HIP_TRY(hipMemcpyAsync(dst, src, sizeof(float) * (size_t)n, hipMemcpyHostToDevice, s));
+    THGPU_HIP_TRY(hipStreamSynchronize(s));
+    return 0;
+}
+
+int copy_d2h(float *dst, const float *src, long n) {
+    if (n <= 0) return 0;
+    hipStream_t s = stream();
+    if (!s) return 1;
+    THGPU_HIP_TRY(hipMemcpyAsync(dst, src, sizeof(float) * (size_t)n, hipMemcpyDeviceToHost, s));
+    THGPU_HIP_TRY(hipStreamSynchronize(s));
+    return 0;
+}
+
+int copy_d2d(float *dst, const float *src, long n) {
+    if (n <= 0 || dst == src) return 0;
+    hipStream_t s = stream();
+    if (!s) return 1;
+    THGPU_HIP_TRY(hipMemcpyAsync(dst, src, sizeof(float) * (size_t)n, hipMemcpyDeviceToDevice, s));
+    return 0;
+}
+
+}  // namespace thgpu
+
+static void release_buffer(THGPUStorage *self) {
+    if (self->data) {
+        // Work enqueued earlier may still use the buffer.
+        hipStream_t s = stream();
+        if (s) (void)hipStreamSynchronize(s);
+        (void)hipFree(self->data);
+    }
+    self->data = nullptr;
+    self->size = 0;
+}
+
+extern "C" {
+
+float *THGPUStorage_data(const THGPUStorage *self) { return self->data; }
+long THGPUStorage_size(const THGPUStorage *self) { return self->size; }
+
+void THGPUStorage_set(THGPUStorage *self, long index, float value) {
+    THGPU_ARGCHECK((index >= 0) && (index < self->size), 2, "index out of bounds", );
+    if (copy_h2d(self->data + index, &value, 1)) raise("%s", thgpu_last_error());
+}
+
+float THGPUStorage_get(const THGPUStorage *self, long index) {
+    float value = 0;
+    THGPU_ARGCHECK((index >= 0) && (index < self->size), 2, "index out of bounds", 0.0f);
+    if (copy_d2h(&value, self->data + index, 1)) raise("%s", thgpu_last_error());
+    return value;
+}
+
+THGPUStorage *THGPUStorage_new(void) {
+    THGPUStorage *s = static_cast<THGPUStorage *>(std::calloc(1, sizeof(THGPUStorage)));
+    if (!s) {
+        raise("out of host memory");
+        return nullptr;
+    }
+    s->refcount = 1;
+    s->flag = TH_STORAGE_REFCOUNTED | TH_STORAGE_RESIZABLE | TH_STORAGE_FREEMEM;
+    return s;
+}
+
+THGPUStorage *THGPUStorage_newWithSize(long size) {
+    THGPU_ARGCHECK(size >= 0, 2, "invalid size", nullptr);
+    THGPUStorage *s = THGPUStorage_new();
+    if (!s || size == 0) return s;
+    if (!stream()) {
+        std::free(s);
+        raise("%s", thgpu_last_error());
+        return nullptr;
+    }
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&s->data), sizeof(float) * (size_t)size);
+    if (e != hipSuccess) {
+        std::free(s);
+        raise("hipMalloc of %ld floats failed: %s", size, hipGetErrorString(e));
+        return nullptr;
+    }
+    s->size = size;
+    return s;
+}
+
+THGPUStorage *THGPUStorage_newWithSize1(float d0) {
+    float v[1] = {d0};
+    return THGPUStorage_newWithData(v, 1);
+}
+THGPUStorage *THGPUStorage_newWithSize2(float d0, float d1) {
+    float v[2] = {d0, d1};
+    return THGPUStorage_newWithData(v, 2);
+}
+THGPUStorage *THGPUStorage_newWithSize3(float d0, float d1, float d2) {
+    float v[3] = {d0, d1, d2};
+    return THGPUStorage_newWithData(v, 3);
+}
+THGPUStorage *THGPUStorage_newWithSize4(float d0, float d1, float d2, float d3) {
+    float v[4] = {d0, d1, d2, d3};
+    return THGPUStorage_newWithData(v, 4);
+}
+
+THGPUStorage *THGPUStorage_newWithMapping(const char *, long, int) {
+    raise("not available yet for THGPUStorage");
+    return nullptr;
+}
+
+THGPUStorage *THGPUStorage_newWithData(float *data, long size) {
+    THGPUStorage *s = THGPUStorage_newWithSize(size);
+    if (!s) return nullptr;
+    if (size > 0 && copy_h2d(s->data, data, size)) {
+        raise("%s", thgpu_last_error());
+    }
+    return s;
+}
+
+void THGPUStorage_setFlag(THGPUStorage *self, const char flag) { self->flag |= flag; }
+void THGPUStorage_clearFlag(THGPUStorage *self, const char flag) { self->flag &= ~flag; }
+
+void THGPUStorage_retain(THGPUStorage *self) {
+    if (self && (self->flag & TH_STORAGE_REFCOUNTED)) ++self->refcount;
+}
+
+void THGPUStorage_free(THGPUStorage *self) {
+    if (!self || !(self->flag & TH_STORAGE_REFCOUNTED)) return;
+    if (--(self->refcount) <= 0) {
+        if (self->flag & TH_STORAGE_FREEMEM) release_buffer(self);
+        std::free(self);
+    }
+}
+
+void THGPUStorage_fill(THGPUStorage *self, float value) {
+    if (fill_device(self->data, self->size, value)) raise("%s", thgpu_last_error());
+}
+
+void THGPUStorage_resize(THGPUStorage *self, long size) {
+    THGPU_ARGCHECK(size >= 0, 2, "invalid size", );
+    if (!(self->flag & TH_STORAGE_RESIZABLE)) return;
+    if (size == 0) {
+        if (self->flag & TH_STORAGE_FREEMEM) release_buffer(self);
+        self->data = nullptr;
+        self->size = 0;
+        return;
+    }
+    if (self->size == size) return;
+    float *fresh = nullptr;
+    if (!stream()) {
+        raise("%s", thgpu_last_error());
+        return;
+    }
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&fresh), sizeof(float) * (size_t)size);
+    if (e != hipSuccess) {
+        raise("hipMalloc of %ld floats failed: %s", size, hipGetErrorString(e));
+        return;
+    }
+    // The first min(old,new) elements survive a resize (THCStorage.cpp:188-189).
+    if (self->data) {
+        long keep = self->size < size ? self->size : size;
+        if (copy_d2d(fresh, self->data, keep)) raise("%s", thgpu_last_error());
+        release_buffer(self);
+    }
+    self->data = fresh;
+    self->size = size;
+}
+
+void THGPUStorage_rawCopy(THGPUStorage *self, float *src) {
+    if (copy_d2d(self->data, src, self->size)) raise("%s", thgpu_last_error());
+}
+
+void THGPUStorage_copy(THGPUStorage *self, THGPUStorage *src) {
+    THGPU_ARGCHECK(self->size == src->size, 2, "size does not match", );
+    if (copy_d2d(self->data, src->data, self->size)) raise("%s", thgpu_last_error());
+}
+
+void THGPUStorage_copyGPU(THGPUStorage *self, THGPUStorage *src) { THGPUStorage_copy(self, src); }
+
+void THGPUStorage_copyFloat(THGPUStorage *self, struct THFloatStorage *src) {
+    THGPU_ARGCHECK(self->size == src->size, 2, "size does not match", );
+    if (copy_h2d(self->data, src->data, self->size)) raise("%s", thgpu_last_error());
+}
+
+void THFloatStorage_copyGPU(THFloatStorage *self, struct THGPUStorage *src) {
+    THGPU_ARGCHECK(self->size == src->size, 2, "size does not match", );
+    if (copy_d2h(self->data, src->data, self->size)) raise("%s", thgpu_last_error());
+}
+
+// Other element types convert through a host float buffer, as the reference
+// does (THCStorageCopy.cpp:12-29, 37-54).
+#define THGPU_STORAGE_COPY_VIA_FLOAT(Name, ctype)                                             \
+    void THGPUStorage_copy##Name(THGPUStorage *self, struct TH##Name##Storage *src) {         \
+        THGPU_ARGCHECK(self->size == src->size, 2, "size does not match", );                  \
+        std::vector<float> buf((size_t)src->size);                                            \
+        for (long i = 0; i < src->size; i++) buf[(size_t)i] = (float)src->data[i];            \
+        if (copy_h2d(self->data, buf.data(), self->size)) raise("%s", thgpu_last_error());    \
+    }                                                                                         \
+    void TH##Name##Storage_copyGPU(TH##Name##Storage *self, struct THGPUStorage *src) {       \
+        THGPU_ARGCHECK(self->size == src->size, 2, "size does not match", );                  \
+        std::vector<float> buf((size_t)src->size);                                            \
+        if (copy_d2h(buf.data(), src->data, src->size)) {                                     \
+            raise("%s", thgpu_last_error());                                                  \
+            return;                                                                           \
+        }                                                                                     \
+        for (long i = 0; i < src->size; i++) self->data[i] = (ctype)buf[(size_t)i];           \
+    }
+THGPU_STORAGE_COPY_VIA_FLOAT(Byte, unsigned char)
+THGPU_STORAGE_COPY_VIA_FLOAT(Char, char)
+THGPU_STORAGE_COPY_VIA_FLOAT(Short, short)
+THGPU_STORAGE_COPY_VIA_FLOAT(Int, int)
+THGPU_STORAGE_COPY_VIA_FLOAT(Long, long)
+THGPU_STORAGE_COPY_VIA_FLOAT(Double, double)
+
+}  // extern "C"

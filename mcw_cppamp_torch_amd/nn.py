@@ -1,0 +1,279 @@
+"""Host-side mirror of the `nn` modules on the convolution hot path, dispatching
+to the C ABI the way the Lua modules dispatch to `input.nn.<Op>_<method>`:
+
+  nn.Module                mcw_nn/Module.lua:1-164
+  nn.Sequential            mcw_nn/Sequential.lua:1-129
+  nn.SpatialConvolutionMM  mcw_nn/SpatialConvolutionMM.lua:1-60
+  nn.SpatialMaxPooling     mcw_nn/SpatialMaxPooling.lua:1-34
+  nn.Threshold / nn.ReLU   mcw_nn/Threshold.lua:1-21, mcw_nn/ReLU.lua:1-5
+
+Same constructor arguments, field names and call order.  Modules are created
+with host tensors (numpy float32, like torch.Tensor) and moved with :gpu();
+only torch.GPUTensor inputs are computed -- there is no CPU implementation in
+this package.
+"""
+import math
+
+import numpy as np
+
+from . import _lib
+from ._lib import THGPUError, lib
+from .gputorch import FloatTensor, GPUTensor
+
+
+def _is_tensor(v):
+    return isinstance(v, (GPUTensor, np.ndarray))
+
+
+def _convert(v, type_name):
+    if isinstance(v, (list, tuple)) and v and all(_is_tensor(x) for x in v):
+        return [_convert(x, type_name) for x in v]
+    if isinstance(v, GPUTensor):
+        return v.type(type_name)
+    if isinstance(v, np.ndarray):
+        if type_name == "torch.GPUTensor":
+            return GPUTensor.from_numpy(v.astype(np.float32, copy=False))
+        if type_name == "torch.FloatTensor":
+            return np.ascontiguousarray(v, np.float32).view(FloatTensor)
+        if type_name == "torch.DoubleTensor":
+            return np.ascontiguousarray(v, np.float64)
+        raise THGPUError("unknown tensor type %s" % type_name)
+    return v
+
+
+def _require_gpu(*tensors):
+    for t in tensors:
+        if not isinstance(t, GPUTensor):
+            raise THGPUError("torch.GPUTensor expected (this package implements only the GPU path; "
+                             "move tensors and modules with :gpu())")
+
+
+class Module(object):
+    def __init__(self):
+        self.gradInput = FloatTensor()
+        self.output = FloatTensor()
+
+    def parameters(self):
+        w, b = getattr(self, "weight", None), getattr(self, "bias", None)
+        if w is not None and b is not None:
+            return [w, b], [self.gradWeight, self.gradBias]
+        if w is not None:
+            return [w], [self.gradWeight]
+        if b is not None:
+            return [b], [self.gradBias]
+        return None, None
+
+    def updateOutput(self, input):
+        return self.output
+
+    def forward(self, input):
+        return self.updateOutput(input)
+
+    def backward(self, input, gradOutput, scale=1):
+        self.updateGradInput(input, gradOutput)
+        self.accGradParameters(input, gradOutput, scale)
+        return self.gradInput
+
+    def updateGradInput(self, input, gradOutput):
+        return self.gradInput
+
+    def accGradParameters(self, input, gradOutput, scale=1):
+        pass
+
+    def zeroGradParameters(self):
+        _, grads = self.parameters()
+        for g in grads or []:
+            if isinstance(g, GPUTensor):
+                g.zero()
+            else:
+                g[...] = 0
+
+    def type(self, type_name):
+        for key, val in list(self.__dict__.items()):
+            if key != "modules":
+                self.__dict__[key] = _convert(val, type_name)
+        for m in getattr(self, "modules", []):
+            m.type(type_name)
+        return self
+
+    def gpu(self):
+        return self.type("torch.GPUTensor")
+
+    def float(self):
+        return self.type("torch.FloatTensor")
+
+    def double(self):
+        return self.type("torch.DoubleTensor")
+
+    def reset(self, stdv=None):
+        pass
+
+
+class Sequential(Module):
+    def __init__(self):
+        Module.__init__(self)
+        self.modules = []
+
+    def add(self, module):
+        if not self.modules:
+            self.gradInput = module.gradInput
+        self.modules.append(module)
+        self.output = module.output
+        return self
+
+    def size(self):
+        return len(self.modules)
+
+    def get(self, index):
+        return self.modules[index]
+
+    def updateOutput(self, input):
+        cur = input
+        for m in self.modules:
+            cur = m.updateOutput(cur)
+        self.output = cur
+        return cur
+
+    def updateGradInput(self, input, gradOutput):
+        cur = gradOutput
+        for i in range(len(self.modules) - 1, 0, -1):
+            cur = self.modules[i].updateGradInput(self.modules[i - 1].output, cur)
+        cur = self.modules[0].updateGradInput(input, cur)
+        self.gradInput = cur
+        return cur
+
+    def accGradParameters(self, input, gradOutput, scale=1):
+        cur = gradOutput
+        for i in range(len(self.modules) - 1, 0, -1):
+            self.modules[i].accGradParameters(self.modules[i - 1].output, cur, scale)
+            cur = self.modules[i].gradInput
+        self.modules[0].accGradParameters(input, cur, scale)
+
+    def zeroGradParameters(self):
+        for m in self.modules:
+            m.zeroGradParameters()
+
+    def reset(self, stdv=None):
+        for m in self.modules:
+            m.reset(stdv)
+
+
+class SpatialConvolutionMM(Module):
+    """nn.SpatialConvolutionMM(nInputPlane, nOutputPlane, kW, kH, dW, dH, padding).
+
+    `padW`/`padH` (keyword only) override the single symmetric `padding` of the
+    reference for kernels that need different vertical and horizontal padding.
+    Unlike the reference CPU module (mcw_nn/generic/SpatialConvolutionMM.c:
+    148-149) any stride is accepted.
+    """
+
+    def __init__(self, nInputPlane, nOutputPlane, kW, kH, dW=1, dH=1, padding=0, padW=None, padH=None, rng=None):
+        Module.__init__(self)
+        self.nInputPlane, self.nOutputPlane = nInputPlane, nOutputPlane
+        self.kW, self.kH, self.dW, self.dH = kW, kH, dW, dH
+        self.padding = padding or 0
+        self.padW = self.padding if padW is None else padW
+        self.padH = self.padding if padH is None else padH
+        K = nInputPlane * kH * kW
+        self.weight = FloatTensor(nOutputPlane, K)
+        self.bias = FloatTensor(nOutputPlane)
+        self.gradWeight = FloatTensor(nOutputPlane, K)
+        self.gradBias = FloatTensor(nOutputPlane)
+        self.finput = FloatTensor()
+        self.fgradInput = FloatTensor()
+        self._rng = rng if rng is not None else np.random.default_rng()
+        self.reset()
+
+    def reset(self, stdv=None):
+        # mcw_nn/SpatialConvolutionMM.lua:29-46
+        if stdv:
+            stdv = stdv * math.sqrt(3)
+        else:
+            stdv = 1.0 / math.sqrt(self.kW * self.kH * self.nInputPlane)
+        w = self._rng.uniform(-stdv, stdv, size=(self.nOutputPlane, self.nInputPlane * self.kH * self.kW))
+        b = self._rng.uniform(-stdv, stdv, size=(self.nOutputPlane,))
+        self._assign("weight", w)
+        self._assign("bias", b)
+
+    def _assign(self, name, host):
+        cur = getattr(self, name)
+        if isinstance(cur, GPUTensor):
+            cur.copy(np.asarray(host, np.float32))
+        else:
+            setattr(self, name, np.asarray(host, np.float32).view(FloatTensor))
+
+    def _geom(self):
+        return (self.kW, self.kH, self.dW, self.dH, self.padW, self.padH)
+
+    def updateOutput(self, input):
+        _require_gpu(input, self.weight, self.bias, self.finput, self.fgradInput, self.output)
+        _lib.check_status(lib.thgpu_SpatialConvolutionMM_updateOutput(
+            input._p, self.weight._p, self.bias._p, self.finput._p, self.fgradInput._p, self.output._p,
+            *self._geom()))
+        return self.output
+
+    def updateGradInput(self, input, gradOutput):
+        if self.gradInput is None:
+            return None
+        _require_gpu(input, gradOutput, self.weight, self.finput, self.fgradInput, self.gradInput)
+        _lib.check_status(lib.thgpu_SpatialConvolutionMM_updateGradInput(
+            input._p, gradOutput._p, self.weight._p, self.finput._p, self.fgradInput._p, self.gradInput._p,
+            *self._geom()))
+        return self.gradInput
+
+    def accGradParameters(self, input, gradOutput, scale=1):
+        _require_gpu(input, gradOutput, self.gradWeight, self.gradBias, self.finput, self.fgradInput)
+        _lib.check_status(lib.thgpu_SpatialConvolutionMM_accGradParameters(
+            input._p, gradOutput._p, self.gradWeight._p, self.gradBias._p, self.finput._p, self.fgradInput._p,
+            *(self._geom() + (float(scale),))))
+
+
+class SpatialMaxPooling(Module):
+    """nn.SpatialMaxPooling(kW, kH, dW, dH); dW, dH default to kW, kH."""
+
+    def __init__(self, kW, kH, dW=None, dH=None):
+        Module.__init__(self)
+        self.kW, self.kH = kW, kH
+        self.dW = dW or kW
+        self.dH = dH or kH
+        self.indices = FloatTensor()
+
+    def updateOutput(self, input):
+        _require_gpu(input, self.output, self.indices)
+        _lib.check_status(lib.thgpu_SpatialMaxPooling_updateOutput(
+            input._p, self.output._p, self.indices._p, self.kW, self.kH, self.dW, self.dH))
+        return self.output
+
+    def updateGradInput(self, input, gradOutput):
+        _require_gpu(input, gradOutput, self.gradInput, self.indices)
+        _lib.check_status(lib.thgpu_SpatialMaxPooling_updateGradInput(
+            input._p, gradOutput._p, self.gradInput._p, self.indices._p, self.kW, self.kH, self.dW, self.dH))
+        return self.gradInput
+
+
+class Threshold(Module):
+    """nn.Threshold(threshold, value)."""
+
+    def __init__(self, th=None, v=None):
+        Module.__init__(self)
+        for a in (th, v):
+            if a is not None and not isinstance(a, (int, float)):
+                raise THGPUError("nn.Threshold(threshold, value)")
+        self.threshold = 1e-6 if th is None else th
+        self.val = 0 if v is None else v
+
+    def updateOutput(self, input):
+        _require_gpu(input, self.output)
+        _lib.check_status(lib.thgpu_Threshold_updateOutput(input._p, self.output._p, self.threshold, self.val))
+        return self.output
+
+    def updateGradInput(self, input, gradOutput):
+        _require_gpu(input, gradOutput, self.gradInput)
+        _lib.check_status(lib.thgpu_Threshold_updateGradInput(input._p, gradOutput._p, self.gradInput._p,
+                                                              self.threshold))
+        return self.gradInput
+
+
+class ReLU(Threshold):
+    def __init__(self):
+        Threshold.__init__(self, 0, 0)

@@ -155,3 +155,49 @@ def rel_err(got, ref):
 def gemm_tol(k_red):
     """Parity bound for fp32 GEMM results: 1e-4 * sqrt(reduction length)."""
     return 1e-4 * math.sqrt(max(int(k_red), 1))
+
+
+# ---- CPU-oracle evaluation of a whole stack --------------------------------
+def oracle_stack(layers, params, x, grad_out, scale=1.0):
+    """Runs forward+backward of a layer list through the CPU oracle with the
+    sequencing of nn.Sequential / nn.Module:backward.  `params` is a list with
+    (weight, bias) for conv layers and None otherwise.  Returns the forward
+    outputs per layer, gradInput per layer and (gradWeight, gradBias) per conv."""
+    import oracle
+    outs, saved = [], []
+    cur = x
+    for l, p in zip(layers, params):
+        if l[0] == "conv":
+            _, cin, cout, kW, kH, dW, dH, pW, pH = l
+            out, finput = oracle.conv_updateOutput(cur, p[0], p[1], kH, kW, pH, pW, dH, dW)
+            saved.append((cur, finput))
+        elif l[0] == "pool":
+            _, kW, kH, dW, dH = l
+            out, ind = oracle.maxpool_updateOutput(cur, kH, kW, dH, dW)
+            saved.append((cur, ind))
+        else:
+            out = oracle.threshold_updateOutput(cur, 0.0, 0.0)
+            saved.append((cur, None))
+        outs.append(out)
+        cur = out
+    gins = [None] * len(layers)
+    grads = [None] * len(layers)
+    g = grad_out
+    for i in range(len(layers) - 1, -1, -1):
+        l, p = layers[i], params[i]
+        inp, aux = saved[i]
+        if l[0] == "conv":
+            _, cin, cout, kW, kH, dW, dH, pW, pH = l
+            gi, _ = oracle.conv_updateGradInput(g, p[0], inp.shape, kH, kW, pH, pW, dH, dW)
+            gw = np.zeros_like(p[0])
+            gb = np.zeros_like(p[1])
+            oracle.conv_accGradParameters(g, aux, gw, gb, scale)
+            grads[i] = (gw, gb)
+        elif l[0] == "pool":
+            _, kW, kH, dW, dH = l
+            gi = oracle.maxpool_updateGradInput(g, aux, inp.shape, dH, dW)
+        else:
+            gi = oracle.threshold_updateGradInput(inp, g, 0.0)
+        gins[i] = gi
+        g = gi
+    return outs, gins, grads

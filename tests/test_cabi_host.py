@@ -1,0 +1,125 @@
+"""CPU-only checks of the product's host side: the C-ABI library loads and
+exports every symbol that include/thgpu.h declares, the ctypes binding covers
+them, the index arithmetic self-test passes, error paths that need no device
+work report through the handler, and the stack bookkeeping reproduces the
+algorithmic work of the benchmark configurations."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "thgpu.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"#define THGPU_DECLARE_HOST_TYPES.*?TH##Name##Tensor;", "", text, flags=re.S)
+    names = set(re.findall(r"\b((?:TH[A-Za-z]*|thgpu)_[A-Za-z0-9_]+)\s*\(", text))
+    names |= {"THGPUSetErrorHandler"}
+    return sorted(n for n in names if not n.startswith("THGPU_"))
+
+
+@pytest.fixture(scope="module")
+def pkg():
+    import mcw_cppamp_torch_amd as p
+    return p
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    names = declared_functions()
+    assert len(names) > 120
+    raw = ctypes.CDLL(pkg._lib.LIB_PATH)
+    missing = [n for n in names if not hasattr(raw, n)]
+    assert not missing, missing
+
+
+def test_ctypes_binding_covers_the_header(pkg):
+    assert set(declared_functions()) == set(pkg._lib.EXPORTED_SYMBOLS)
+
+
+def test_struct_layouts_match_the_header_as_a_c_compiler_sees_it(pkg, tmp_path):
+    # The two structs are ABI (LuaJIT FFI reads them, gputorch/FFI.lua:5-29): compile the
+    # header with gcc as plain C and compare sizes/offsets with the ctypes mirror.
+    import subprocess
+    src = tmp_path / "layout.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <stddef.h>\n#include "thgpu.h"\n'
+        'int main(void){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\\n",'
+        'sizeof(THGPUStorage),offsetof(THGPUStorage,size),offsetof(THGPUStorage,refcount),'
+        'offsetof(THGPUStorage,flag),offsetof(THGPUStorage,allocator),offsetof(THGPUStorage,allocatorContext),'
+        'sizeof(THGPUTensor),offsetof(THGPUTensor,nDimension),offsetof(THGPUTensor,storage),'
+        'offsetof(THGPUTensor,storageOffset),offsetof(THGPUTensor,refcount),offsetof(THGPUTensor,flag));return 0;}\n')
+    exe = tmp_path / "layout"
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src),
+                           "-o", str(exe)])
+    c_view = [int(v) for v in subprocess.check_output([str(exe)]).split()]
+    L = pkg._lib
+    S, T = L.THGPUStorage, L.THGPUTensor
+    py_view = [ctypes.sizeof(S), S.size.offset, S.refcount.offset, S.flag.offset, S.allocator.offset,
+               S.allocatorContext.offset, ctypes.sizeof(T), T.nDimension.offset, T.storage.offset,
+               T.storageOffset.offset, T.refcount.offset, T.flag.offset]
+    assert c_view == py_view == [40, 8, 16, 20, 24, 32, 48, 16, 24, 32, 40, 44]
+
+
+def test_index_math_selftest(pkg):
+    assert pkg._lib.lib.thgpu_selftest_index_math() == 0
+
+
+def test_metadata_only_tensor_ops_and_error_handler(pkg):
+    # Views and argument errors need no device memory.
+    t = pkg.GPUTensor()
+    assert t.dim() == 0 and t.nElement() == 0 and t.isContiguous()
+    s = pkg.GPUStorage()
+    assert s.size() == 0
+    with pytest.raises(pkg.THGPUError, match="index out of bounds"):
+        s[0]
+    with pytest.raises(pkg.THGPUError, match="not available yet"):
+        pkg._lib.lib.THGPUStorage_newWithMapping(b"x", 1, 0)
+        pkg._lib.check()
+    with pytest.raises(pkg.THGPUError, match="out of range"):
+        t.size(0)
+
+
+def test_ops_reject_bad_arguments_without_a_device(pkg):
+    nn = pkg.nn
+    conv = nn.SpatialConvolutionMM(3, 4, 3, 3)
+    with pytest.raises(pkg.THGPUError, match="GPUTensor expected"):
+        conv.forward(np.zeros((1, 3, 8, 8), np.float32))
+    L = pkg._lib
+    empty = [pkg.GPUTensor() for _ in range(6)]
+    rc = L.lib.thgpu_SpatialConvolutionMM_updateOutput(*([e._p for e in empty] + [3, 3, 1, 1, 0, 0]))
+    assert rc != 0 and b"3D or 4D" in L.lib.thgpu_last_error()
+    rc = L.lib.thgpu_SpatialMaxPooling_updateOutput(empty[0]._p, empty[1]._p, empty[2]._p, 2, 2, 2, 2)
+    assert rc != 0 and b"3D or 4D" in L.lib.thgpu_last_error()
+    with pytest.raises(pkg.THGPUError, match="nn.Threshold"):
+        nn.Threshold("a", 1)
+
+
+def test_module_defaults_follow_the_lua_constructors(pkg):
+    nn = pkg.nn
+    c = nn.SpatialConvolutionMM(3, 8, 5, 7)
+    assert (c.dW, c.dH, c.padding) == (1, 1, 0) and c.weight.shape == (8, 3 * 7 * 5)
+    stdv = 1 / np.sqrt(5 * 7 * 3)
+    assert np.abs(c.weight).max() <= stdv and np.abs(c.bias).max() <= stdv
+    p = nn.SpatialMaxPooling(3, 2)
+    assert (p.dW, p.dH) == (3, 2)
+    t = nn.Threshold()
+    assert t.threshold == 1e-6 and t.val == 0
+    r = nn.ReLU()
+    assert r.threshold == 0 and r.val == 0
+    seq = nn.Sequential().add(c).add(r).add(p)
+    assert seq.size() == 3 and seq.get(0) is c
+
+
+def test_stack_bookkeeping_reproduces_the_benchmark_work(pkg):
+    st = pkg.stacks
+    assert abs(st.work("alexnet")["gemm_flops"] / 1e9 - 503.5) < 0.05
+    assert abs(st.work("overfeat")["gemm_flops"] / 1e9 - 2051.7) < 0.05
+    assert abs(st.work("vgg_a")["gemm_flops"] / 1e9 - 2874.4) < 0.05
+    assert abs(st.work("conv1_b16")["gemm_flops"] / 1e9 - 6.75) < 0.01
+    assert st.output_shape("alexnet") == (128, 256, 6, 6)
+    assert st.output_shape("overfeat") == (128, 1024, 6, 6)
+    assert st.output_shape("vgg_a") == (64, 512, 7, 7)
