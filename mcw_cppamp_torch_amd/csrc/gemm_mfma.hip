@@ -88,7 +88,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(const GemmArgs g) {
     if (A_RC)
         pA = g.A + (long)(i0 + a_i) * g.sA + a_r;
     else
-        pA = g.A + (long)(i0 + a_i) + (long)a_r * g.sA;
+        pA = g.A + (long)(i0 + a_i);  // the row offset (a_r and the step) is added per fetch
 
     const float *pB;
     bool b_col_ok = true;
@@ -98,7 +98,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(const GemmArgs g) {
         unsigned jg = (unsigned)(j0 + b_j), img, n;
         b_col_ok = (int)jg < g.J;
         g.divN.divmod(b_col_ok ? jg : 0u, img, n);
-        pB = g.B + (long)img * g.bsB + n + (long)b_r * g.sB;
+        pB = g.B + (long)img * g.bsB + n;  // the row offset (b_r and the step) is added per fetch
     }
 
     floatx16 acc[TM][TN];
