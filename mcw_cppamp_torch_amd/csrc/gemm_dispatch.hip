@@ -1,0 +1,239 @@
+// Host side of the fp32 MFMA GEMM: picks a tile configuration, the operand
+// loaders and a reduction split for a GemmProblem, launches the kernel and,
+// when the reduction was split, the fixed-order reduction of the partial sums.
+// Also the THGPUBlas_gemm entry point.
+#include "gemm_mfma.h"
+
+#include <cstdlib>
+#include <cstring>
+
+namespace thgpu {
+
+namespace {
+
+// C(i, j) = beta*C + alpha * sum_s ws[s][i][j] (+ bias[i]), s ascending; j is
+// mapped through (image, n) when the output is column batched.
+__global__ __launch_bounds__(256) void split_reduce_kernel(const float *__restrict__ ws, float *__restrict__ C,
+                                                           const float *__restrict__ bias, int M, int J, int N,
+                                                           long sC, long bsC, FastDiv divJ, FastDiv divN, int nsplit,
+                                                           float alpha, float beta) {
+    unsigned idx = blockIdx.x * blockDim.x + threadIdx.x;
+    const unsigned total = (unsigned)M * (unsigned)J;
+    if (idx >= total) return;
+    float sum = 0.0f;
+    for (int s = 0; s < nsplit; ++s) sum += ws[(long)s * total + idx];
+    unsigned i, j;
+    divJ.divmod(idx, i, j);
+    long coff = j;
+    if (N != J) {
+        unsigned im, n;
+        divN.divmod(j, im, n);
+        coff = (long)im * bsC + n;
+    }
+    float *c = C + (long)i * sC + coff;
+    float val = alpha * sum;
+    if (bias) val += bias[i];
+    if (beta != 0.0f) val += beta * *c;
+    *c = val;
+}
+
+struct TileCfg {
+    const char *name;
+    int bm, bn;
+    int resident;  // workgroups that fit a CU at once (registers / LDS)
+    double eff;    // fraction of the MFMA rate the inner loop sustains
+    int (*launch)(const GemmArgs &, int, int, bool, hipStream_t);
+};
+
+const TileCfg kCfgs[] = {
+    {"128x256", 128, 256, 2, 0.86, gemm_fast_128x256},
+    {"256x128", 256, 128, 2, 0.86, gemm_fast_256x128},
+    {"128x128", 128, 128, 3, 0.80, gemm_fast_128x128},
+    {"64x64", 64, 64, 4, 0.66, gemm_fast_64x64},
+};
+
+inline long cdiv(long a, long b) { return (a + b - 1) / b; }
+
+// Rough time model (in CU-cycles) used only to rank candidates: a CU retires
+// 256 flops per cycle at best; the busiest CU gets ceil(workgroups / CUs)
+// workgroups; every workgroup pays a fixed prologue/epilogue; a split adds the
+// traffic of writing and re-reading the partial sums.
+double model_cycles(const TileCfg &c, long M, long J, long steps_total, int nsplit, int cus) {
+    const long tiles = cdiv(M, c.bm) * cdiv(J, c.bn);
+    const long wgs = tiles * nsplit;
+    const long steps = cdiv(steps_total, nsplit);
+    const double per_step = 2.0 * c.bm * c.bn * GEMM_BK / 256.0 / c.eff;
+    const double per_wg = steps * per_step + 2500.0 + 1.5 * c.bm * c.bn / 64.0;
+    // Workgroups beyond what is resident at once run in further rounds; a partly
+    // filled last round leaves the CUs under-occupied, which costs efficiency.
+    const long slots = (long)cus * c.resident;
+    const long full_rounds = wgs / slots, rest = wgs % slots;
+    double t = full_rounds * c.resident * per_wg;
+    if (rest) {
+        const long on_busiest = cdiv(rest, cus);
+        const double occ_penalty = on_busiest >= 2 ? 1.0 : 1.18;  // a lone workgroup cannot hide its own latencies
+        t += on_busiest * per_wg * occ_penalty;
+    }
+    if (nsplit > 1) t += (double)(nsplit + 2) * M * J * 4.0 / (4.0e12 / 2.4e9) ;  // bytes / (bytes per cycle, whole chip)
+    return t;
+}
+
+}  // namespace
+
+int gemm_launch(const GemmProblem &p) {
+    hipStream_t s = stream();
+    if (!s) return 1;
+    if (p.M <= 0 || p.J <= 0) return 0;
+    if ((long)p.M * p.J >= (1L << 31)) return fail("gemm: output of %d x %d exceeds 32-bit tile indexing", p.M, p.J);
+
+    const bool red = p.nb > 1;
+    if (red && !(p.a_rc && p.b_rc)) return fail("gemm: reduction batching needs r-contiguous operands");
+
+    GemmArgs g;
+    std::memset(&g, 0, sizeof(g));
+    g.A = p.A;
+    g.B = p.B;
+    g.C = p.C;
+    g.bias = p.bias;
+    g.M = p.M;
+    g.J = p.J;
+    g.R = p.R;
+    g.N = p.N > 0 ? p.N : p.J;
+    g.sA = p.sA;
+    g.sB = p.sB;
+    g.sC = p.sC;
+    g.bsB = p.bsB;
+    g.bsC = p.bsC;
+    g.rbA = p.rbA;
+    g.rbB = p.rbB;
+    g.nb = p.nb;
+    g.divN = FastDiv((uint32_t)g.N);
+    g.alpha = p.alpha;
+    g.beta = p.beta;
+    g.steps_per_img = (p.R + GEMM_BK - 1) / GEMM_BK;
+    g.steps_total = g.steps_per_img * (red ? p.nb : 1);
+    g.divSpi = FastDiv((uint32_t)(g.steps_per_img > 0 ? g.steps_per_img : 1));
+
+    // ---- tile configuration and reduction split --------------------------------------
+    const int cus = num_cus();
+    const TileCfg *best = nullptr;
+    int best_split = 1;
+    double best_t = 0;
+    const char *force = std::getenv("THGPU_GEMM_TILE");  // tuning aid: force a configuration by name
+    for (const TileCfg &c : kCfgs) {
+        if (p.M < c.bm || p.J < c.bn) continue;
+        if (force && std::strcmp(force, c.name) != 0) continue;
+        const long tiles = cdiv(p.M, c.bm) * cdiv(p.J, c.bn);
+        const int max_split = (int)(g.steps_total / 8 > 0 ? (g.steps_total / 8 < 64 ? g.steps_total / 8 : 64) : 1);
+        for (int ns = 1; ns <= max_split; ++ns) {
+            if (tiles * ns > 16L * cus * c.resident && ns > 1) break;
+            const int sps = (int)cdiv(g.steps_total, ns);
+            if ((int)cdiv(g.steps_total, sps) != ns) continue;  // would leave an empty split
+            const double t = model_cycles(c, p.M, p.J, g.steps_total, ns, cus);
+            if (!best || t < best_t) {
+                best = &c;
+                best_split = ns;
+                best_t = t;
+            }
+        }
+    }
+
+    g.nsplit = best ? best_split : 1;
+    const int bm = best ? best->bm : 64, bn = best ? best->bn : 64;
+    if (!best && red) {
+        // The generic kernel splits too: enough workgroups to fill the chip.
+        const long tiles = cdiv(p.M, 64) * cdiv(p.J, 64);
+        long want = cdiv(2L * cus, tiles);
+        const long cap = g.steps_total / 8 > 0 ? g.steps_total / 8 : 1;
+        if (want > cap) want = cap;
+        if (want < 1) want = 1;
+        const int sps = (int)cdiv(g.steps_total, want);
+        g.nsplit = (int)cdiv(g.steps_total, sps);
+    }
+    g.steps_per_split = (int)cdiv(g.steps_total, g.nsplit);
+    g.tilesM = (unsigned)cdiv(p.M, bm);
+    g.tilesJ = (unsigned)cdiv(p.J, bn);
+    g.divTilesM = FastDiv(g.tilesM);
+    g.divTilesJ = FastDiv(g.tilesJ);
+    const long total = (long)g.tilesM * g.tilesJ * g.nsplit;
+    if (total <= 0 || total >= (1L << 31)) return fail("gemm: tile count %ld out of range", total);
+    g.total = (unsigned)total;
+    if (g.nsplit > 1) {
+        g.ws = workspace(sizeof(float) * (size_t)g.nsplit * p.M * p.J);
+        if (!g.ws) return 1;
+    }
+
+    // ---- loaders: 128-bit loads along r where every row start is 16-byte aligned ------
+    auto aligned_rc = [](const float *base, long stride, long batch_stride, int R) {
+        return ((uintptr_t)base & 15) == 0 && stride % 4 == 0 && batch_stride % 4 == 0 && R >= GEMM_BK;
+    };
+    const int la = !p.a_rc ? LD_XC_SCALAR : aligned_rc(p.A, p.sA, red ? p.rbA : 0, p.R) ? LD_RC_VEC : LD_RC_SCALAR;
+    const int lb = !p.b_rc ? LD_XC_SCALAR : aligned_rc(p.B, p.sB, red ? p.rbB : 0, p.R) ? LD_RC_VEC : LD_RC_SCALAR;
+
+    int rc;
+    {
+        LaunchScope scope(p.tag, 2.0 * p.M * p.J * (double)p.R * (red ? p.nb : 1), 0.0);
+        rc = best ? best->launch(g, la, lb, red, s) : gemm_generic_64x64(g, p.a_rc, p.b_rc, red, s);
+    }
+    if (rc) return rc;
+    if (check_launch(p.tag)) return 1;
+    if (g.nsplit > 1) {
+        const long n = (long)p.M * p.J;
+        {
+            LaunchScope scope("gemm_split_reduce", 0.0, 4.0 * n * (g.nsplit + 2));
+            hipLaunchKernelGGL(split_reduce_kernel, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, s, g.ws, p.C, p.bias,
+                               p.M, p.J, g.N, p.sC, p.bsC, FastDiv((uint32_t)p.J), g.divN, g.nsplit, p.alpha,
+                               p.beta);
+        }
+        if (check_launch("gemm_split_reduce")) return 1;
+    }
+    return 0;
+}
+
+}  // namespace thgpu
+
+using namespace thgpu;
+
+extern "C" void THGPUBlas_gemm(char transa, char transb, long m, long n, long k, float alpha, float *a, long lda,
+                               float *b, long ldb, float beta, float *c, long ldc) {
+    const bool ta = (transa == 't' || transa == 'T');
+    const bool tb = (transb == 't' || transb == 'T');
+    // Quick returns of the reference dispatcher (gputorch/lib/THC/THCBlas.cpp:257).
+    if (!m || !n || ((alpha == 0 || !k) && beta == 1)) return;
+    // Degenerate leading dimensions as TH fixes them up (TH/generic/THBlas.c:275-298).
+    if (n == 1) ldc = m;
+    if (ta) {
+        if (m == 1) lda = k;
+    } else {
+        if (k == 1) lda = m;
+    }
+    if (tb) {
+        if (k == 1) ldb = n;
+    } else {
+        if (n == 1) ldb = k;
+    }
+    if (m >= (1L << 31) || n >= (1L << 31) || k >= (1L << 31)) {
+        raise("THGPUBlas_gemm: dimension exceeds 2^31");
+        return;
+    }
+    // Column-major C(m x n) is the row-major n x m matrix C'(i', j') =
+    // c[j' + i'*ldc]; C' = op(B)' * op(A)' with
+    //   A'(i', r) = op(B)(r, i'),  B'(r, j') = op(A)(j', r).
+    GemmProblem p;
+    p.A = b;
+    p.B = a;
+    p.C = c;
+    p.M = (int)n;
+    p.J = (int)m;
+    p.R = alpha == 0 ? 0 : (int)k;  // empty sum: C = beta*C, whatever A and B hold
+    p.N = (int)m;
+    p.a_rc = !tb;  // 'n': b[r + i'*ldb]
+    p.sA = ldb;
+    p.b_rc = ta;  // 't': a[r + j'*lda]
+    p.sB = lda;
+    p.sC = ldc;
+    p.alpha = alpha;
+    p.beta = beta;
+    p.tag = "gemm_blas";
+    if (gemm_launch(p)) raise("%s", thgpu_last_error());
+}

@@ -1,0 +1,12 @@
+// Fast fp32 MFMA GEMM, 64 x 64 workgroup tile (2 x 2 wavefronts).
+#include "gemm_fast.h"
+
+#include <type_traits>
+
+namespace thgpu {
+
+int gemm_fast_64x64(const GemmArgs &g, int la, int lb, bool red, hipStream_t s) {
+    return gemm_fast_dispatch<64, 64, 2, 2>(g, la, lb, red, s);
+}
+
+}  // namespace thgpu

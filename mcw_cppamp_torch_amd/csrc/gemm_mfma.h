@@ -1,16 +1,17 @@
 // fp32 GEMM on CDNA4 matrix cores (v_mfma_f32_32x32x2_f32), shared by
 // THGPUBlas_gemm and the three GEMMs of nn.SpatialConvolutionMM.
 //
-// The kernel computes, in row-major terms with the output contiguous along j,
+// The kernels compute, in row-major terms with the output contiguous along j,
 //     C(i, j) = alpha * sum_r A(i, r) * B(r, j)  [+ beta * C(i, j)]  [+ bias(i)]
 // with each operand contiguous either along the reduction index r or along
 // its free index.  Two batching schemes cover the convolution:
 //   * column batching: j enumerates (image, n) pairs, j = image*N + n; B and C
 //     take a per-image stride, A is shared (forward and gradInput);
 //   * reduction batching: r enumerates (image, n) pairs and both operands
-//     take a per-image stride (gradWeight); the image range can be split over
-//     several workgroups that write partial sums to a workspace which a
-//     second kernel adds in a fixed order, so results are reproducible.
+//     take a per-image stride (gradWeight).
+// The reduction can be split over several workgroups; the partial sums go to a
+// workspace and a second kernel adds them in a fixed order, so results are
+// reproducible run to run (no atomics anywhere).
 #pragma once
 
 #include "common.h"
@@ -42,5 +43,56 @@ struct GemmProblem {
 
 // Enqueues the GEMM on the library stream.  Returns 0 or a recorded error.
 int gemm_launch(const GemmProblem &p);
+
+// ---- shared between the kernel translation units ------------------------------
+
+constexpr int GEMM_BK = 16;  // reduction step of every kernel
+
+struct GemmArgs {
+    const float *A;
+    const float *B;
+    float *C;
+    const float *bias;
+    float *ws;  // partial sums [nsplit][M][J] when nsplit > 1
+    int M, J, R, N;
+    long sA, sB, sC, bsB, bsC, rbA, rbB;
+    int nb;
+    int steps_per_img;    // ceil(R / GEMM_BK)
+    int steps_per_split;  // reduction steps one workgroup walks
+    int steps_total;      // nb * steps_per_img
+    int nsplit;
+    unsigned tilesM, tilesJ, total;
+    FastDiv divN, divTilesM, divTilesJ, divSpi;
+    float alpha, beta;
+};
+
+// Workgroups are handed to the 8 XCDs round-robin by linear id.  Remap so that
+// each XCD walks a contiguous range of tiles: neighbours in that range share
+// the same B tile (and the whole of A), which then stays in that XCD's L2.
+__device__ inline unsigned xcd_remap(unsigned id, unsigned total) {
+    constexpr unsigned XCDS = 8;
+    unsigned q = total / XCDS, rem = total % XCDS;
+    unsigned xcd = id % XCDS, slot = id / XCDS;
+    unsigned base = xcd * q + (xcd < rem ? xcd : rem);
+    return base + slot;
+}
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+// How an operand tile travels from global memory to LDS.
+enum Loader {
+    LD_RC_VEC = 0,     // contiguous along r, 16-byte aligned rows: 128-bit loads along r
+    LD_RC_SCALAR = 1,  // contiguous along r, any alignment: 16 lanes read 16 consecutive r
+    LD_XC_SCALAR = 2,  // contiguous along the free index: lanes read consecutive rows/columns
+};
+
+// Launch one tile configuration of the fast kernel (gemm_fast.h).  la/lb are
+// Loader values; returns 0 or a recorded error.
+int gemm_fast_128x128(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
+int gemm_fast_128x256(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
+int gemm_fast_256x128(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
+int gemm_fast_64x64(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
+// The bounds-checked kernel for shapes smaller than a tile (gemm_generic.hip).
+int gemm_generic_64x64(const GemmArgs &g, bool a_rc, bool b_rc, bool red, hipStream_t s);
 
 }  // namespace thgpu
