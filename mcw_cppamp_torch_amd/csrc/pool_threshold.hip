@@ -23,9 +23,12 @@ namespace {
 
 struct PoolGeom {
     int H, W, Ho, Wo, kH, kW, dH, dW;
-    FastDiv divWo, divHoWo, divW, divHW;
+    FastDiv divWo, divHoWo, divW, divHW, divDH, divDW;
 };
 
+// KH, KW > 0 fix the window at compile time (fully unrolled: all loads of a
+// window are in flight before the compare chain); 0 takes the run-time sizes.
+template <int KH, int KW>
 __global__ __launch_bounds__(256) void maxpool_fwd_kernel(const float *__restrict__ in, float *__restrict__ out,
                                                           float *__restrict__ indy, float *__restrict__ indx,
                                                           const PoolGeom g, unsigned total) {
@@ -37,13 +40,30 @@ __global__ __launch_bounds__(256) void maxpool_fwd_kernel(const float *__restric
     const float *win = in + ((long)plane * g.H + (long)i * g.dH) * g.W + (long)j * g.dW;
     float best = -INFINITY;
     int by = -1, bx = 0;
-    for (int y = 0; y < g.kH; ++y) {
-        for (int x = 0; x < g.kW; ++x) {
-            float v = win[y * g.W + x];
-            if (v > best) {
-                best = v;
-                by = y;
-                bx = x;
+    if (KH > 0) {
+        float v[KH > 0 ? KH : 1][KW > 0 ? KW : 1];
+#pragma unroll
+        for (int y = 0; y < KH; ++y)
+#pragma unroll
+            for (int x = 0; x < KW; ++x) v[y][x] = win[y * g.W + x];
+#pragma unroll
+        for (int y = 0; y < KH; ++y)
+#pragma unroll
+            for (int x = 0; x < KW; ++x)
+                if (v[y][x] > best) {
+                    best = v[y][x];
+                    by = y;
+                    bx = x;
+                }
+    } else {
+        for (int y = 0; y < g.kH; ++y) {
+            for (int x = 0; x < g.kW; ++x) {
+                float v = win[y * g.W + x];
+                if (v > best) {
+                    best = v;
+                    by = y;
+                    bx = x;
+                }
             }
         }
     }
@@ -54,32 +74,64 @@ __global__ __launch_bounds__(256) void maxpool_fwd_kernel(const float *__restric
     indx[o] = by < 0 ? 0.0f : (float)(bx + 1);
 }
 
+// TH x TW = the most windows that can cover one pixel (ceil(kH/dH) x ceil(kW/dW));
+// candidates outside [lo, hi] are read at a clamped address and contribute +0.0f,
+// so the loads of all candidates are in flight together.
+template <int TH, int TW>
 __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const float *__restrict__ gout,
                                                           const float *__restrict__ indy,
                                                           const float *__restrict__ indx, float *__restrict__ gin,
-                                                          const PoolGeom g, unsigned total) {
+                                                          const PoolGeom g, unsigned total, int th_rt, int tw_rt) {
     unsigned p = blockIdx.x * blockDim.x + threadIdx.x;
     if (p >= total) return;
     unsigned plane, rem, h, w;
     g.divHW.divmod(p, plane, rem);
     g.divW.divmod(rem, h, w);
-    // Windows (i, j) covering the pixel: i*dH <= h <= i*dH + kH - 1.
-    int i_lo = (int)h - g.kH + 1;
-    i_lo = i_lo <= 0 ? 0 : (i_lo + g.dH - 1) / g.dH;
-    int i_hi = (int)h / g.dH;
+    // Windows (i, j) covering the pixel: i*dH <= h <= i*dH + kH - 1, i.e.
+    // i from ceil((h - kH + 1) / dH) (at least 0) to floor(h / dH) (at most Ho-1).
+    const int ht = (int)h - g.kH + g.dH, wt = (int)w - g.kW + g.dW;  // numerators of the ceilings
+    const int i_lo = ht <= 0 ? 0 : (int)g.divDH.div((unsigned)ht);
+    const int j_lo = wt <= 0 ? 0 : (int)g.divDW.div((unsigned)wt);
+    int i_hi = (int)g.divDH.div(h);
     if (i_hi > g.Ho - 1) i_hi = g.Ho - 1;
-    int j_lo = (int)w - g.kW + 1;
-    j_lo = j_lo <= 0 ? 0 : (j_lo + g.dW - 1) / g.dW;
-    int j_hi = (int)w / g.dW;
+    int j_hi = (int)g.divDW.div(w);
     if (j_hi > g.Wo - 1) j_hi = g.Wo - 1;
-    const long obase = (long)plane * g.Ho * g.Wo;
+    const float *go = gout + (long)plane * g.Ho * g.Wo;
+    const float *iy = indy + (long)plane * g.Ho * g.Wo;
+    const float *ix = indx + (long)plane * g.Ho * g.Wo;
     float acc = 0.0f;
-    for (int i = i_lo; i <= i_hi; ++i) {
-        const float wy = (float)((int)h - i * g.dH + 1);  // 1-based ky that would hit this row
-        for (int j = j_lo; j <= j_hi; ++j) {
-            long o = obase + (long)i * g.Wo + j;
-            const float wx = (float)((int)w - j * g.dW + 1);
-            if (indy[o] == wy && indx[o] == wx) acc += gout[o];
+    if (TH > 0) {
+        float vy[TH > 0 ? TH : 1][TW > 0 ? TW : 1], vx[TH > 0 ? TH : 1][TW > 0 ? TW : 1],
+            vg[TH > 0 ? TH : 1][TW > 0 ? TW : 1];
+#pragma unroll
+        for (int a = 0; a < TH; ++a)
+#pragma unroll
+            for (int b = 0; b < TW; ++b) {
+                const int i = i_lo + a, j = j_lo + b;
+                const int o = (i <= i_hi && j <= j_hi) ? i * g.Wo + j : 0;
+                vy[a][b] = iy[o];
+                vx[a][b] = ix[o];
+                vg[a][b] = go[o];
+            }
+#pragma unroll
+        for (int a = 0; a < TH; ++a)
+#pragma unroll
+            for (int b = 0; b < TW; ++b) {
+                const int i = i_lo + a, j = j_lo + b;
+                const float wy = (float)((int)h - i * g.dH + 1), wx = (float)((int)w - j * g.dW + 1);
+                const bool hit = i <= i_hi && j <= j_hi && vy[a][b] == wy && vx[a][b] == wx;
+                acc += hit ? vg[a][b] : 0.0f;
+            }
+    } else {
+        (void)th_rt;
+        (void)tw_rt;
+        for (int i = i_lo; i <= i_hi; ++i) {
+            const float wy = (float)((int)h - i * g.dH + 1);  // 1-based ky that would hit this row
+            for (int j = j_lo; j <= j_hi; ++j) {
+                const int o = i * g.Wo + j;
+                const float wx = (float)((int)w - j * g.dW + 1);
+                if (iy[o] == wy && ix[o] == wx) acc += go[o];
+            }
         }
     }
     gin[p] = acc;
@@ -130,13 +182,18 @@ __global__ __launch_bounds__(256) void threshold_bwd_scalar(const float *__restr
     if (i < n) gin[i] = in[i] > th ? gout[i] : 0.0f;
 }
 
-// gradBias[m] += scale * sum over images and positions of gradOutput[b][m][n].
-// One workgroup per output plane; fixed-shape tree, so reruns are identical.
-__global__ __launch_bounds__(256) void gradbias_kernel(const float *__restrict__ gout, float *__restrict__ gbias,
-                                                       int B, int M, int N, float scale) {
-    const int m = blockIdx.x;
+// gradBias[m] += scale * sum over images and positions of gradOutput[b][m][n],
+// in two fixed-shape stages so that reruns are bit-identical: stage 1 sums a
+// slice of the batch per workgroup into part[m][slice], stage 2 adds the slices
+// in order.
+__global__ __launch_bounds__(256) void gradbias_partial_kernel(const float *__restrict__ gout,
+                                                               float *__restrict__ part, int B, int M, int N,
+                                                               int imgs_per_slice, int nslices) {
+    const int m = blockIdx.x, slice = blockIdx.y;
+    const int b0 = slice * imgs_per_slice;
+    const int b1 = b0 + imgs_per_slice < B ? b0 + imgs_per_slice : B;
     float sum = 0.0f;
-    for (int b = 0; b < B; ++b) {
+    for (int b = b0; b < b1; ++b) {
         const float *row = gout + ((long)b * M + m) * N;
         for (int n = threadIdx.x; n < N; n += 256) sum += row[n];
     }
@@ -147,7 +204,17 @@ __global__ __launch_bounds__(256) void gradbias_kernel(const float *__restrict__
         if ((int)threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
         __syncthreads();
     }
-    if (threadIdx.x == 0) gbias[m] += scale * red[0];
+    if (threadIdx.x == 0) part[(long)m * nslices + slice] = red[0];
+}
+
+__global__ __launch_bounds__(256) void gradbias_final_kernel(const float *__restrict__ part,
+                                                             float *__restrict__ gbias, int M, int nslices,
+                                                             float scale) {
+    const int m = blockIdx.x * blockDim.x + threadIdx.x;
+    if (m >= M) return;
+    float sum = 0.0f;
+    for (int s = 0; s < nslices; ++s) sum += part[(long)m * nslices + s];
+    gbias[m] += scale * sum;
 }
 
 }  // namespace
@@ -170,8 +237,16 @@ int maxpool_fwd_launch(const float *in, long planes, int H, int W, int kH, int k
     g.divHW = FastDiv((uint32_t)(H * W));
     {
         LaunchScope scope("maxpool_fwd", 0.0, 4.0 * (planes * (double)H * W + 3.0 * total));
-        hipLaunchKernelGGL(maxpool_fwd_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, in, out,
-                           indices, indices + total, g, (unsigned)total);
+        const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+        if (kH == 3 && kW == 3)
+            hipLaunchKernelGGL((maxpool_fwd_kernel<3, 3>), grid, block, 0, s, in, out, indices, indices + total, g,
+                               (unsigned)total);
+        else if (kH == 2 && kW == 2)
+            hipLaunchKernelGGL((maxpool_fwd_kernel<2, 2>), grid, block, 0, s, in, out, indices, indices + total, g,
+                               (unsigned)total);
+        else
+            hipLaunchKernelGGL((maxpool_fwd_kernel<0, 0>), grid, block, 0, s, in, out, indices, indices + total, g,
+                               (unsigned)total);
     }
     return check_launch("maxpool_fwd");
 }
@@ -189,10 +264,21 @@ int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int
     g.divHoWo = FastDiv((uint32_t)(Ho * Wo > 0 ? Ho * Wo : 1));
     g.divW = FastDiv((uint32_t)W);
     g.divHW = FastDiv((uint32_t)(H * W));
+    g.divDH = FastDiv((uint32_t)dH);
+    g.divDW = FastDiv((uint32_t)dW);
     {
         LaunchScope scope("maxpool_bwd", 0.0, 4.0 * ((double)total + 3.0 * ototal));
-        hipLaunchKernelGGL(maxpool_bwd_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, gout, indices,
-                           indices + ototal, gin, g, (unsigned)total);
+        const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+        const int th = (kH + dH - 1) / dH, tw = (kW + dW - 1) / dW;
+        if (th == 2 && tw == 2)
+            hipLaunchKernelGGL((maxpool_bwd_kernel<2, 2>), grid, block, 0, s, gout, indices, indices + ototal, gin, g,
+                               (unsigned)total, th, tw);
+        else if (th == 1 && tw == 1)
+            hipLaunchKernelGGL((maxpool_bwd_kernel<1, 1>), grid, block, 0, s, gout, indices, indices + ototal, gin, g,
+                               (unsigned)total, th, tw);
+        else
+            hipLaunchKernelGGL((maxpool_bwd_kernel<0, 0>), grid, block, 0, s, gout, indices, indices + ototal, gin, g,
+                               (unsigned)total, th, tw);
     }
     return check_launch("maxpool_bwd");
 }
@@ -238,12 +324,30 @@ int gradbias_launch(const float *gout, float *gbias, long B, int M, long N, floa
     if (!s) return 1;
     if (M == 0) return 0;
     if (B >= (1L << 31) || N >= (1L << 31)) return fail("gradBias: tensor too large");
+    // About four workgroups per CU in stage 1.
+    long nslices = (4L * num_cus() + M - 1) / M;
+    if (nslices > B) nslices = B;
+    if (nslices > 65535) nslices = 65535;
+    if (nslices < 1) nslices = 1;
+    const int ips = (int)((B + nslices - 1) / nslices);
+    nslices = (B + ips - 1) / ips;
+    if (nslices < 1) nslices = 1;
+    // The partial sums live behind the GEMM's split workspace, which the
+    // gradWeight GEMM enqueued before has finished with (same stream).
+    float *part = workspace(sizeof(float) * (size_t)M * nslices);
+    if (!part) return 1;
     {
         LaunchScope scope("gradbias", 0.0, 4.0 * B * M * N);
-        hipLaunchKernelGGL(gradbias_kernel, dim3((unsigned)M), dim3(256), 0, s, gout, gbias, (int)B, M, (int)N,
-                           scale);
+        hipLaunchKernelGGL(gradbias_partial_kernel, dim3((unsigned)M, (unsigned)nslices), dim3(256), 0, s, gout,
+                           part, (int)B, M, (int)N, ips, (int)nslices);
     }
-    return check_launch("gradbias");
+    if (check_launch("gradbias")) return 1;
+    {
+        LaunchScope scope("gradbias_final", 0.0, 4.0 * M * (nslices + 2));
+        hipLaunchKernelGGL(gradbias_final_kernel, dim3((unsigned)((M + 255) / 256)), dim3(256), 0, s, part, gbias,
+                           M, (int)nslices, scale);
+    }
+    return check_launch("gradbias_final");
 }
 
 }  // namespace thgpu
