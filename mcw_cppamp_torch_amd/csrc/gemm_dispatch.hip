@@ -41,40 +41,41 @@ struct TileCfg {
     const char *name;
     int bm, bn;
     int resident;  // workgroups that fit a CU at once (registers / LDS)
-    double eff;    // fraction of the MFMA rate the inner loop sustains
+    double eff;    // fraction of the MFMA rate the inner loop sustains with a full CU
     int (*launch)(const GemmArgs &, int, int, bool, hipStream_t);
 };
 
 const TileCfg kCfgs[] = {
+    {"128x128", 128, 128, 4, 0.90, gemm_fast_128x128},
+    {"64x256", 64, 256, 3, 0.88, gemm_fast_64x256},
     {"128x256", 128, 256, 2, 0.86, gemm_fast_128x256},
     {"256x128", 256, 128, 2, 0.86, gemm_fast_256x128},
-    {"128x128", 128, 128, 3, 0.80, gemm_fast_128x128},
-    {"64x64", 64, 64, 4, 0.66, gemm_fast_64x64},
+    {"64x64", 64, 64, 4, 0.74, gemm_fast_64x64},
 };
 
 inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 
-// Rough time model (in CU-cycles) used only to rank candidates: a CU retires
-// 256 flops per cycle at best; the busiest CU gets ceil(workgroups / CUs)
-// workgroups; every workgroup pays a fixed prologue/epilogue; a split adds the
-// traffic of writing and re-reading the partial sums.
+// Rough time model (in CU-cycles) used only to rank (tile, split) candidates.
+// A CU retires 256 flops per cycle at best; with fewer workgroups resident it
+// hides less of their latencies (kOcc); workgroups beyond what fits at once
+// run in further rounds; every round pays a prologue/epilogue; a split adds
+// the traffic of writing and re-reading the partial sums.
 double model_cycles(const TileCfg &c, long M, long J, long steps_total, int nsplit, int cus) {
+    static const double kOcc[5] = {0.0, 0.70, 0.88, 0.96, 1.0};
     const long tiles = cdiv(M, c.bm) * cdiv(J, c.bn);
     const long wgs = tiles * nsplit;
     const long steps = cdiv(steps_total, nsplit);
     const double per_step = 2.0 * c.bm * c.bn * GEMM_BK / 256.0 / c.eff;
-    const double per_wg = steps * per_step + 2500.0 + 1.5 * c.bm * c.bn / 64.0;
-    // Workgroups beyond what is resident at once run in further rounds; a partly
-    // filled last round leaves the CUs under-occupied, which costs efficiency.
+    const double ovh = 3000.0 + 6.0 * c.bm * c.bn / 64.0;
     const long slots = (long)cus * c.resident;
-    const long full_rounds = wgs / slots, rest = wgs % slots;
-    double t = full_rounds * c.resident * per_wg;
-    if (rest) {
+    const long full = wgs / slots, rest = wgs - full * slots;
+    double t = full * (c.resident * steps * per_step / kOcc[c.resident] + ovh);
+    if (rest > 0) {
         const long on_busiest = cdiv(rest, cus);
-        const double occ_penalty = on_busiest >= 2 ? 1.0 : 1.18;  // a lone workgroup cannot hide its own latencies
-        t += on_busiest * per_wg * occ_penalty;
+        const int k = (int)(on_busiest < c.resident ? on_busiest : c.resident);
+        t += on_busiest * steps * per_step / kOcc[k] + ovh * (k > 1 ? 1.0 : 1.5);
     }
-    if (nsplit > 1) t += (double)(nsplit + 2) * M * J * 4.0 / (4.0e12 / 2.4e9) ;  // bytes / (bytes per cycle, whole chip)
+    if (nsplit > 1) t += (double)(nsplit + 2) * M * J * 4.0 / (4.5e12 / 2.4e9);  // bytes / (bytes per cycle)
     return t;
 }
 
@@ -119,14 +120,29 @@ int gemm_launch(const GemmProblem &p) {
     const TileCfg *best = nullptr;
     int best_split = 1;
     double best_t = 0;
-    const char *force = std::getenv("THGPU_GEMM_TILE");  // tuning aid: force a configuration by name
+    // Tuning aids: THGPU_GEMM_TILE forces a configuration by name, THGPU_GEMM_SPLIT a split count.
+    const char *force = std::getenv("THGPU_GEMM_TILE");
+    const char *force_split = std::getenv("THGPU_GEMM_SPLIT");
+    const int fsplit = force_split ? std::atoi(force_split) : 0;
+    // The fast kernel addresses each operand as a uniform base plus a 32-bit
+    // per-thread byte offset and moves a partial last step back by up to 15
+    // reduction indices: it needs R >= 16 and tile-local offsets below 2^30 floats.
+    const long n_img = g.N;
+    auto offsets_fit = [&](int bm, int bn) {
+        const long offA = p.a_rc ? (long)(bm - 1) * p.sA + GEMM_BK : (long)(GEMM_BK - 1) * p.sA + bm;
+        const long span = (bn - 1) / n_img + 2;  // images a tile's columns can touch
+        const long offB = p.b_rc ? (long)(bn - 1) * p.sB + GEMM_BK : (long)(GEMM_BK - 1) * p.sB + span * p.bsB + n_img;
+        return offA < (1L << 30) && offB < (1L << 30);
+    };
+    const bool fast_ok = p.R == 0 || p.R >= GEMM_BK;
     for (const TileCfg &c : kCfgs) {
-        if (p.M < c.bm || p.J < c.bn) continue;
+        if (!fast_ok || p.M < c.bm || p.J < c.bn || !offsets_fit(c.bm, c.bn)) continue;
         if (force && std::strcmp(force, c.name) != 0) continue;
         const long tiles = cdiv(p.M, c.bm) * cdiv(p.J, c.bn);
-        const int max_split = (int)(g.steps_total / 8 > 0 ? (g.steps_total / 8 < 64 ? g.steps_total / 8 : 64) : 1);
+        const int max_split = (int)(g.steps_total / 8 > 0 ? (g.steps_total / 8 < 256 ? g.steps_total / 8 : 256) : 1);
         for (int ns = 1; ns <= max_split; ++ns) {
-            if (tiles * ns > 16L * cus * c.resident && ns > 1) break;
+            if (fsplit > 0 && ns != (fsplit < max_split ? fsplit : max_split)) continue;
+            if (tiles * ns > 8L * cus * c.resident && ns > 1 && fsplit <= 0) break;
             const int sps = (int)cdiv(g.steps_total, ns);
             if ((int)cdiv(g.steps_total, sps) != ns) continue;  // would leave an empty split
             const double t = model_cycles(c, p.M, p.J, g.steps_total, ns, cus);
@@ -163,12 +179,9 @@ int gemm_launch(const GemmProblem &p) {
         if (!g.ws) return 1;
     }
 
-    // ---- loaders: 128-bit loads along r where every row start is 16-byte aligned ------
-    auto aligned_rc = [](const float *base, long stride, long batch_stride, int R) {
-        return ((uintptr_t)base & 15) == 0 && stride % 4 == 0 && batch_stride % 4 == 0 && R >= GEMM_BK;
-    };
-    const int la = !p.a_rc ? LD_XC_SCALAR : aligned_rc(p.A, p.sA, red ? p.rbA : 0, p.R) ? LD_RC_VEC : LD_RC_SCALAR;
-    const int lb = !p.b_rc ? LD_XC_SCALAR : aligned_rc(p.B, p.sB, red ? p.rbB : 0, p.R) ? LD_RC_VEC : LD_RC_SCALAR;
+    // ---- loaders: r-contiguous operands use 128-bit loads (4-byte alignment suffices) --------
+    const int la = p.a_rc ? LD_RC_VEC : LD_XC_SCALAR;
+    const int lb = p.b_rc ? LD_RC_VEC : LD_XC_SCALAR;
 
     int rc;
     {

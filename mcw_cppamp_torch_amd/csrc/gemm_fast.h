@@ -5,11 +5,12 @@
 //   * A workgroup of WGM x WGN wavefronts owns a BM x BN tile of C, each
 //     wavefront TM x TN blocks of 32x32 outputs, one v_mfma_f32_32x32x2_f32
 //     accumulator (16 registers per lane) per block.
-//   * No bounds checks in the main loop.  A tile at the lower/right edge is
-//     shifted back so that it lies inside the matrix (needs M >= BM, J >= BN;
-//     smaller problems take the bounds-checked generic kernel) and stores only
-//     the rows/columns no other tile owns.  Only the last reduction step of an
-//     image can be partial; it takes a separate, masked fetch.
+//   * No bounds checks and no branches around loads.  A tile at the lower/right
+//     edge is shifted back so that it lies inside the matrix and stores only the
+//     rows/columns no other tile owns; a reduction step that would run past R is
+//     shifted back to end at R and the part the previous step already covered
+//     is zeroed on its way to LDS.  Needs M >= BM, J >= BN, R >= 16; smaller
+//     problems take the bounds-checked generic kernel.
 //   * LDS holds both operand tiles as [x][r] (x the free index, r the
 //     reduction index, 16 + 4 floats per row).  Each lane fetches its MFMA
 //     operands with 128-bit LDS reads: lane (x, h) reads r = 8h .. 8h+7, and
@@ -30,6 +31,13 @@ namespace thgpu {
 
 constexpr int LDK = GEMM_BK + 4;  // LDS row pitch in floats
 
+// Four floats at a 4-byte aligned address: the hardware handles the
+// misalignment of a 128-bit global load; the type only keeps the compiler from
+// assuming 16-byte alignment.
+struct __attribute__((packed, aligned(4))) float4u {
+    float x, y, z, w;
+};
+
 // Wavefronts per SIMD the register allocation must leave room for: the
 // accumulators take (BM/WGM)*(BN/WGN)/64 registers of the 512 a lane has.
 template <int BM, int BN, int WGM, int WGN>
@@ -37,7 +45,9 @@ constexpr int gemm_min_waves() {
     return (BM / WGM) * (BN / WGN) / 64 >= 128 ? 2 : 3;
 }
 
-template <int BM, int BN, int WGM, int WGN, int LA, int LB, bool RED>
+// DBG is 0 in the library; experiments switch phases off with it (1: no global
+// fetch in the loop, 2: no LDS operand reads, 4: no LDS stores, 8: no barrier).
+template <int BM, int BN, int WGM, int WGN, int LA, int LB, bool RED, int DBG = 0>
 __global__ __launch_bounds__(WGM *WGN * 64)
     __attribute__((amdgpu_waves_per_eu(gemm_min_waves<BM, BN, WGM, WGN>()))) void gemm_fast_kernel(const GemmArgs g) {
     constexpr int NT = WGM * WGN * 64;
@@ -79,40 +89,44 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     }
 
     // ---- loader set-up -------------------------------------------------------------
-    // Per operand: a 64-bit per-thread base pointer (tile origin + thread part)
-    // and compile-time multiples of the uniform stride for the thread's elements.
-    const float *pA;
-    int a_x, a_r;  // thread's first (x, r) inside the tile
-    if (LA == LD_RC_VEC) {
-        a_x = tid >> 2;
-        a_r = (tid & 3) * 4;
-        pA = g.A + (long)(i0 + a_x) * g.sA + a_r;
-    } else if (LA == LD_RC_SCALAR) {
-        a_x = tid >> 4;
-        a_r = tid & 15;
-        pA = g.A + (long)(i0 + a_x) * g.sA + a_r;
-    } else {
+    // Thread -> (x, r) of its first element inside an operand tile:
+    //   LD_RC_VEC     x = tid/4 (+64 per load), r = 4*(tid%4) .. +3   (one 128-bit load each)
+    //   LD_RC_SCALAR  x = tid/16 (+16 per load), r = tid%16
+    //   LD_XC_SCALAR  x = tid % X, r = (tid / X) * CNT .. + CNT-1     (CNT loads down the column)
+    // A load address is a wave-uniform base (tile, image, step, load number: all
+    // scalar) plus a per-thread byte offset that never changes, so the loop
+    // spends no vector ALU work on addressing.
+    int a_x, a_r, b_x, b_r;
+    unsigned voffA, voffB;
+    const char *tileA, *tileB;
+    if (LA == LD_XC_SCALAR) {
         a_x = tid % BM;
-        a_r = (tid / BM) * NA;  // NA consecutive r per thread (NT >= BM), or all 16 (NT < BM)
-        pA = g.A + (long)(i0 + a_x);
-    }
-    const float *pB;
-    int b_x, b_r;
-    if (LB == LD_RC_VEC) {
-        b_x = tid >> 2;
-        b_r = (tid & 3) * 4;
-        pB = g.B + (long)(j0 + b_x) * g.sB + b_r;
-    } else if (LB == LD_RC_SCALAR) {
-        b_x = tid >> 4;
-        b_r = tid & 15;
-        pB = g.B + (long)(j0 + b_x) * g.sB + b_r;
+        a_r = (tid / BM) * NA;
+        voffA = (unsigned)(((long)a_r * g.sA + a_x) * 4);
+        tileA = reinterpret_cast<const char *>(g.A + i0);
     } else {
+        a_x = LA == LD_RC_VEC ? tid >> 2 : tid >> 4;
+        a_r = LA == LD_RC_VEC ? (tid & 3) * 4 : tid & 15;
+        voffA = (unsigned)(((long)a_x * g.sA + a_r) * 4);
+        tileA = reinterpret_cast<const char *>(g.A + (long)i0 * g.sA);
+    }
+    if (LB == LD_XC_SCALAR) {
         b_x = tid % BN;
         b_r = (tid / BN) * NB;
-        unsigned img, n;
+        unsigned img0, n0, img, n;
+        g.divN.divmod((unsigned)j0, img0, n0);
         g.divN.divmod((unsigned)(j0 + b_x), img, n);
-        pB = g.B + (long)img * g.bsB + n;
+        voffB = (unsigned)(((long)b_r * g.sB + (long)(img - img0) * g.bsB + n) * 4);
+        tileB = reinterpret_cast<const char *>(g.B + (long)img0 * g.bsB);
+    } else {
+        b_x = LB == LD_RC_VEC ? tid >> 2 : tid >> 4;
+        b_r = LB == LD_RC_VEC ? (tid & 3) * 4 : tid & 15;
+        voffB = (unsigned)(((long)b_x * g.sB + b_r) * 4);
+        tileB = reinterpret_cast<const char *>(g.B + (long)j0 * g.sB);
     }
+    constexpr int UA = LA == LD_RC_VEC ? NA / 4 : NA;  // load instructions per step and operand
+    constexpr int UB = LB == LD_RC_VEC ? NB / 4 : NB;
+
     floatx16 acc[TM][TN];
 #pragma unroll
     for (int a = 0; a < TM; ++a)
@@ -123,74 +137,47 @@ __global__ __launch_bounds__(WGM *WGN * 64)
 
     float ra[NA], rb[NB];
 
-    // One operand's global loads for the step at (ld_img, ld_r0).  TAIL handles
-    // a step that runs past R: addresses are clamped into the row and the
-    // values past R are zeroed.
-    auto fetch_one = [&](auto tail_tag, auto kind_tag, const float *base, long stride, int t_r, float *dst,
-                         auto count_tag) {
-        constexpr bool TAIL = decltype(tail_tag)::value;
+    // Load number u of an operand for the step whose uniform base is `base`.
+    auto load_unit = [&](auto kind_tag, const char *base, long stride, unsigned voff, float *dst, int u) {
         constexpr int KIND = decltype(kind_tag)::value;
-        constexpr int CNT = decltype(count_tag)::value;
-        const int r_base = ld_r0 + t_r;
         if (KIND == LD_RC_VEC) {
-            // element q*4+e: row q*(NT/4), r = r_base + e
-#pragma unroll
-            for (int q = 0; q < CNT / 4; ++q) {
-                const float *p = base + (long)(q * (NT / 4)) * stride + ld_r0;
-                if (!TAIL) {
-                    float4 v = *reinterpret_cast<const float4 *>(p);
-                    dst[q * 4 + 0] = v.x;
-                    dst[q * 4 + 1] = v.y;
-                    dst[q * 4 + 2] = v.z;
-                    dst[q * 4 + 3] = v.w;
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int r = r_base + e;
-                        const int back = r < g.R ? 0 : r - (g.R - 1);
-                        const float v = p[e - back];
-                        dst[q * 4 + e] = r < g.R ? v : 0.0f;
-                    }
-                }
-            }
+            const float4u v = *reinterpret_cast<const float4u *>(base + (long)(u * (NT / 4)) * stride * 4 + voff);
+            dst[u * 4 + 0] = v.x;
+            dst[u * 4 + 1] = v.y;
+            dst[u * 4 + 2] = v.z;
+            dst[u * 4 + 3] = v.w;
         } else if (KIND == LD_RC_SCALAR) {
-            // element q: row q*(NT/16), r = r_base
-            const int back = (!TAIL || r_base < g.R) ? 0 : r_base - (g.R - 1);
-#pragma unroll
-            for (int q = 0; q < CNT; ++q) {
-                const float v = base[(long)(q * (NT / 16)) * stride + (ld_r0 - back)];
-                dst[q] = (!TAIL || r_base < g.R) ? v : 0.0f;
-            }
+            dst[u] = *reinterpret_cast<const float *>(base + (long)(u * (NT / 16)) * stride * 4 + voff);
         } else {
-            // element e: r = r_base + e, the thread's own row/column
-#pragma unroll
-            for (int e = 0; e < CNT; ++e) {
-                const int r = r_base + e;
-                const int rr = (!TAIL || r < g.R) ? r : g.R - 1;
-                const float v = base[(long)rr * stride];
-                dst[e] = (!TAIL || r < g.R) ? v : 0.0f;
-            }
+            dst[u] = *reinterpret_cast<const float *>(base + (long)u * stride * 4 + voff);
         }
     };
 
-    auto fetch = [&]() {
-        const float *a = pA + (RED ? (long)ld_img * g.rbA : 0L);
-        const float *b = pB + (RED ? (long)ld_img * g.rbB : 0L);
-        if (ld_r0 + BK <= g.R) {
-            fetch_one(std::false_type{}, std::integral_constant<int, LA>{}, a, g.sA, a_r, ra,
-                      std::integral_constant<int, NA>{});
-            fetch_one(std::false_type{}, std::integral_constant<int, LB>{}, b, g.sB, b_r, rb,
-                      std::integral_constant<int, NB>{});
-        } else {
-            fetch_one(std::true_type{}, std::integral_constant<int, LA>{}, a, g.sA, a_r, ra,
-                      std::integral_constant<int, NA>{});
-            fetch_one(std::true_type{}, std::integral_constant<int, LB>{}, b, g.sB, b_r, rb,
-                      std::integral_constant<int, NB>{});
-        }
+    // Uniform bases of the step at (ld_img, ld_r0).  A step that would run past
+    // R is moved back to end at R (every address stays inside the operand;
+    // needs R >= BK); `shift` says how many of its leading reduction indices the
+    // previous step already covered -- those are zeroed before they reach LDS.
+    auto step_bases = [&](const char *&ga, const char *&gb, int &shift) {
+        const int r0 = ld_r0 + BK <= g.R ? ld_r0 : g.R - BK;
+        shift = ld_r0 - r0;
+        ga = tileA + ((RED ? (long)ld_img * g.rbA : 0L) + (LA == LD_XC_SCALAR ? (long)r0 * g.sA : (long)r0)) * 4;
+        gb = tileB + ((RED ? (long)ld_img * g.rbB : 0L) + (LB == LD_XC_SCALAR ? (long)r0 * g.sB : (long)r0)) * 4;
+    };
+    auto advance = [&]() {
         ld_r0 += BK;
         if (RED && ld_r0 >= g.R) {
             ld_r0 = 0;
             ++ld_img;
+        }
+    };
+    // Zero the elements whose position inside the step window is below `shift`.
+    auto mask_one = [&](auto kind_tag, int t_r, float *v, auto count_tag, int shift) {
+        constexpr int KIND = decltype(kind_tag)::value;
+        constexpr int CNT = decltype(count_tag)::value;
+#pragma unroll
+        for (int q = 0; q < CNT; ++q) {
+            const int rel = KIND == LD_RC_VEC ? t_r + (q & 3) : KIND == LD_RC_SCALAR ? t_r : t_r + q;
+            v[q] = rel < shift ? 0.0f : v[q];
         }
     };
 
@@ -212,26 +199,51 @@ __global__ __launch_bounds__(WGM *WGN * 64)
                     make_float4(src[w * 4], src[w * 4 + 1], src[w * 4 + 2], src[w * 4 + 3]);
         }
     };
-
-    auto stash = [&](int buf) {
+    auto stash = [&](int buf, int shift) {
+        if (shift > 0) {  // uniform: only the last step of an image can be partial
+            mask_one(std::integral_constant<int, LA>{}, a_r, ra, std::integral_constant<int, NA>{}, shift);
+            mask_one(std::integral_constant<int, LB>{}, b_r, rb, std::integral_constant<int, NB>{}, shift);
+        }
         stash_one(std::integral_constant<int, LA>{}, As[buf], a_x, a_r, ra, std::integral_constant<int, NA>{});
         stash_one(std::integral_constant<int, LB>{}, Bs[buf], b_x, b_r, rb, std::integral_constant<int, NB>{});
     };
 
+    // ---- prologue: first step ---------------------------------------------------------
+    const char *ga = tileA, *gb = tileB;
+    int shift = 0;
     if (nsteps > 0) {
-        fetch();
-        stash(0);
+        step_bases(ga, gb, shift);
+#pragma unroll
+        for (int u = 0; u < UA; ++u) load_unit(std::integral_constant<int, LA>{}, ga, g.sA, voffA, ra, u);
+#pragma unroll
+        for (int u = 0; u < UB; ++u) load_unit(std::integral_constant<int, LB>{}, gb, g.sB, voffB, rb, u);
+        stash(0, shift);
+        advance();
     }
     __syncthreads();
 
+    // ---- main loop ----------------------------------------------------------------------
+    // Step s computes from LDS buffer s&1 while the loads of step s+1 are issued
+    // in slices between its MFMAs (a steady trickle of requests; a burst at the
+    // head of the step would hold the wavefront, and with it its MFMAs, in the
+    // memory pipeline's queue) and written to the other buffer afterwards.
     for (int s = 0; s < nsteps; ++s) {
         const int buf = s & 1;
-        if (s + 1 < nsteps) fetch();
+        const bool more = !(DBG & 1) && s + 1 < nsteps;
+        // The last step has nothing to fetch; it re-reads the previous addresses
+        // (valid, cached) rather than branching around the loads.
+        if (more) step_bases(ga, gb, shift);
 
         // MFMA operands: 8 reduction indices per lane and block, two 128-bit reads.
         float4 av[TM][2], bv[TN][2];
+        if (DBG & 2) {
+            for (int h2 = 0; h2 < 2; ++h2) {
+                for (int a = 0; a < TM; ++a) av[a][h2] = make_float4(1.f + lane, 2.f, 3.f, 4.f);
+                for (int b = 0; b < TN; ++b) bv[b][h2] = make_float4(1.f, 2.f + lane, 3.f, 4.f);
+            }
+        }
 #pragma unroll
-        for (int h2 = 0; h2 < 2; ++h2) {
+        for (int h2 = 0; h2 < 2 && !(DBG & 2); ++h2) {
 #pragma unroll
             for (int a = 0; a < TM; ++a)
                 av[a][h2] = *reinterpret_cast<const float4 *>(&As[buf][wm * (TM * 32) + a * 32 + l32][8 * half + 4 * h2]);
@@ -243,6 +255,8 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         for (int h2 = 0; h2 < 2; ++h2) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
+                constexpr int SLICES = 8;
+                const int slice = h2 * 4 + e;
 #pragma unroll
                 for (int a = 0; a < TM; ++a) {
                     const float x = e == 0 ? av[a][h2].x : e == 1 ? av[a][h2].y : e == 2 ? av[a][h2].z : av[a][h2].w;
@@ -253,10 +267,24 @@ __global__ __launch_bounds__(WGM *WGN * 64)
                         acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, acc[a][b], 0, 0, 0);
                     }
                 }
+                if (!(DBG & 1)) {
+#pragma unroll
+                    for (int u = 0; u < UA; ++u)
+                        if (u * SLICES / UA == slice)
+                            load_unit(std::integral_constant<int, LA>{}, ga, g.sA, voffA, ra, u);
+#pragma unroll
+                    for (int u = 0; u < UB; ++u)
+                        if (u * SLICES / UB == slice)
+                            load_unit(std::integral_constant<int, LB>{}, gb, g.sB, voffB, rb, u);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-        if (s + 1 < nsteps) stash(buf ^ 1);
-        __syncthreads();
+        if (more) {
+            if (!(DBG & 4)) stash(buf ^ 1, shift);
+            advance();
+        }
+        if (!(DBG & 8)) __syncthreads();
     }
 
     // ---- epilogue ----------------------------------------------------------------------

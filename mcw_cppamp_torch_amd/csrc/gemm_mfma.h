@@ -81,8 +81,8 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 // How an operand tile travels from global memory to LDS.
 enum Loader {
-    LD_RC_VEC = 0,     // contiguous along r, 16-byte aligned rows: 128-bit loads along r
-    LD_RC_SCALAR = 1,  // contiguous along r, any alignment: 16 lanes read 16 consecutive r
+    LD_RC_VEC = 0,     // contiguous along r: 128-bit loads along r (rows need 4-byte alignment only)
+    LD_RC_SCALAR = 1,  // contiguous along r: 16 lanes read 16 consecutive r, one float each
     LD_XC_SCALAR = 2,  // contiguous along the free index: lanes read consecutive rows/columns
 };
 
@@ -92,6 +92,7 @@ int gemm_fast_128x128(const GemmArgs &g, int la, int lb, bool red, hipStream_t s
 int gemm_fast_128x256(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
 int gemm_fast_256x128(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
 int gemm_fast_64x64(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
+int gemm_fast_64x256(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
 // The bounds-checked kernel for shapes smaller than a tile (gemm_generic.hip).
 int gemm_generic_64x64(const GemmArgs &g, bool a_rc, bool b_rc, bool red, hipStream_t s);
 

@@ -4,16 +4,17 @@
 // SpatialConvolutionMM.c:179): col[b][k][n], k = (c*kH + kh)*kW + kw,
 // n = ho*Wo + wo; flat, the buffer is [B*C planes][kH*kW taps][Ho][Wo].
 //
-// im2col is store-bound (K*N floats out for C*H*W in).  Both kernels give a
-// wavefront a strip of consecutive output positions n of one (plane, kh) pair
-// and let it walk the kW taps, so the index arithmetic is paid once per strip
-// and every store instruction writes consecutive floats of one column row:
-//   * unit horizontal stride: a lane owns four consecutive n; per tap it reads
-//     four consecutive input pixels (one 128-bit load when they share an output
-//     row) and writes them with one 128-bit store;
-//   * strided: a lane owns one n and reads four consecutive taps at once (one
-//     128-bit load: consecutive lanes are sW floats apart, so the wavefront
-//     reads a contiguous span), writing one float to each of four column rows.
+// im2col is store-bound (K*N floats out for C*H*W in), so both kernels are
+// organised around the stores:
+//   * unit horizontal stride: the batch of columns is one flat array, a lane
+//     owns four consecutive floats of it and writes them with one aligned
+//     128-bit store (a wavefront covers 1 KiB: a strip of output rows of one
+//     tap); consecutive lanes read consecutive input pixels;
+//   * strided: a wavefront takes a strip of output positions n of one
+//     (plane, kh) pair, a lane owns one n and reads four consecutive taps at
+//     once (one 128-bit load: consecutive lanes are sW floats apart, so the
+//     wavefront reads a contiguous span) and writes one float to each of four
+//     column rows.
 // The input stays cache resident; HBM sees the image once and the columns once.
 //
 // col2im is a gather with no atomics: one lane per image pixel adds the
@@ -32,8 +33,7 @@ namespace {
 
 struct ConvGeom {
     int C, H, W, kH, kW, pH, pW, sH, sW, Ho, Wo, N;
-    int G;                              // groups of four output positions per column row
-    FastDiv divG, divN, divKH, divWo;   // im2col decomposition
+    FastDiv divN, divKH, divWo, divTaps, divKW;  // im2col decomposition
     FastDiv divW, divHW, divSH, divSW;  // col2im decomposition
 };
 
@@ -43,69 +43,61 @@ struct __attribute__((packed, aligned(4))) float4u {
     float x, y, z, w;
 };
 
-// Unit horizontal stride.  Thread t: prow = t / G (= plane*kH + kh), group = t % G.
-__global__ __launch_bounds__(256) void im2col_nvec_kernel(const float *__restrict__ im, float *__restrict__ col,
-                                                          const ConvGeom g, unsigned threads) {
-    const unsigned t = blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= threads) return;
-    unsigned prow, gi, plane, kh, ho, wo;
-    g.divG.divmod(t, prow, gi);
-    g.divKH.divmod(prow, plane, kh);
-    const int n0 = (int)gi * 4;
-    g.divWo.divmod((unsigned)n0, ho, wo);
-    const float *src = im + (long)plane * g.H * g.W;
-    float *out = col + (long)prow * g.kW * g.N + n0;
-    const bool full = n0 + 3 < g.N;
-    if ((int)wo + 3 < g.Wo) {
-        // The four outputs share an output row (and all exist).
-        const int iy = (int)ho * g.sH - g.pH + (int)kh;
-        const bool row_ok = iy >= 0 && iy < g.H;
-        const float *row = src + (long)(row_ok ? iy : 0) * g.W;
-        int ix = (int)wo - g.pW;
-        for (int kw = 0; kw < g.kW; ++kw, ++ix, out += g.N) {
-            float4u v;
-            if (row_ok && ix >= 0 && ix + 3 < g.W) {
-                v = *reinterpret_cast<const float4u *>(row + ix);
-            } else {
-                v.x = (row_ok && ix >= 0 && ix < g.W) ? row[ix] : 0.0f;
-                v.y = (row_ok && ix + 1 >= 0 && ix + 1 < g.W) ? row[ix + 1] : 0.0f;
-                v.z = (row_ok && ix + 2 >= 0 && ix + 2 < g.W) ? row[ix + 2] : 0.0f;
-                v.w = (row_ok && ix + 3 >= 0 && ix + 3 < g.W) ? row[ix + 3] : 0.0f;
-            }
-            *reinterpret_cast<float4u *>(out) = v;
-        }
-        return;
+__device__ inline float im2col_tap(const float *__restrict__ im, const ConvGeom &g, unsigned plane, unsigned tap,
+                                   unsigned ho, unsigned wo) {
+    unsigned kh, kw;
+    g.divKW.divmod(tap, kh, kw);
+    int iy = (int)ho * g.sH - g.pH + (int)kh;
+    int ix = (int)wo * g.sW - g.pW + (int)kw;
+    if (iy < 0 || iy >= g.H || ix < 0 || ix >= g.W) return 0.0f;
+    return im[((long)plane * g.H + iy) * g.W + ix];
+}
+
+// Unit horizontal stride: the whole column buffer is one flat array and every
+// lane owns four consecutive floats of it (one aligned 128-bit store; a
+// wavefront writes 1 KiB of consecutive columns).  total = floats in col.
+template <bool VEC>
+__global__ __launch_bounds__(256) void im2col_flat_kernel(const float *__restrict__ im, float *__restrict__ col,
+                                                     const ConvGeom g, long total, long chunk_base) {
+    long f = chunk_base + ((long)blockIdx.x * blockDim.x + threadIdx.x) * (VEC ? 4 : 1);
+    if (f >= total) return;
+    // f = row*N + n with row = plane*taps + tap; 32-bit magic division when the
+    // whole buffer is below 2^31 floats (uniform branch), 64-bit otherwise.
+    unsigned row, n;
+    if (total < (1L << 31)) {
+        g.divN.divmod((unsigned)f, row, n);
+    } else {
+        const long N = (long)g.Ho * g.Wo;
+        long r64 = f / N;
+        row = (unsigned)r64;
+        n = (unsigned)(f - r64 * N);
     }
-    // The group wraps to the next output row or runs past the end of the column row.
-    int yy[4], xx[4];
-    bool ok[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        ok[e] = n0 + e < g.N;
-        yy[e] = (int)ho * g.sH - g.pH + (int)kh;
-        xx[e] = (int)wo - g.pW;
-        if (++wo == (unsigned)g.Wo) {
-            wo = 0;
-            ++ho;
-        }
-    }
-    for (int kw = 0; kw < g.kW; ++kw, out += g.N) {
+    unsigned plane, tap, ho, wo;
+    g.divTaps.divmod(row, plane, tap);
+    g.divWo.divmod(n, ho, wo);
+    if (VEC) {
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const int x = xx[e] + kw;
-            const bool in = ok[e] && yy[e] >= 0 && yy[e] < g.H && x >= 0 && x < g.W;
-            v[e] = in ? src[(long)yy[e] * g.W + x] : 0.0f;
+            v[e] = (f + e < total) ? im2col_tap(im, g, plane, tap, ho, wo) : 0.0f;
+            if (++wo == (unsigned)g.Wo) {
+                wo = 0;
+                if (++ho == (unsigned)g.Ho) {
+                    ho = 0;
+                    if (++tap == g.divTaps.d) {
+                        tap = 0;
+                        ++plane;
+                    }
+                }
+            }
         }
-        if (full) {
-            float4u q;
-            q.x = v[0]; q.y = v[1]; q.z = v[2]; q.w = v[3];
-            *reinterpret_cast<float4u *>(out) = q;
+        if (f + 3 < total) {
+            *reinterpret_cast<float4 *>(col + f) = make_float4(v[0], v[1], v[2], v[3]);
         } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (ok[e]) out[e] = v[e];
+            for (int e = 0; e < 4 && f + e < total; ++e) col[f + e] = v[e];
         }
+    } else {
+        col[f] = im2col_tap(im, g, plane, tap, ho, wo);
     }
 }
 
@@ -192,8 +184,8 @@ int make_geom(ConvGeom &g, long B, int C, int H, int W, int kH, int kW, int pH, 
     g.Wo = (W + 2 * pW - kW) / sW + 1;
     if ((long)g.Ho * g.Wo >= (1L << 31)) return fail("im2col/col2im: output plane exceeds 32-bit indexing");
     g.N = g.Ho * g.Wo;
-    g.G = (g.N + 3) / 4;
-    g.divG = FastDiv((uint32_t)g.G);
+    g.divTaps = FastDiv((uint32_t)(kH * kW));
+    g.divKW = FastDiv((uint32_t)kW);
     g.divN = FastDiv((uint32_t)g.N);
     g.divKH = FastDiv((uint32_t)kH);
     g.divWo = FastDiv((uint32_t)g.Wo);
@@ -215,26 +207,43 @@ int im2col_launch(const float *im, long B, int C, int H, int W, int kH, int kW, 
     if (make_geom(g, B, C, H, W, kH, kW, pH, pW, sH, sW)) return 1;
     hipStream_t s = stream();
     if (!s) return 1;
+    const long total = B * (long)C * kH * kW * g.N;
+    if (total == 0) return 0;
+    const double bytes = 4.0 * ((double)B * C * H * W + (double)total);
+    if (sW == 1) {
+        const bool vec = ((uintptr_t)col & 15) == 0;
+        const long per_thread = vec ? 4 : 1;
+        const long threads = (total + per_thread - 1) / per_thread;
+        // At most 2^30 threads per launch keeps blockIdx.x*blockDim.x in range.
+        const long max_threads = 1L << 30;
+        for (long t0 = 0; t0 < threads; t0 += max_threads) {
+            const long nthr = threads - t0 < max_threads ? threads - t0 : max_threads;
+            const unsigned blocks = (unsigned)((nthr + 255) / 256);
+            {
+                LaunchScope scope("im2col", 0.0, bytes * ((double)nthr / threads));
+                if (vec)
+                    hipLaunchKernelGGL(im2col_flat_kernel<true>, dim3(blocks), dim3(256), 0, s, im, col, g, total,
+                                       t0 * 4);
+                else
+                    hipLaunchKernelGGL(im2col_flat_kernel<false>, dim3(blocks), dim3(256), 0, s, im, col, g, total,
+                                       t0);
+            }
+            if (check_launch("im2col")) return 1;
+        }
+        return 0;
+    }
     const long prows = B * (long)C * kH;  // (plane, kh) pairs
-    if (prows == 0) return 0;
-    const bool nvec = sW == 1;
-    const long per_prow = nvec ? g.G : g.N;
-    // The batch is cut into launches of at most 2^31 - 1 threads (whole prows each).
-    const long max_prows = ((1L << 31) - 256) / per_prow / kH * kH;  // whole planes per launch
+    const long max_prows = ((1L << 31) - 256) / g.N / kH * kH;  // whole planes per launch
     if (max_prows < kH) return fail("im2col: column rows too long for one launch");
-    const double bytes_per_prow = 4.0 * ((double)kW * g.N + (double)H * W / kH);
     for (long p0 = 0; p0 < prows; p0 += max_prows) {
         const long np = prows - p0 < max_prows ? prows - p0 : max_prows;
-        const unsigned threads = (unsigned)(np * per_prow);
+        const unsigned threads = (unsigned)(np * g.N);
         const unsigned blocks = (threads + 255) / 256;
         const float *im0 = im + (p0 / kH) * (long)H * W;
         float *col0 = col + p0 * (long)kW * g.N;
         {
-            LaunchScope scope("im2col", 0.0, bytes_per_prow * np);
-            if (nvec)
-                hipLaunchKernelGGL(im2col_nvec_kernel, dim3(blocks), dim3(256), 0, s, im0, col0, g, threads);
-            else
-                hipLaunchKernelGGL(im2col_tapvec_kernel, dim3(blocks), dim3(256), 0, s, im0, col0, g, threads);
+            LaunchScope scope("im2col", 0.0, bytes * ((double)np / prows));
+            hipLaunchKernelGGL(im2col_tapvec_kernel, dim3(blocks), dim3(256), 0, s, im0, col0, g, threads);
         }
         if (check_launch("im2col")) return 1;
     }
