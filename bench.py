@@ -144,6 +144,16 @@ def main():
     dev_ms = ev0.elapsed_ms(ev1)
     ms_per_step = wall * 1e3 / args.steps
 
+    # Host<->device copies of one batch (blocking, pageable host memory), outside the timed region.
+    host_x = stacks.make_input(name, B, seed=1000)
+    t1 = time.perf_counter()
+    x.copy(host_x)
+    gputorch.synchronize()
+    h2d_ms = (time.perf_counter() - t1) * 1e3
+    t1 = time.perf_counter()
+    net.gradInput.float()
+    d2h_ms = (time.perf_counter() - t1) * 1e3
+
     w = stacks.work(name, B)
     kernels, roofline = {}, None
     if not args.no_kernel_timing:
@@ -191,6 +201,8 @@ def main():
                                "updateGradInput, accGradParameters)" % (name, B, "x".join(map(str, stacks.STACKS[name]["input"]))),
                    "batch": B, "device": gputorch.getDeviceProperties()["name"]},
         "device_ms_per_step": round(dev_ms / args.steps, 4),
+        "transfers": {"h2d_input_ms": round(h2d_ms, 3), "d2h_gradinput_ms": round(d2h_ms, 3),
+                      "images_per_s_including_transfers": round(B / ((ms_per_step + h2d_ms + d2h_ms) / 1e3), 1)},
         "gemm_tflops_over_whole_step": round(w["gemm_flops"] / (ms_per_step / 1e3) / 1e12, 2),
         "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels,
     }
