@@ -101,7 +101,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="alexnet", choices=["alexnet", "overfeat", "vgg_a", "conv1_b16"])
     ap.add_argument("--batch", type=int, default=None, help="override the workload's batch size")
-    ap.add_argument("--cpu-sample-batch", type=int, default=16)
+    ap.add_argument("--cpu-sample-batch", type=int, default=128)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     args = ap.parse_args()
