@@ -127,12 +127,14 @@ int gemm_launch(const GemmProblem &p) {
     // The fast kernel addresses each operand as a uniform base plus a 32-bit
     // per-thread byte offset and moves a partial last step back by up to 15
     // reduction indices: it needs R >= 16 and tile-local offsets below 2^30 floats.
+    // The output is addressed the same way (four rows and a tile's columns per lane).
     const long n_img = g.N;
     auto offsets_fit = [&](int bm, int bn) {
         const long offA = p.a_rc ? (long)(bm - 1) * p.sA + GEMM_BK : (long)(GEMM_BK - 1) * p.sA + bm;
         const long span = (bn - 1) / n_img + 2;  // images a tile's columns can touch
         const long offB = p.b_rc ? (long)(bn - 1) * p.sB + GEMM_BK : (long)(GEMM_BK - 1) * p.sB + span * p.bsB + n_img;
-        return offA < (1L << 30) && offB < (1L << 30);
+        const long offC = 4 * (p.sC > p.J ? p.sC : (long)p.J) + span * p.bsC + n_img;
+        return offA < (1L << 30) && offB < (1L << 30) && offC < (1L << 30);
     };
     const bool fast_ok = p.R == 0 || p.R >= GEMM_BK;
     for (const TileCfg &c : kCfgs) {

@@ -46,7 +46,8 @@ constexpr int gemm_min_waves() {
 }
 
 // DBG is 0 in the library; experiments switch phases off with it (1: no global
-// fetch in the loop, 2: no LDS operand reads, 4: no LDS stores, 8: no barrier).
+// fetch in the loop, 2: no LDS operand reads, 4: no LDS stores, 8: no barrier,
+// 16: epilogue stores only one value per lane).
 template <int BM, int BN, int WGM, int WGN, int LA, int LB, bool RED, int DBG = 0>
 __global__ __launch_bounds__(WGM *WGN * 64)
     __attribute__((amdgpu_waves_per_eu(gemm_min_waves<BM, BN, WGM, WGN>()))) void gemm_fast_kernel(const GemmArgs g) {
@@ -63,7 +64,7 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     __shared__ __attribute__((aligned(16))) float Bs[2][BN][LDK];
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: row bases stay uniform
     const int wm = wave / WGN, wn = wave % WGN;
     const int half = lane >> 5, l32 = lane & 31;
 
@@ -208,6 +209,16 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         stash_one(std::integral_constant<int, LB>{}, Bs[buf], b_x, b_r, rb, std::integral_constant<int, NB>{});
     };
 
+    if (DBG & 32) {
+        // experiment: stagger the first generation of workgroups
+        if (blockIdx.x < 1024u) {
+            const unsigned phase = (blockIdx.x * 2654435761u >> 13) & 3u;
+            const long wait = (long)phase * nsteps * (2048L * 4 / 4);
+            const long t0 = (long)__builtin_readcyclecounter();
+            while ((long)__builtin_readcyclecounter() - t0 < wait) __builtin_amdgcn_s_sleep(32);
+        }
+    }
+
     // ---- prologue: first step ---------------------------------------------------------
     const char *ga = tileA, *gb = tileB;
     int shift = 0;
@@ -289,39 +300,67 @@ __global__ __launch_bounds__(WGM *WGN * 64)
 
     // ---- epilogue ----------------------------------------------------------------------
     // Accumulator register v of lane l holds D[8*(v/4) + 4*(l/32) + v%4][l%32].
-    const bool partial = g.nsplit > 1;
+    // A store address is a wave-uniform row base plus a constant per-lane byte
+    // offset (column, image and the lane half's four rows), as for the loads.
+    // MODE 0: partial sums to the workspace; 1: alpha*acc (+bias); 2: also + beta*C.
+    const bool rows_shifted = i0 != own_i0;
+    auto write_out = [&](auto mode_tag, auto check_tag) {
+        constexpr int MODE = decltype(mode_tag)::value;
+        constexpr bool CHECK = decltype(check_tag)::value;
+        const long row_bytes = (MODE == 0 ? (long)g.J : g.sC) * 4;
+        char *const out0 = MODE == 0 ? reinterpret_cast<char *>(g.ws + (long)split * g.M * g.J)
+                                     : reinterpret_cast<char *>(g.C);
+        unsigned img0 = 0, n0 = 0;
+        const bool per_image = MODE != 0 && !RED && g.N != g.J;
+        if (per_image) g.divN.divmod((unsigned)j0, img0, n0);
+        char *const out = out0 + (per_image ? (long)img0 * g.bsC : (long)j0) * 4;
 #pragma unroll
-    for (int b = 0; b < TN; ++b) {
-        const int jg = j0 + wn * (TN * 32) + b * 32 + l32;
-        if (jg < own_j0) continue;  // owned by the neighbouring tile
-        long coff;
-        if (partial) {
-            coff = (long)split * g.M * g.J + jg;
-        } else if (!RED && g.N != g.J) {
-            unsigned im, n;
-            g.divN.divmod((unsigned)jg, im, n);
-            coff = (long)im * g.bsC + n;
-        } else {
-            coff = jg;
-        }
+        for (int b = 0; b < TN; ++b) {
+            const int jg = j0 + wn * (TN * 32) + b * 32 + l32;
+            if (jg < own_j0) continue;  // owned by the neighbouring tile
+            long col = jg - j0;
+            if (per_image) {
+                unsigned im, n;
+                g.divN.divmod((unsigned)jg, im, n);
+                col = (long)(im - img0) * g.bsC + n;
+            }
+            const unsigned voff = (unsigned)(col * 4 + 4 * half * row_bytes);
 #pragma unroll
-        for (int a = 0; a < TM; ++a) {
+            for (int a = 0; a < TM; ++a) {
+                const int iu = i0 + wm * (TM * 32) + a * 32;  // uniform
+                float bias_v[16];
+                if (MODE != 0 && g.bias) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int i = i0 + wm * (TM * 32) + a * 32 + 8 * (v / 4) + 4 * half + (v % 4);
-                if (i < own_i0) continue;
-                float val = acc[a][b][v];
-                if (partial) {
-                    g.ws[coff + (long)i * g.J] = val;
+                    for (int v = 0; v < 16; ++v)
+                        bias_v[v] = *reinterpret_cast<const float *>(
+                            reinterpret_cast<const char *>(g.bias + iu + 8 * (v / 4) + (v % 4)) + 16 * half);
                 } else {
-                    float *c = g.C + (long)i * g.sC + coff;
-                    val *= g.alpha;
-                    if (g.bias) val += g.bias[i];
-                    if (g.beta != 0.0f) val += g.beta * *c;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) bias_v[v] = 0.0f;
+                }
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int ir = iu + 8 * (v / 4) + (v % 4);  // uniform; the lane's row is ir + 4*half
+                    if (CHECK && ir + 4 * half < own_i0) continue;
+                    float *c = reinterpret_cast<float *>(out + (long)ir * row_bytes + voff);
+                    float val = acc[a][b][v];
+                    if ((DBG & 16) && (v != 0 || val != 12345.0f)) continue;
+                    if (MODE != 0) val = val * g.alpha + bias_v[v];
+                    if (MODE == 2) val += g.beta * *c;
                     *c = val;
                 }
             }
         }
+    };
+    using std::integral_constant;
+    if (g.nsplit > 1) {
+        if (rows_shifted) write_out(integral_constant<int, 0>{}, integral_constant<bool, true>{});
+        else write_out(integral_constant<int, 0>{}, integral_constant<bool, false>{});
+    } else if (g.beta == 0.0f) {
+        if (rows_shifted) write_out(integral_constant<int, 1>{}, integral_constant<bool, true>{});
+        else write_out(integral_constant<int, 1>{}, integral_constant<bool, false>{});
+    } else {
+        write_out(integral_constant<int, 2>{}, integral_constant<bool, true>{});
     }
 }
 
