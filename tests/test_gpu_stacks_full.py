@@ -1,0 +1,79 @@
+"""GPU parity at the full benchmark sizes, layer by layer.
+
+Each stack (AlexNet-style b128, OverFeat-fast-style b128, VGG-A-style b64) runs
+once through the CPU oracle; then every GPU module is fed the ORACLE's input and
+gradOutput of its layer, so a layer's result is compared at the strict bar and
+does not inherit the rounding of the layers before it:
+  * conv output / gradInput / gradWeight / gradBias within 1e-4*sqrt(reduction
+    length) (max error relative to the largest reference magnitude);
+  * the im2col buffer, max-pool output, argmax-driven gradient and ReLU
+    bit-exact.
+The oracle's sgemm runs on the host BLAS here (tests/test_oracle_math.py pins
+that path against the reference's plain loops).
+"""
+import numpy as np
+import pytest
+
+from helpers import gemm_tol, oracle_stack, rel_err, rng_for, uniform
+
+pytestmark = pytest.mark.gpu
+
+import oracle  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def gt():
+    import mcw_cppamp_torch_amd as pkg
+    assert pkg._lib.lib.thgpu_init() == 0, pkg._lib.lib.thgpu_last_error()
+    return pkg
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+def dev(gt, a):
+    return gt.GPUTensor.from_numpy(np.ascontiguousarray(a, np.float32))
+
+
+@pytest.mark.parametrize("name", ["alexnet", "overfeat", "vgg_a"])
+def test_full_size_stack_layerwise(gt, name):
+    stacks = gt.stacks
+    cfg = stacks.STACKS[name]
+    B, layers = cfg["batch"], cfg["layers"]
+    net = stacks.build(name, seed_base=4000)
+    params = [(np.array(m.weight), np.array(m.bias)) if hasattr(m, "weight") else None for m in net.modules]
+    x = stacks.make_input(name, B, seed=4000)
+    go = uniform(rng_for(4003), stacks.output_shape(name, B))
+    oracle.use_blas(True)
+    try:
+        outs, gins, grads = oracle_stack(layers, params, x, go)
+    finally:
+        oracle.use_blas(False)
+    net.gpu()
+    ins = [x] + outs[:-1]
+    gouts = gins[1:] + [go]
+    for i, (l, m) in enumerate(zip(layers, net.modules)):
+        print("%s layer %d %s in %s" % (name, i, l, ins[i].shape), flush=True)
+        dx, dgo = dev(gt, ins[i]), dev(gt, gouts[i])
+        m.zeroGradParameters()
+        out = m.forward(dx).float()
+        gi = m.backward(dx, dgo).float()
+        if l[0] == "conv":
+            _, cin, cout, kW, kH, dW, dH, pW, pH = l
+            K = cin * kH * kW
+            N = outs[i].shape[2] * outs[i].shape[3]
+            assert rel_err(out, outs[i]) < gemm_tol(K), (name, i)
+            assert rel_err(gi, gins[i]) < gemm_tol(cout), (name, i)
+            assert rel_err(m.gradWeight.float(), grads[i][0]) < gemm_tol(B * N), (name, i)
+            assert rel_err(m.gradBias.float(), grads[i][1]) < gemm_tol(B * N), (name, i)
+            if B * K * N * 4 <= (1 << 30):  # the column buffer, where the copy back stays modest
+                ref_cols = oracle.im2col(ins[i], kH, kW, pH, pW, dH, dW)
+                assert np.array_equal(bits(m.finput.float()), bits(ref_cols)), (name, i)
+        else:
+            assert np.array_equal(bits(out), bits(outs[i])), (name, i)
+            assert np.array_equal(bits(gi), bits(gins[i])), (name, i)
+            if l[0] == "pool":
+                _, ind_ref = oracle.maxpool_updateOutput(ins[i], l[2], l[1], l[4], l[3])
+                assert np.array_equal(bits(m.indices.float()), bits(ind_ref)), (name, i)
+        del dx, dgo, out, gi
