@@ -4,18 +4,22 @@
 // SpatialConvolutionMM.c:179): col[b][k][n], k = (c*kH + kh)*kW + kw,
 // n = ho*Wo + wo; flat, the buffer is [B*C planes][kH*kW taps][Ho][Wo].
 //
-// im2col is store-bound (K*N floats out for C*H*W in), so both kernels are
-// organised around the stores:
-//   * unit horizontal stride: the batch of columns is one flat array, a lane
-//     owns four consecutive floats of it and writes them with one aligned
-//     128-bit store (a wavefront covers 1 KiB: a strip of output rows of one
-//     tap); consecutive lanes read consecutive input pixels;
-//   * strided: a wavefront takes a strip of output positions n of one
-//     (plane, kh) pair, a lane owns one n and reads four consecutive taps at
-//     once (one 128-bit load: consecutive lanes are sW floats apart, so the
-//     wavefront reads a contiguous span) and writes one float to each of four
-//     column rows.
-// The input stays cache resident; HBM sees the image once and the columns once.
+// im2col is store-bound (K*N floats out for C*H*W in) and, at four cycles per
+// wavefront instruction, easily instruction-bound as well, so the kernel is
+// organised to spend about three instructions per 64 floats written.  A
+// workgroup takes a strip of output rows of one plane (or several whole planes
+// when they are small) and copies the input rows that strip needs into LDS
+// once, zero padding included, so nothing downstream checks a bound.  Then a
+// lane owns a few output positions n, keeps their LDS addresses in registers,
+// and walks the taps: per tap and position one LDS read at a scalar offset and
+// one 4-byte store whose address is a scalar row base plus the lane's fixed
+// offset -- the wavefront writes 256 consecutive bytes of one column row.  HBM
+// sees the image once (plus the halo rows between strips) and the columns
+// once, for any stride, and no store depends on the alignment of a row.
+// Geometries whose strip of input rows does not fit in LDS (rows of many
+// thousands of pixels) fall back to two direct kernels: a flat one for unit
+// horizontal stride (a lane owns four consecutive floats of the column buffer)
+// and one that reads four taps at a time for strided convolutions.
 //
 // col2im is a gather with no atomics: one lane per image pixel adds the
 // column entries that cover it, kh ascending then kw ascending from +0.0f --
@@ -25,6 +29,9 @@
 // consecutive in wo.  Candidate taps are visited in groups of four with
 // clamped addresses and the invalid ones contribute +0.0f (which leaves a
 // float sum unchanged), so the loads of a group are in flight together.
+#include <cstdio>
+#include <cstdlib>
+
 #include "common.h"
 
 namespace thgpu {
@@ -51,6 +58,207 @@ __device__ inline float im2col_tap(const float *__restrict__ im, const ConvGeom 
     int ix = (int)wo * g.sW - g.pW + (int)kw;
     if (iy < 0 || iy >= g.H || ix < 0 || ix >= g.W) return 0.0f;
     return im[((long)plane * g.H + iy) * g.W + ix];
+}
+
+// Launch shape of the LDS-staged im2col.
+struct StripPlan {
+    int G;        // planes per workgroup (more than one only when a strip is the whole plane)
+    int TR;       // output rows per strip
+    int tiles;    // strips per plane
+    int PL;       // lanes along the positions (multiple of 64)
+    int TG;       // lane groups along the taps
+    int LW;       // input columns kept per row: (Wo-1)*sW + kW
+    int LH;       // input rows kept per strip: (TR-1)*sH + kH
+    FastDiv divTiles, divLP, divLW;
+};
+
+// The LDS-staged kernel described at the top of the file.  NS = position slots per lane and pass.
+template <int NS>
+__global__ __launch_bounds__(256) void im2col_strip_kernel(const float *__restrict__ im, float *__restrict__ col,
+                                                           const ConvGeom g, const StripPlan p, unsigned planes) {
+    extern __shared__ float tile[];
+    const int tid = threadIdx.x, nthr = blockDim.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), nwaves = nthr >> 6;
+    unsigned grp, strip;
+    p.divTiles.divmod(blockIdx.x, grp, strip);
+    const unsigned plane0 = grp * (unsigned)p.G;
+    const int np = (int)(planes - plane0 < (unsigned)p.G ? planes - plane0 : (unsigned)p.G);
+    const int r0 = (int)strip * p.TR;
+    const int nr = g.Ho - r0 < p.TR ? g.Ho - r0 : p.TR;
+    const int LP = p.LH * p.LW;
+
+    // ---- stage the input rows -----------------------------------------------------------
+    // tile[pl][r][c] is input pixel (r0*sH - pH + r, c - pW) of plane plane0+pl,
+    // or zero outside the image.  Eight loads are in flight per lane before
+    // the first is written to LDS.
+    const int iy0 = r0 * g.sH - g.pH;
+    if (p.LW >= 48 && p.LW <= 128) {
+        // a wavefront takes whole rows: row number and source pointer are scalar, lanes run along the row
+        const int rows = np * p.LH;
+        for (int rb = wave; rb < rows; rb += 4 * nwaves) {
+            float v[4][2];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int row = rb + u * nwaves;
+                const int pl = row / p.LH, r = row - pl * p.LH;
+                const int iy = iy0 + r;
+                const bool row_ok = row < rows && iy >= 0 && iy < g.H;
+                const float *src = im + ((long)(plane0 + pl) * g.H + (row_ok ? iy : 0)) * g.W - g.pW;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int c = lane + 64 * h, ix = c - g.pW;
+                    v[u][h] = (row_ok && c < p.LW && ix >= 0 && ix < g.W) ? src[c] : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int row = rb + u * nwaves;
+                if (row < rows) {
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const int c = lane + 64 * h;
+                        if (c < p.LW) tile[row * p.LW + c] = v[u][h];
+                    }
+                }
+            }
+        }
+    } else {
+        // narrow or very wide rows: the tile as one flat array
+        const int E = np * LP;
+        for (int e0 = tid; e0 < E; e0 += nthr * 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int idx = e0 + u * nthr;
+                unsigned pl, rem, r, c;
+                p.divLP.divmod((unsigned)(idx < E ? idx : 0), pl, rem);
+                p.divLW.divmod(rem, r, c);
+                const int iy = iy0 + (int)r, ix = (int)c - g.pW;
+                const bool ok = idx < E && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
+                v[u] = ok ? im[((long)(plane0 + pl) * g.H + iy) * g.W + ix] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int idx = e0 + u * nthr;
+                if (idx < E) tile[idx] = v[u];
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- write the columns --------------------------------------------------------------
+    // Positions of the workgroup: i = pl*Pn + n' over its planes and the strip's
+    // Pn output positions.  A lane takes positions i = pi, pi + PL, ... (at
+    // most four per pass) and keeps, for each, the LDS address of its tap
+    // (0,0) and its byte offset from the column row of plane0 and tap 0.
+    const int Pn = nr * g.Wo;
+    const int total = np * Pn;
+    const int pi = tid % p.PL;
+    const int tg = __builtin_amdgcn_readfirstlane(tid / p.PL);  // PL is a multiple of 64: uniform
+    const int taps = g.kH * g.kW;
+    const long plane_floats = (long)taps * g.N;
+    // scalar: start of (plane0, tap 0, first position of the strip)
+    char *const row0 = reinterpret_cast<char *>(col + (long)plane0 * plane_floats + (long)r0 * g.Wo);
+    for (int base = 0; base < total; base += NS * p.PL) {
+        int lb[NS];
+        unsigned voff[NS];
+#pragma unroll
+        for (int e = 0; e < NS; ++e) {
+            // A lane past the end repeats the last position: the same value to the same address.
+            int i = base + e * p.PL + pi;
+            i = i < total ? i : total - 1;
+            unsigned pl = 0, n = (unsigned)i, hr, wo;
+            if (p.G > 1) g.divN.divmod(n, pl, n);  // grouped planes are whole: Pn == N
+            g.divWo.divmod(n, hr, wo);
+            lb[e] = ((int)pl * LP + (int)hr * g.sH * p.LW + (int)wo * g.sW) * 4;
+            voff[e] = (unsigned)(((long)pl * plane_floats + n) * 4);
+            asm volatile("" : "+v"(lb[e]), "+v"(voff[e]));  // keep both as single registers
+        }
+        int kh = tg / g.kW, kw = tg - kh * g.kW;
+        for (int tap = tg; tap < taps; tap += p.TG) {
+            const int loff = (kh * p.LW + kw) * 4;
+            char *const row = row0 + (long)tap * g.N * 4;  // scalar
+            float v[NS];
+#pragma unroll
+            for (int e = 0; e < NS; ++e)
+                v[e] = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(tile) + (lb[e] + loff));
+#pragma unroll
+            for (int e = 0; e < NS; ++e) *reinterpret_cast<float *>(row + voff[e]) = v[e];
+            kw += p.TG;
+            while (kw >= g.kW) {
+                kw -= g.kW;
+                ++kh;
+            }
+        }
+    }
+}
+
+// Chooses the strip shape; false when even one output row's input rows exceed the LDS budget.
+// A workgroup of PL*TG lanes runs ceil(positions/PL) slots (at most four, one
+// pass) over ceil(taps/TG) taps; lanes past the strip's end repeat stores.
+// Measured on gfx950 (strip-shape sweeps over the AlexNet/OverFeat/VGG layer
+// geometries): three slots of a wide PL run best, planes of up to 1024
+// positions are best taken whole, small planes are best grouped by few.
+bool plan_strips(const ConvGeom &g, long planes, StripPlan &p) {
+    constexpr long kLdsBytes = 32 * 1024;
+    p.LW = (g.Wo - 1) * g.sW + g.kW;
+    auto bytes = [&](long G, long TR) { return G * ((TR - 1) * g.sH + g.kH) * (long)p.LW * 4; };
+    if (bytes(1, 1) > kLdsBytes) return false;
+    const int taps = g.kH * g.kW;
+    const bool grouped = g.N <= 256;                 // several whole planes per workgroup
+    const bool whole = !grouped && g.N <= 1024 && bytes(1, g.Ho) <= kLdsBytes;  // one whole plane
+    if (grouped && bytes(1, g.Ho) > kLdsBytes) return false;
+    // THGPU_IM2COL_PLAN="v,PL,TG" pins the shape (a tuning aid): v = planes per group or rows per strip.
+    int fv = 0, fPL = 0, fTG = 0;
+    if (const char *e = std::getenv("THGPU_IM2COL_PLAN")) std::sscanf(e, "%d,%d,%d", &fv, &fPL, &fTG);
+    long vmax = grouped ? 1024 / g.N : whole ? g.Ho : 1024 / g.Wo;
+    if (grouped && vmax > planes) vmax = planes;
+    if (!grouped && vmax > g.Ho) vmax = g.Ho;
+    if (vmax < 1) vmax = 1;
+    double best = -1;
+    for (long v = whole ? g.Ho : 1; v <= vmax; ++v) {
+        if (fv > 0 && v != (fv < vmax ? fv : vmax)) continue;
+        const long G = grouped ? v : 1, TR = grouped ? g.Ho : v;
+        if (bytes(G, TR) > kLdsBytes) break;
+        if ((long)G * taps * g.N * 4 >= (1L << 32)) break;  // lane offsets are 32-bit
+        if (!grouped && !whole && fv == 0) {
+            const long tiles = (g.Ho + TR - 1) / TR;
+            if (TR != (g.Ho + tiles - 1) / tiles) continue;  // only even strips
+        }
+        const long positions = grouped ? G * (long)g.N : TR * (long)g.Wo;
+        for (int PL = 64; PL <= 256; PL += 64) {
+            if (fPL > 0 && PL != fPL) continue;
+            const long slots = (positions + PL - 1) / PL;
+            if (slots > 4 && !(v == 1 && PL == 256)) continue;  // more than one pass only when unavoidable
+            static const double kSlotWeight[5] = {0, 0.8, 0.9, 1.0, 0.95};
+            double score = (double)positions / (double)(slots * PL) * (slots <= 4 ? kSlotWeight[slots] : 0.5);
+            if (!grouped && PL < 256) score *= 0.9;          // strips: wide workgroups measured faster
+            score += grouped ? -1e-4 * v : 0.0;              // ties: few planes per group
+            if (score > best) {
+                best = score;
+                p.G = (int)G;
+                p.TR = (int)TR;
+                p.PL = PL;
+            }
+        }
+    }
+    if (best < 0) return false;
+    p.TG = 1;
+    double eff_best = 0;
+    for (int tg = 1; tg <= 256 / p.PL; ++tg) {
+        if (fTG > 0 && tg != (fTG < 256 / p.PL ? fTG : 256 / p.PL)) continue;
+        const double eff = (double)taps / (tg * ((taps + tg - 1) / tg));
+        if (eff >= eff_best) {
+            eff_best = eff;
+            p.TG = tg;
+        }
+    }
+    p.tiles = (g.Ho + p.TR - 1) / p.TR;
+    p.LH = (p.TR - 1) * g.sH + g.kH;
+    p.divTiles = FastDiv((uint32_t)p.tiles);
+    p.divLP = FastDiv((uint32_t)(p.LH * p.LW));
+    p.divLW = FastDiv((uint32_t)p.LW);
+    return true;
 }
 
 // Unit horizontal stride: the whole column buffer is one flat array and every
@@ -210,6 +418,33 @@ int im2col_launch(const float *im, long B, int C, int H, int W, int kH, int kW, 
     const long total = B * (long)C * kH * kW * g.N;
     if (total == 0) return 0;
     const double bytes = 4.0 * ((double)B * C * H * W + (double)total);
+    StripPlan plan;
+    const long planes = B * (long)C;
+    // THGPU_IM2COL_DIRECT=1 forces the direct kernels, =0 the LDS-staged one (testing and tuning aids).
+    const char *direct = std::getenv("THGPU_IM2COL_DIRECT");
+    // Strided convolutions (few, large first layers) measured faster on the direct kernel.
+    if (!(direct && direct[0] == '1') && (sW == 1 || (direct && direct[0] == '0')) && plan_strips(g, planes, plan)) {
+        const long groups = (planes + plan.G - 1) / plan.G;
+        const long blocks = groups * plan.tiles;
+        if (blocks < (1L << 31) && planes < (1L << 31)) {
+            const size_t lds = sizeof(float) * (size_t)plan.G * plan.LH * plan.LW;
+            {
+                LaunchScope scope("im2col", 0.0, bytes);
+                const long positions = (long)plan.G * plan.TR * g.Wo;
+                const long slots = (positions + plan.PL - 1) / plan.PL;
+                const dim3 grid((unsigned)blocks), block(plan.PL * plan.TG);
+                if (slots <= 1)
+                    hipLaunchKernelGGL(im2col_strip_kernel<1>, grid, block, lds, s, im, col, g, plan, (unsigned)planes);
+                else if (slots == 2)
+                    hipLaunchKernelGGL(im2col_strip_kernel<2>, grid, block, lds, s, im, col, g, plan, (unsigned)planes);
+                else if (slots == 3)
+                    hipLaunchKernelGGL(im2col_strip_kernel<3>, grid, block, lds, s, im, col, g, plan, (unsigned)planes);
+                else
+                    hipLaunchKernelGGL(im2col_strip_kernel<4>, grid, block, lds, s, im, col, g, plan, (unsigned)planes);
+            }
+            return check_launch("im2col");
+        }
+    }
     if (sW == 1) {
         const bool vec = ((uintptr_t)col & 15) == 0;
         const long per_thread = vec ? 4 : 1;

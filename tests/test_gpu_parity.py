@@ -54,8 +54,18 @@ GEOMS = [
 ]
 
 
+@pytest.fixture(params=[None, "0", "1"], ids=["auto", "lds_staged", "direct"])
+def im2col_kernel(request, monkeypatch):
+    """Runs a test with the library's own kernel choice, then with each im2col kernel forced."""
+    if request.param is None:
+        monkeypatch.delenv("THGPU_IM2COL_DIRECT", raising=False)
+    else:
+        monkeypatch.setenv("THGPU_IM2COL_DIRECT", request.param)
+    return request.param
+
+
 @pytest.mark.parametrize("geo", GEOMS)
-def test_im2col_bit_exact(gt, geo):
+def test_im2col_bit_exact(gt, geo, im2col_kernel):
     B, C, H, W, kH, kW, pH, pW, sH, sW = geo
     im = uniform(rng_for(21), (B, C, H, W))
     ref = oracle.im2col(im, kH, kW, pH, pW, sH, sW)
@@ -67,7 +77,7 @@ def test_im2col_bit_exact(gt, geo):
     assert np.array_equal(bits(d_col.float()), bits(ref))
 
 
-def test_im2col_unaligned_destination_uses_scalar_path(gt):
+def test_im2col_unaligned_destination(gt, im2col_kernel):
     B, C, H, W, kH, kW, pH, pW, sH, sW = 2, 3, 9, 11, 3, 3, 1, 1, 2, 1
     im = uniform(rng_for(22), (B, C, H, W))
     ref = oracle.im2col(im, kH, kW, pH, pW, sH, sW)
