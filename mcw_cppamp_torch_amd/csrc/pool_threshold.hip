@@ -6,16 +6,21 @@
 // (mcw_nn/generic/SpatialMaxPooling.c:30-45).  The two index planes hold
 // ky+1 and kx+1 as floats (:51-52).
 //
-// Max-pool backward is index driven and atomics-free: one lane per input
-// pixel visits the windows that cover it in (i ascending, j ascending) order
-// and adds gradOutput where the saved argmax points back at the pixel.  This
-// is the float addition order of the CPU module's scatter (:165-174), so
-// overlapping windows give bit-identical sums, and no zero-fill pass is
-// needed.  It replaces gpunn-impl/SpatialMaxPooling.cpp:87-203, which only
-// handled non-overlapping windows.
+// Max-pool backward is index driven and atomics-free: every input pixel visits
+// the windows that cover it in (i ascending, j ascending) order and adds
+// gradOutput where the saved argmax points back at the pixel.  This is the
+// float addition order of the CPU module's scatter (:165-174), so overlapping
+// windows give bit-identical sums, and no zero-fill pass is needed.  It
+// replaces gpunn-impl/SpatialMaxPooling.cpp:87-203, which only handled
+// non-overlapping windows.  A workgroup takes a strip of pixel rows of one
+// plane (or several small planes), turns the windows that can reach it into
+// (target pixel, gradient) pairs in LDS -- padded with pairs that target no
+// pixel, so the pixel loop has no bounds to check -- and then each pixel
+// compares at most ceil(kH/dH)*ceil(kW/dW) pairs against its own index.
 #include "common.h"
 
 #include <cmath>
+#include <cstdlib>
 
 namespace thgpu {
 
@@ -74,6 +79,127 @@ __global__ __launch_bounds__(256) void maxpool_fwd_kernel(const float *__restric
     indx[o] = by < 0 ? 0.0f : (float)(bx + 1);
 }
 
+// Launch shape of the LDS-tile backward kernel.
+struct PoolBwdPlan {
+    int G;      // planes per workgroup (more than one only when a strip is the whole plane)
+    int PR;     // pixel rows per strip
+    int tiles;  // strips per plane
+    int RW;     // window rows kept per strip (with TH-1 rows of history)
+    int CW;     // window columns kept per row (with TW-1 columns of history and the uncovered right edge)
+    FastDiv divTiles, divEnt, divCW, divPix;
+};
+
+// TH x TW = the most windows that can cover one pixel.  Pixel (h, w) can only
+// be the argmax of windows (i_hi - a, j_hi - b), i_hi = h / dH, j_hi = w / dW,
+// a < TH, b < TW; visiting a and b downwards is (i ascending, j ascending).
+template <int TH, int TW>
+__global__ __launch_bounds__(256) void maxpool_bwd_tile_kernel(const float *__restrict__ gout,
+                                                               const float *__restrict__ indy,
+                                                               const float *__restrict__ indx,
+                                                               float *__restrict__ gin, const PoolGeom g,
+                                                               const PoolBwdPlan p, unsigned planes) {
+    extern __shared__ int2 ent[];  // [G][RW][CW]: (target pixel inside the plane or -1, gradient bits)
+    const int tid = threadIdx.x, nthr = blockDim.x;
+    unsigned grp, strip;
+    p.divTiles.divmod(blockIdx.x, grp, strip);
+    const unsigned plane0 = grp * (unsigned)p.G;
+    const int np = (int)(planes - plane0 < (unsigned)p.G ? planes - plane0 : (unsigned)p.G);
+    const int h0 = (int)strip * p.PR;
+    const int nh = g.H - h0 < p.PR ? g.H - h0 : p.PR;
+    const int i_first = (int)g.divDH.div((unsigned)h0) - (TH - 1);
+    const int per_plane = p.RW * p.CW;
+    const int HoWo = g.Ho * g.Wo;
+
+    // ---- windows -> (target, gradient) pairs ------------------------------------------------
+    const int E = np * per_plane;
+    for (int e0 = tid; e0 < E; e0 += 4 * nthr) {
+        float vy[4], vx[4], vg[4];
+        int wi[4], wj[4];
+        bool ok[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int idx = e0 + u * nthr;
+            unsigned pl, rem, rr, cc;
+            p.divEnt.divmod((unsigned)(idx < E ? idx : 0), pl, rem);
+            p.divCW.divmod(rem, rr, cc);
+            wi[u] = i_first + (int)rr;
+            wj[u] = (int)cc - (TW - 1);
+            ok[u] = idx < E && wi[u] >= 0 && wi[u] < g.Ho && wj[u] >= 0 && wj[u] < g.Wo;
+            const long o = (long)(plane0 + pl) * HoWo + (ok[u] ? wi[u] * g.Wo + wj[u] : 0);
+            vy[u] = indy[o];
+            vx[u] = indx[o];
+            vg[u] = gout[o];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int idx = e0 + u * nthr;
+            if (idx < E) {
+                const int t = (wi[u] * g.dH + (int)vy[u] - 1) * g.W + wj[u] * g.dW + (int)vx[u] - 1;
+                ent[idx] = make_int2(ok[u] ? t : -1, __float_as_int(vg[u]));
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- pixels ----------------------------------------------------------------------------------
+    const int P = nh * g.W;
+    const int total = np * P;
+    for (int q = tid; q < total; q += nthr) {
+        unsigned pl = 0, r = (unsigned)q, hh, w;
+        if (p.G > 1) p.divPix.divmod(r, pl, r);  // grouped planes are whole: P == H*W
+        g.divW.divmod(r, hh, w);
+        const int h = h0 + (int)hh;
+        const int i_hi = (int)g.divDH.div((unsigned)h), j_hi = (int)g.divDW.div(w);
+        const int2 *e = ent + (int)pl * per_plane + (i_hi - i_first) * p.CW + j_hi + (TW - 1);
+        const int pix = h * g.W + (int)w;
+        float acc = 0.0f;
+#pragma unroll
+        for (int a = TH - 1; a >= 0; --a)
+#pragma unroll
+            for (int b = TW - 1; b >= 0; --b) {
+                const int2 c = e[-a * p.CW - b];
+                acc += c.x == pix ? __int_as_float(c.y) : 0.0f;
+            }
+        gin[(long)(plane0 + pl) * g.H * g.W + pix] = acc;
+    }
+}
+
+// The most LDS the tile kernel may ask for.
+constexpr long kPoolBwdLdsBytes = 32 * 1024;
+
+// Strip shape of the tile kernel; false when one pixel row's windows do not fit in LDS.
+bool plan_pool_bwd(const PoolGeom &g, long planes, int TH, int TW, PoolBwdPlan &p) {
+    const int right = (g.W - 1) / g.dW - (g.Wo - 1);
+    p.CW = g.Wo + (TW - 1) + (right > 0 ? right : 0);
+    auto rows = [&](long PR) { return (PR + g.dH - 1) / g.dH + TH; };
+    auto bytes = [&](long G, long PR) { return G * rows(PR) * (long)p.CW * 8; };
+    if (bytes(1, 1) > kPoolBwdLdsBytes) return false;
+    const long want = 2048;  // pixels per workgroup
+    p.G = 1;
+    if ((long)g.H * g.W <= want / 2 && bytes(1, g.H) <= kPoolBwdLdsBytes) {
+        p.PR = g.H;
+        long G = want / ((long)g.H * g.W);
+        if (G > planes) G = planes;
+        while (G > 1 && bytes(G, p.PR) > kPoolBwdLdsBytes) --G;
+        p.G = (int)(G < 1 ? 1 : G);
+    } else {
+        long PR = want / g.W;
+        if (PR < 1) PR = 1;
+        if (PR > g.H) PR = g.H;
+        while (PR > 1 && bytes(1, PR) > kPoolBwdLdsBytes) --PR;
+        const long tiles = (g.H + PR - 1) / PR;
+        p.PR = (int)((g.H + tiles - 1) / tiles);
+    }
+    p.tiles = (g.H + p.PR - 1) / p.PR;
+    p.RW = (int)rows(p.PR);
+    p.divTiles = FastDiv((uint32_t)p.tiles);
+    p.divEnt = FastDiv((uint32_t)(p.RW * p.CW));
+    p.divCW = FastDiv((uint32_t)p.CW);
+    p.divPix = FastDiv((uint32_t)(g.H * g.W));
+    return true;
+}
+
+// The direct kernel, for windows the tile kernel is not built for.
 // TH x TW = the most windows that can cover one pixel (ceil(kH/dH) x ceil(kW/dW));
 // candidates outside [lo, hi] are read at a clamped address and contribute +0.0f,
 // so the loads of all candidates are in flight together.
@@ -266,10 +392,31 @@ int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int
     g.divHW = FastDiv((uint32_t)(H * W));
     g.divDH = FastDiv((uint32_t)dH);
     g.divDW = FastDiv((uint32_t)dW);
+    const int th = (kH + dH - 1) / dH, tw = (kW + dW - 1) / dW;
+    const double bytes = 4.0 * ((double)total + 3.0 * ototal);
+    PoolBwdPlan plan;
+    // THGPU_POOL_BWD_DIRECT=1 forces the direct kernel (a testing and tuning aid).
+    const char *direct = std::getenv("THGPU_POOL_BWD_DIRECT");
+    if (!(direct && direct[0] == '1') && ((th == 2 && tw == 2) || (th == 1 && tw == 1)) &&
+        plan_pool_bwd(g, planes, th, tw, plan)) {
+        const long blocks = ((planes + plan.G - 1) / plan.G) * plan.tiles;
+        if (blocks < (1L << 31)) {
+            const size_t lds = sizeof(int2) * (size_t)plan.G * plan.RW * plan.CW;
+            {
+                LaunchScope scope("maxpool_bwd", 0.0, bytes);
+                if (th == 2)
+                    hipLaunchKernelGGL((maxpool_bwd_tile_kernel<2, 2>), dim3((unsigned)blocks), dim3(256), lds, s, gout,
+                                       indices, indices + ototal, gin, g, plan, (unsigned)planes);
+                else
+                    hipLaunchKernelGGL((maxpool_bwd_tile_kernel<1, 1>), dim3((unsigned)blocks), dim3(256), lds, s, gout,
+                                       indices, indices + ototal, gin, g, plan, (unsigned)planes);
+            }
+            return check_launch("maxpool_bwd");
+        }
+    }
     {
-        LaunchScope scope("maxpool_bwd", 0.0, 4.0 * ((double)total + 3.0 * ototal));
+        LaunchScope scope("maxpool_bwd", 0.0, bytes);
         const dim3 grid((unsigned)((total + 255) / 256)), block(256);
-        const int th = (kH + dH - 1) / dH, tw = (kW + dW - 1) / dW;
         if (th == 2 && tw == 2)
             hipLaunchKernelGGL((maxpool_bwd_kernel<2, 2>), grid, block, 0, s, gout, indices, indices + ototal, gin, g,
                                (unsigned)total, th, tw);

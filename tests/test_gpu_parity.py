@@ -227,12 +227,24 @@ def test_blas_gemm_integer_exact_beta0_ignores_nan_and_quick_returns(gt):
 
 
 POOLS = [(2, 3, 7, 7, 3, 3, 2, 2), (3, 2, 9, 8, 2, 2, 2, 2), (2, 2, 10, 11, 3, 2, 1, 3), (1, 1, 6, 6, 4, 4, 1, 1),
-         (4, 16, 55, 55, 3, 3, 2, 2), (2, 8, 13, 13, 3, 3, 2, 2), (2, 4, 24, 24, 2, 2, 2, 2)]
+         (4, 16, 55, 55, 3, 3, 2, 2), (2, 8, 13, 13, 3, 3, 2, 2), (2, 4, 24, 24, 2, 2, 2, 2),
+         (2, 3, 11, 12, 2, 2, 3, 3),       # windows smaller than the stride: uncovered pixels
+         (1, 2, 224, 224, 2, 2, 2, 2), (3, 5, 14, 9, 3, 3, 2, 2), (2, 2, 10, 10, 3, 3, 3, 3), (1, 1, 3, 300, 3, 3, 2, 2)]
+
+
+@pytest.fixture(params=[None, "1"], ids=["auto", "direct"])
+def pool_bwd_kernel(request, monkeypatch):
+    """Runs a test with the library's own backward kernel choice, then with the direct kernel forced."""
+    if request.param is None:
+        monkeypatch.delenv("THGPU_POOL_BWD_DIRECT", raising=False)
+    else:
+        monkeypatch.setenv("THGPU_POOL_BWD_DIRECT", request.param)
+    return request.param
 
 
 @pytest.mark.parametrize("cfg", POOLS)
 @pytest.mark.parametrize("ties", [False, True])
-def test_maxpool_fwd_bwd_bit_exact(gt, cfg, ties):
+def test_maxpool_fwd_bwd_bit_exact(gt, cfg, ties, pool_bwd_kernel):
     B, C, H, W, kH, kW, dH, dW = cfg
     rng = rng_for(51)
     x = rng.integers(0, 8, size=(B, C, H, W)).astype(np.float32) if ties else uniform(rng, (B, C, H, W))
@@ -263,7 +275,7 @@ def test_maxpool_reference_known_answers_and_3d_input(gt):
     assert np.array_equal(gi, np.array(cfg["gradInput"], np.float32))
 
 
-def test_maxpool_edge_c_tied_integers_large(gt):
+def test_maxpool_edge_c_tied_integers_large(gt, pool_bwd_kernel):
     # edge sweep (c) at a reduced batch: overlapping 3x3 s2 on 256x27x27 maps of integers 0..7
     rng = rng_for(52)
     x = rng.integers(0, 8, size=(8, 256, 27, 27)).astype(np.float32)
