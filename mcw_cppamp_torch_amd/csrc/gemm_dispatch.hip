@@ -20,8 +20,17 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(const float *__restri
     unsigned idx = blockIdx.x * blockDim.x + threadIdx.x;
     const unsigned total = (unsigned)M * (unsigned)J;
     if (idx >= total) return;
+    // Eight partials are requested before the first is added; the adds stay in split order.
     float sum = 0.0f;
-    for (int s = 0; s < nsplit; ++s) sum += ws[(long)s * total + idx];
+    const float *src = ws + idx;
+    for (int s0 = 0; s0 < nsplit; s0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = s0 + u < nsplit ? src[(long)(s0 + u) * total] : 0.0f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (s0 + u < nsplit) sum += v[u];
+    }
     unsigned i, j;
     divJ.divmod(idx, i, j);
     long coff = j;

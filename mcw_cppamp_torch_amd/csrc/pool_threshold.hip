@@ -314,14 +314,26 @@ __global__ __launch_bounds__(256) void threshold_bwd_scalar(const float *__restr
 // in order.
 __global__ __launch_bounds__(256) void gradbias_partial_kernel(const float *__restrict__ gout,
                                                                float *__restrict__ part, int B, int M, int N,
-                                                               int imgs_per_slice, int nslices) {
+                                                               int imgs_per_slice, int nslices, const FastDiv divN) {
     const int m = blockIdx.x, slice = blockIdx.y;
     const int b0 = slice * imgs_per_slice;
     const int b1 = b0 + imgs_per_slice < B ? b0 + imgs_per_slice : B;
+    // The slice is (b1-b0) rows of N floats, M*N apart; lanes walk it as one
+    // flat array, eight loads in flight each, whatever N is.
+    const unsigned total = (unsigned)(b1 - b0) * (unsigned)N;
+    const float *base = gout + ((long)b0 * M + m) * N;
+    const long row_gap = (long)(M - 1) * N;  // from the end of one row to the start of the next
     float sum = 0.0f;
-    for (int b = b0; b < b1; ++b) {
-        const float *row = gout + ((long)b * M + m) * N;
-        for (int n = threadIdx.x; n < N; n += 256) sum += row[n];
+    for (unsigned f0 = threadIdx.x; f0 < total; f0 += 256 * 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const unsigned f = f0 + 256u * u;
+            const unsigned row = divN.div(f < total ? f : 0);
+            v[u] = f < total ? base[f + row * row_gap] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sum += v[u];
     }
     __shared__ float red[256];
     red[threadIdx.x] = sum;
@@ -469,8 +481,8 @@ int threshold_bwd_launch(const float *in, const float *gout, float *gin, long n,
 int gradbias_launch(const float *gout, float *gbias, long B, int M, long N, float scale) {
     hipStream_t s = stream();
     if (!s) return 1;
-    if (M == 0) return 0;
-    if (B >= (1L << 31) || N >= (1L << 31)) return fail("gradBias: tensor too large");
+    if (M == 0 || N == 0 || B == 0) return 0;  // an empty sum leaves gradBias as it is
+    if (B >= (1L << 31) || N >= (1L << 31) || B * N >= (1L << 32)) return fail("gradBias: tensor too large");
     // About four workgroups per CU in stage 1.
     long nslices = (4L * num_cus() + M - 1) / M;
     if (nslices > B) nslices = B;
@@ -486,7 +498,7 @@ int gradbias_launch(const float *gout, float *gbias, long B, int M, long N, floa
     {
         LaunchScope scope("gradbias", 0.0, 4.0 * B * M * N);
         hipLaunchKernelGGL(gradbias_partial_kernel, dim3((unsigned)M, (unsigned)nslices), dim3(256), 0, s, gout,
-                           part, (int)B, M, (int)N, ips, (int)nslices);
+                           part, (int)B, M, (int)N, ips, (int)nslices, FastDiv((uint32_t)N));
     }
     if (check_launch("gradbias")) return 1;
     {
