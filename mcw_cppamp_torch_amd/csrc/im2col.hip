@@ -383,6 +383,45 @@ __global__ __launch_bounds__(256) void col2im_kernel(const float *__restrict__ c
     im[idx] = acc;
 }
 
+// col2im for unit strides and a window known at compile time.  With unit
+// strides every tap can reach a pixel, and the column entry of tap (kh, kw) for
+// pixel (h, w) sits at a per-tap scalar offset from a per-lane constant:
+//   col[plane][kh*KW + kw][(h+pH-kh)*Wo + (w+pW-kw)]
+//     = plane block + (tap*N - kh*Wo - kw)  +  ((h+pH)*Wo + (w+pW)).
+// All KH*KW loads of a pixel are requested before the first add; the adds run
+// kh ascending, kw ascending, out-of-range taps contributing +0.0f.
+template <int KH, int KW>
+__global__ __launch_bounds__(256) void col2im_unit_kernel(const float *__restrict__ col, float *__restrict__ im,
+                                                          const ConvGeom g, unsigned total) {
+    const unsigned q0 = blockIdx.x * 256u;  // scalar
+    const unsigned q = q0 + threadIdx.x;
+    const unsigned plane_first = g.divHW.div(q0);
+    unsigned plane, pix, h, w;
+    g.divHW.divmod(q < total ? q : total - 1, plane, pix);
+    g.divW.divmod(pix, h, w);
+    const int hp = (int)h + g.pH, wp = (int)w + g.pW;
+    const long plane_floats = (long)(KH * KW) * g.N;
+    const unsigned voff = (unsigned)(((long)(plane - plane_first) * plane_floats + (long)hp * g.Wo + wp) * 4);
+    const char *base = reinterpret_cast<const char *>(col + (long)plane_first * plane_floats);
+    float v[KH][KW];
+#pragma unroll
+    for (int kh = 0; kh < KH; ++kh) {
+        const bool okh = (unsigned)(hp - kh) < (unsigned)g.Ho;
+#pragma unroll
+        for (int kw = 0; kw < KW; ++kw) {
+            const bool ok = okh && (unsigned)(wp - kw) < (unsigned)g.Wo;
+            const long tap_off = ((long)(kh * KW + kw) * g.N - (long)kh * g.Wo - kw) * 4;  // scalar, never negative
+            v[kh][kw] = ok ? *reinterpret_cast<const float *>(base + tap_off + voff) : 0.0f;
+        }
+    }
+    float acc = 0.0f;
+#pragma unroll
+    for (int kh = 0; kh < KH; ++kh)
+#pragma unroll
+        for (int kw = 0; kw < KW; ++kw) acc += v[kh][kw];
+    if (q < total) im[q] = acc;
+}
+
 int make_geom(ConvGeom &g, long B, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW) {
     if (B < 0 || C <= 0 || H <= 0 || W <= 0 || kH <= 0 || kW <= 0 || sH <= 0 || sW <= 0 || pH < 0 || pW < 0)
         return fail("im2col/col2im: invalid geometry");
@@ -496,6 +535,23 @@ int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW,
     const long blocks = (total + 255) / 256;
     if (blocks >= (1L << 31)) return fail("col2im: image batch too large for one launch");
     const double bytes = 4.0 * ((double)total + (double)B * C * kH * kW * g.Ho * g.Wo);
+    // Lane offsets of the unit-stride kernel are 32-bit: the planes one workgroup can touch must span < 4 GiB.
+    const long span_planes = 256 / ((long)H * W) + 2;
+    // THGPU_COL2IM_GENERIC=1 forces the general kernel (a testing and tuning aid).
+    const char *generic = std::getenv("THGPU_COL2IM_GENERIC");
+    if (!(generic && generic[0] == '1') && sH == 1 && sW == 1 && kH == kW && (kH == 3 || kH == 5) &&
+        span_planes * kH * kW * g.N * 4 < (1L << 32) && total < (1L << 32)) {
+        {
+            LaunchScope scope("col2im", 0.0, bytes);
+            if (kH == 3)
+                hipLaunchKernelGGL((col2im_unit_kernel<3, 3>), dim3((unsigned)blocks), dim3(256), 0, s, col, im, g,
+                                   (unsigned)total);
+            else
+                hipLaunchKernelGGL((col2im_unit_kernel<5, 5>), dim3((unsigned)blocks), dim3(256), 0, s, col, im, g,
+                                   (unsigned)total);
+        }
+        return check_launch("col2im");
+    }
     {
         LaunchScope scope("col2im", 0.0, bytes);
         hipLaunchKernelGGL(col2im_kernel, dim3((unsigned)blocks), dim3(256), 0, s, col, im, g, total,

@@ -51,6 +51,10 @@ GEOMS = [
     (2, 3, 128, 96, 3, 7, 1, 3, 1, 2),
     (4, 16, 27, 27, 5, 5, 2, 2, 1, 1),
     (3, 8, 13, 13, 3, 3, 1, 1, 1, 1),
+    (2, 5, 56, 56, 3, 3, 1, 1, 1, 1),
+    (3, 2, 24, 28, 5, 5, 0, 0, 1, 1),
+    (300, 2, 3, 4, 3, 3, 2, 2, 1, 1),       # planes much smaller than a workgroup
+    (2, 3, 9, 7, 5, 5, 4, 4, 1, 1),         # padding as large as the window allows
 ]
 
 
@@ -92,8 +96,18 @@ def test_im2col_unaligned_destination(gt, im2col_kernel):
     assert np.array_equal(bits(host[1:]), bits(ref.ravel()))
 
 
+@pytest.fixture(params=[None, "1"], ids=["auto", "generic"])
+def col2im_kernel(request, monkeypatch):
+    """Runs a test with the library's own col2im kernel choice, then with the general kernel forced."""
+    if request.param is None:
+        monkeypatch.delenv("THGPU_COL2IM_GENERIC", raising=False)
+    else:
+        monkeypatch.setenv("THGPU_COL2IM_GENERIC", request.param)
+    return request.param
+
+
 @pytest.mark.parametrize("geo", GEOMS)
-def test_col2im_bit_exact(gt, geo):
+def test_col2im_bit_exact(gt, geo, col2im_kernel):
     B, C, H, W, kH, kW, pH, pW, sH, sW = geo
     Ho, Wo = oracle.conv_out_size(H, W, kH, kW, pH, pW, sH, sW)
     col = uniform(rng_for(23), (B, C * kH * kW, Ho * Wo))
