@@ -5,32 +5,34 @@
 // n = ho*Wo + wo; flat, the buffer is [B*C planes][kH*kW taps][Ho][Wo].
 //
 // im2col is store-bound (K*N floats out for C*H*W in) and, at four cycles per
-// wavefront instruction, easily instruction-bound as well, so the kernel is
-// organised to spend about three instructions per 64 floats written.  A
-// workgroup takes a strip of output rows of one plane (or several whole planes
-// when they are small) and copies the input rows that strip needs into LDS
-// once, zero padding included, so nothing downstream checks a bound.  Then a
-// lane owns a few output positions n, keeps their LDS addresses in registers,
-// and walks the taps: per tap and position one LDS read at a scalar offset and
-// one 4-byte store whose address is a scalar row base plus the lane's fixed
-// offset -- the wavefront writes 256 consecutive bytes of one column row.  HBM
-// sees the image once (plus the halo rows between strips) and the columns
-// once, for any stride, and no store depends on the alignment of a row.
-// Geometries whose strip of input rows does not fit in LDS (rows of many
-// thousands of pixels) fall back to two direct kernels: a flat one for unit
-// horizontal stride (a lane owns four consecutive floats of the column buffer)
-// and one that reads four taps at a time for strided convolutions.
+// wavefront instruction, easily instruction-bound as well, so every kernel
+// spends only a few instructions per 64 floats written and builds addresses
+// as a scalar (per tap) part plus a per-lane constant:
+//   * unit strides, 3x3 (or 5x5) window known at compile time: a lane owns one
+//     output position, requests its KH*KW input pixels at once and writes one
+//     float into each column row (the wavefront: 256 consecutive bytes a row);
+//   * other unit-stride layers: a workgroup copies the input rows of a strip
+//     of output rows (or of several small planes) into LDS once, zero padding
+//     included, and its lanes walk the taps with one LDS read and one store
+//     per position and tap;
+//   * strided layers, and rows too long for LDS: two direct kernels, a flat one
+//     for unit horizontal stride (a lane owns four consecutive floats of the
+//     column buffer) and one that reads four taps at a time.
+// HBM sees the image once (plus halo rows between strips; neighbouring lanes
+// share input through the caches) and the columns once.
 //
 // col2im is a gather with no atomics: one lane per image pixel adds the
 // column entries that cover it, kh ascending then kw ascending from +0.0f --
 // the float addition order of nn_(unfolded_acc) (mcw_nn/generic/
 // SpatialConvolutionMM.c:6-50), which makes the result bit-identical to the
 // CPU module's.  Lanes run along w, so for a fixed tap the reads are
-// consecutive in wo.  Candidate taps are visited in groups of four with
-// clamped addresses and the invalid ones contribute +0.0f (which leaves a
-// float sum unchanged), so the loads of a group are in flight together.
+// consecutive in wo.  Taps that do not reach a pixel contribute +0.0f (which
+// leaves a float sum unchanged), so no add depends on a branch.  Unit-stride
+// 3x3 and 5x5 layers have all their taps in flight per pixel; the general
+// kernel visits candidate taps in groups of four with clamped addresses.
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 
 #include "common.h"
 
@@ -383,6 +385,46 @@ __global__ __launch_bounds__(256) void col2im_kernel(const float *__restrict__ c
     im[idx] = acc;
 }
 
+// im2col for unit strides and a window known at compile time: the mirror of
+// col2im_unit_kernel below.  A lane owns one output position (plane, ho, wo),
+// requests its KH*KW input pixels (neighbouring lanes share them through the
+// vector cache), then writes one float to each of the KH*KW column rows at a
+// per-tap scalar offset from a per-lane constant.
+template <int KH, int KW>
+__global__ __launch_bounds__(256) void im2col_unit_kernel(const float *__restrict__ im, float *__restrict__ col,
+                                                          const ConvGeom g, unsigned total) {
+    const unsigned q0 = blockIdx.x * 256u;  // scalar
+    const unsigned q = q0 + threadIdx.x;
+    const unsigned plane_first = g.divN.div(q0);
+    unsigned plane, n, ho, wo;
+    g.divN.divmod(q < total ? q : total - 1, plane, n);
+    g.divWo.divmod(n, ho, wo);
+    const int hi = (int)ho - g.pH, wi = (int)wo - g.pW;  // input pixel of tap (0, 0)
+    const long in_plane = (long)g.H * g.W, out_plane = (long)(KH * KW) * g.N;
+    const char *src = reinterpret_cast<const char *>(im + (long)plane_first * in_plane);
+    char *dst = reinterpret_cast<char *>(col + (long)plane_first * out_plane);
+    // 32-bit lane offsets; the input one may start before the plane (padding) but is only used where valid
+    const long in_lane = (long)(plane - plane_first) * in_plane + (long)hi * g.W + wi;
+    const unsigned out_off = (unsigned)(((long)(plane - plane_first) * out_plane + n) * 4);
+    float v[KH][KW];
+#pragma unroll
+    for (int kh = 0; kh < KH; ++kh) {
+        const bool okh = (unsigned)(hi + kh) < (unsigned)g.H;
+#pragma unroll
+        for (int kw = 0; kw < KW; ++kw) {
+            const bool ok = okh && (unsigned)(wi + kw) < (unsigned)g.W;
+            v[kh][kw] = ok ? *reinterpret_cast<const float *>(src + (in_lane + (long)kh * g.W + kw) * 4) : 0.0f;
+        }
+    }
+    if (q < total) {
+#pragma unroll
+        for (int kh = 0; kh < KH; ++kh)
+#pragma unroll
+            for (int kw = 0; kw < KW; ++kw)
+                *reinterpret_cast<float *>(dst + (long)(kh * KW + kw) * g.N * 4 + out_off) = v[kh][kw];
+    }
+}
+
 // col2im for unit strides and a window known at compile time.  With unit
 // strides every tap can reach a pixel, and the column entry of tap (kh, kw) for
 // pixel (h, w) sits at a per-tap scalar offset from a per-lane constant:
@@ -459,10 +501,32 @@ int im2col_launch(const float *im, long B, int C, int H, int W, int kH, int kW, 
     const double bytes = 4.0 * ((double)B * C * H * W + (double)total);
     StripPlan plan;
     const long planes = B * (long)C;
-    // THGPU_IM2COL_DIRECT=1 forces the direct kernels, =0 the LDS-staged one (testing and tuning aids).
-    const char *direct = std::getenv("THGPU_IM2COL_DIRECT");
-    // Strided convolutions (few, large first layers) measured faster on the direct kernel.
-    if (!(direct && direct[0] == '1') && (sW == 1 || (direct && direct[0] == '0')) && plan_strips(g, planes, plan)) {
+    // Kernel choice.  Measured on gfx950: 3x3 unit-stride layers run fastest on the
+    // per-position kernel, other unit-stride layers on the LDS-staged strips
+    // (many column rows per workgroup favour its few, long stores), strided
+    // first layers on the direct kernel.  THGPU_IM2COL_KERNEL=unit|strip|direct
+    // forces one where it applies (a testing and tuning aid).
+    const char *force = std::getenv("THGPU_IM2COL_KERNEL");
+    const bool f_unit = force && !std::strcmp(force, "unit"), f_strip = force && !std::strcmp(force, "strip"),
+               f_direct = force && !std::strcmp(force, "direct");
+    const long span_out = 256 / (long)g.N + 2;  // planes one workgroup of the per-position kernel can touch
+    const bool unit_ok = sH == 1 && sW == 1 && kH == kW && (kH == 3 || kH == 5) && planes * g.N < (1L << 32) &&
+                         span_out * kH * kW * g.N * 4 < (1L << 32) && span_out * H * W * 4 < (1L << 31);
+    if (unit_ok && !f_strip && !f_direct && (kH == 3 || f_unit)) {
+        const long positions = planes * g.N;
+        const unsigned blocks = (unsigned)((positions + 255) / 256);
+        {
+            LaunchScope scope("im2col", 0.0, bytes);
+            if (kH == 3)
+                hipLaunchKernelGGL((im2col_unit_kernel<3, 3>), dim3(blocks), dim3(256), 0, s, im, col, g,
+                                   (unsigned)positions);
+            else
+                hipLaunchKernelGGL((im2col_unit_kernel<5, 5>), dim3(blocks), dim3(256), 0, s, im, col, g,
+                                   (unsigned)positions);
+        }
+        return check_launch("im2col");
+    }
+    if (!f_direct && (sW == 1 || f_strip) && plan_strips(g, planes, plan)) {
         const long groups = (planes + plan.G - 1) / plan.G;
         const long blocks = groups * plan.tiles;
         if (blocks < (1L << 31) && planes < (1L << 31)) {

@@ -58,13 +58,14 @@ GEOMS = [
 ]
 
 
-@pytest.fixture(params=[None, "0", "1"], ids=["auto", "lds_staged", "direct"])
+@pytest.fixture(params=[None, "unit", "strip", "direct"])
 def im2col_kernel(request, monkeypatch):
-    """Runs a test with the library's own kernel choice, then with each im2col kernel forced."""
+    """Runs a test with the library's own kernel choice, then with each im2col kernel forced
+    (a forced kernel that does not apply to a geometry falls through to the next)."""
     if request.param is None:
-        monkeypatch.delenv("THGPU_IM2COL_DIRECT", raising=False)
+        monkeypatch.delenv("THGPU_IM2COL_KERNEL", raising=False)
     else:
-        monkeypatch.setenv("THGPU_IM2COL_DIRECT", request.param)
+        monkeypatch.setenv("THGPU_IM2COL_KERNEL", request.param)
     return request.param
 
 
