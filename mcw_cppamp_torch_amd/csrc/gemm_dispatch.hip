@@ -50,16 +50,19 @@ struct TileCfg {
     const char *name;
     int bm, bn;
     int resident;  // workgroups that fit a CU at once (registers / LDS)
-    double eff;    // fraction of the MFMA rate the inner loop sustains with a full CU
+    // Fraction of the MFMA rate the inner loop sustains with a full CU, by operand layout (measured
+    // on the AlexNet layer shapes): [0] A along r, B along j (forward); [1] both along their free
+    // index (gradInput); [2] both along r (gradWeight); [3] A along i, B along r.
+    double eff[4];
     int (*launch)(const GemmArgs &, int, int, bool, hipStream_t);
 };
 
 const TileCfg kCfgs[] = {
-    {"128x128", 128, 128, 4, 0.90, gemm_fast_128x128},
-    {"64x256", 64, 256, 3, 0.88, gemm_fast_64x256},
-    {"128x256", 128, 256, 2, 0.86, gemm_fast_128x256},
-    {"256x128", 256, 128, 2, 0.86, gemm_fast_256x128},
-    {"64x64", 64, 64, 4, 0.74, gemm_fast_64x64},
+    {"128x128", 128, 128, 4, {0.90, 0.90, 0.86, 0.86}, gemm_fast_128x128},
+    {"64x256", 64, 256, 3, {0.76, 0.74, 0.90, 0.74}, gemm_fast_64x256},
+    {"128x256", 128, 256, 2, {0.85, 0.87, 0.90, 0.85}, gemm_fast_128x256},
+    {"256x128", 256, 128, 2, {0.90, 0.75, 0.90, 0.75}, gemm_fast_256x128},
+    {"64x64", 64, 64, 4, {0.68, 0.60, 0.74, 0.60}, gemm_fast_64x64},
 };
 
 inline long cdiv(long a, long b) { return (a + b - 1) / b; }
@@ -69,12 +72,12 @@ inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 // hides less of their latencies (kOcc); workgroups beyond what fits at once
 // run in further rounds; every round pays a prologue/epilogue; a split adds
 // the traffic of writing and re-reading the partial sums.
-double model_cycles(const TileCfg &c, long M, long J, long steps_total, int nsplit, int cus) {
+double model_cycles(const TileCfg &c, int layout, long M, long J, long steps_total, int nsplit, int cus) {
     static const double kOcc[5] = {0.0, 0.70, 0.88, 0.96, 1.0};
     const long tiles = cdiv(M, c.bm) * cdiv(J, c.bn);
     const long wgs = tiles * nsplit;
     const long steps = cdiv(steps_total, nsplit);
-    const double per_step = 2.0 * c.bm * c.bn * GEMM_BK / 256.0 / c.eff;
+    const double per_step = 2.0 * c.bm * c.bn * GEMM_BK / 256.0 / c.eff[layout];
     const double ovh = 3000.0 + 6.0 * c.bm * c.bn / 64.0;
     const long slots = (long)cus * c.resident;
     const long full = wgs / slots, rest = wgs - full * slots;
@@ -146,6 +149,7 @@ int gemm_launch(const GemmProblem &p) {
         return offA < (1L << 30) && offB < (1L << 30) && offC < (1L << 30);
     };
     const bool fast_ok = p.R == 0 || p.R >= GEMM_BK;
+    const int layout = p.a_rc ? (p.b_rc ? 2 : 0) : (p.b_rc ? 3 : 1);
     for (const TileCfg &c : kCfgs) {
         if (!fast_ok || p.M < c.bm || p.J < c.bn || !offsets_fit(c.bm, c.bn)) continue;
         if (force && std::strcmp(force, c.name) != 0) continue;
@@ -156,7 +160,7 @@ int gemm_launch(const GemmProblem &p) {
             if (tiles * ns > 8L * cus * c.resident && ns > 1 && fsplit <= 0) break;
             const int sps = (int)cdiv(g.steps_total, ns);
             if ((int)cdiv(g.steps_total, sps) != ns) continue;  // would leave an empty split
-            const double t = model_cycles(c, p.M, p.J, g.steps_total, ns, cus);
+            const double t = model_cycles(c, layout, p.M, p.J, g.steps_total, ns, cus);
             if (!best || t < best_t) {
                 best = &c;
                 best_split = ns;
