@@ -29,6 +29,11 @@ sys.path.insert(0, ROOT)
 METRIC = "images/sec fwd+bwd, AlexNet-style conv stack b128 fp32; GEMM % fp32 MFMA peak"
 PEAK_MFMA_F32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per GEMM launch (average over the 15 launches of a step), from two rocprofv3 --pmc runs of this
+# script (FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0, the factors a plain copy kernel of known size gives);
+# the summary with the commands is profiles/hbm_traffic_alexnet_b128_pmc.txt.  Counters cannot be read
+# from inside the timed process, so the figure is carried here for the configuration it was measured on.
+MEASURED_GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("alexnet", 128): 6.061e8}
 
 
 def cpu_baseline(workload, sample_batch, budget_s=20.0):
@@ -182,9 +187,10 @@ def main():
             kernels[kname] = ent
         if g_ms > 0:
             roofline = {
-                "bound": "mfma", "kernel": "gemm_kernel<...> (all conv GEMM launches of a step)",
+                "bound": "mfma", "kernel": "gemm_fast_kernel<...> (all conv GEMM launches of a step)",
                 "achieved": round(g_fl / g_ms / 1e9, 2), "peak": PEAK_MFMA_F32_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(g_fl / g_ms / 1e9 / PEAK_MFMA_F32_TFLOPS, 4), "traffic": None,
+                "frac": round(g_fl / g_ms / 1e9 / PEAK_MFMA_F32_TFLOPS, 4),
+                "traffic": MEASURED_GEMM_TRAFFIC_BYTES_PER_LAUNCH.get((name, B)),
                 "launches_per_step": g_calls / args.steps, "ms_per_step": round(g_ms, 4),
                 "flops_per_step": g_fl,
             }
