@@ -28,8 +28,10 @@
 // CPU module's.  Lanes run along w, so for a fixed tap the reads are
 // consecutive in wo.  Taps that do not reach a pixel contribute +0.0f (which
 // leaves a float sum unchanged), so no add depends on a branch.  Unit-stride
-// 3x3 and 5x5 layers have all their taps in flight per pixel; the general
-// kernel visits candidate taps in groups of four with clamped addresses.
+// 3x3 and 5x5 layers have all their taps in flight per pixel; strided layers
+// with wide rows walk the pixels by residue class of (h+pH, w+pW) modulo the
+// strides, which makes every read a long contiguous run; the general kernel
+// visits candidate taps in groups of four with clamped addresses.
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -43,7 +45,7 @@ namespace {
 struct ConvGeom {
     int C, H, W, kH, kW, pH, pW, sH, sW, Ho, Wo, N;
     FastDiv divN, divKH, divWo, divTaps, divKW;  // im2col decomposition
-    FastDiv divW, divHW, divSH, divSW;  // col2im decomposition
+    FastDiv divW, divHW, divSH, divSW, divH;  // col2im decomposition
 };
 
 // Four floats at a 4-byte aligned address (the hardware handles the
@@ -464,6 +466,70 @@ __global__ __launch_bounds__(256) void col2im_unit_kernel(const float *__restric
     if (q < total) im[q] = acc;
 }
 
+// col2im for strided convolutions with wide rows.  Write (h+pH, w+pW) =
+// (qh*sH + rh, qw*sW + rw).  For one residue pair (rh, rw) the taps that reach
+// a pixel are kh = rh + th*sH, kw = rw + tw*sW -- scalars -- and the column
+// entry of tap (th, tw) for quotient pair (qh, qw) is
+//   col[plane][kh*kW + kw][(qh-th)*Wo + (qw-tw)]
+//     = scalar(plane, kh, kw, th, tw) + (qh*Wo + qw),
+// a per-lane constant again, and lanes with consecutive (qh, qw) read
+// consecutive column entries: the reads, nearly all of this kernel's traffic,
+// are long contiguous runs.  A workgroup owns R quotient rows of one plane
+// (R*sH image rows), one lane per (qh, qw) pair, walks the sH*sW residue pairs
+// with all TH*TW taps of a pixel in flight (kh ascending, kw ascending, an
+// unreachable tap contributing +0.0f), and collects the sums in an LDS copy of
+// its image rows so that the image is written contiguously as well.
+template <int TH, int TW>
+__global__ __launch_bounds__(256) void col2im_strided_kernel(const float *__restrict__ col, float *__restrict__ im,
+                                                             const ConvGeom g, int R, int Qw, int qtiles,
+                                                             const FastDiv divQw, const FastDiv divTiles) {
+    extern __shared__ float rows[];  // [R*sH][W]
+    unsigned plane, qt;
+    divTiles.divmod(blockIdx.x, plane, qt);
+    const int qh0 = (int)qt * R;
+    const int h_base = qh0 * g.sH - g.pH;  // image row of the tile's first LDS row (may be negative)
+    const float *src = col + (long)plane * (g.kH * g.kW) * g.N;
+    for (int e = threadIdx.x; e < R * Qw; e += blockDim.x) {
+        unsigned ql, qw;
+        divQw.divmod((unsigned)e, ql, qw);
+        const int qh = qh0 + (int)ql;
+        const int lane_off = qh * g.Wo + (int)qw;
+        for (int rh = 0; rh < g.sH; ++rh) {
+            const int h = qh * g.sH + rh - g.pH;
+            for (int rw = 0; rw < g.sW; ++rw) {
+                const int w = (int)qw * g.sW + rw - g.pW;
+                float v[TH][TW];
+#pragma unroll
+                for (int th = 0; th < TH; ++th) {
+                    const int kh = rh + th * g.sH;
+                    const bool okh = kh < g.kH && qh - th >= 0 && qh - th < g.Ho;
+#pragma unroll
+                    for (int tw = 0; tw < TW; ++tw) {
+                        const int kw = rw + tw * g.sW;
+                        const bool tap = kh < g.kH && kw < g.kW;  // scalar
+                        const long tap_off = tap ? (long)(kh * g.kW + kw) * g.N - (long)th * g.Wo - tw : 0L;  // scalar
+                        const bool ok = tap && okh && (int)qw - tw >= 0 && (int)qw - tw < g.Wo;
+                        v[th][tw] = ok ? src[tap_off + lane_off] : 0.0f;
+                    }
+                }
+                float acc = 0.0f;
+#pragma unroll
+                for (int th = 0; th < TH; ++th)
+#pragma unroll
+                    for (int tw = 0; tw < TW; ++tw) acc += v[th][tw];
+                if (h >= 0 && h < g.H && w >= 0 && w < g.W) rows[(h - h_base) * g.W + w] = acc;
+            }
+        }
+    }
+    __syncthreads();
+    // The tile's image rows [max(h_base, 0), min(h_base + R*sH, H)) are contiguous in the image.
+    const int h_lo = h_base < 0 ? 0 : h_base;
+    const int h_hi = h_base + R * g.sH < g.H ? h_base + R * g.sH : g.H;
+    float *dst = im + ((long)plane * g.H + h_lo) * g.W;
+    const float *from = rows + (h_lo - h_base) * g.W;
+    for (int i = threadIdx.x; i < (h_hi - h_lo) * g.W; i += blockDim.x) dst[i] = from[i];
+}
+
 int make_geom(ConvGeom &g, long B, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW) {
     if (B < 0 || C <= 0 || H <= 0 || W <= 0 || kH <= 0 || kW <= 0 || sH <= 0 || sW <= 0 || pH < 0 || pW < 0)
         return fail("im2col/col2im: invalid geometry");
@@ -482,6 +548,7 @@ int make_geom(ConvGeom &g, long B, int C, int H, int W, int kH, int kW, int pH, 
     g.divHW = FastDiv((uint32_t)(H * W));
     g.divSH = FastDiv((uint32_t)sH);
     g.divSW = FastDiv((uint32_t)sW);
+    g.divH = FastDiv((uint32_t)H);
     if ((long)g.Ho * g.Wo >= (1L << 31) || (long)H * W >= (1L << 31) || B * C * (long)kH * kW >= (1L << 31) ||
         (long)kH * kW * g.Ho * g.Wo >= (1L << 31))
         return fail("im2col/col2im: plane or row count exceeds 32-bit indexing");
@@ -615,6 +682,33 @@ int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW,
                                    (unsigned)total);
         }
         return check_launch("col2im");
+    }
+    const int th = (kH + sH - 1) / sH, tw = (kW + sW - 1) / sW;
+    const int Qh = (H - 1 + pH) / sH + 1, Qw = (W - 1 + pW) / sW + 1;  // quotient ranges of (h+pH)/sH, (w+pW)/sW
+    if (!(generic && generic[0] == '1') && (sW > 1 || sH > 1) && W >= 64 && th <= 3 && tw <= 3) {
+        // R quotient rows per workgroup: about 256 (qh, qw) pairs, image rows within the LDS budget
+        int R = 256 / Qw;
+        if (const char *e = std::getenv("THGPU_COL2IM_R")) R = atoi(e);
+        if (R < 1) R = 1;
+        if (R > Qh) R = Qh;
+        while (R > 1 && (long)R * sH * W * 4 > 48 * 1024) --R;
+        const int qtiles = (Qh + R - 1) / R;
+        const long wgs = B * (long)C * qtiles;
+        if ((long)R * sH * W * 4 <= 48 * 1024 && wgs < (1L << 31)) {
+            const size_t lds = sizeof(float) * (size_t)R * sH * W;
+            const int lanes = (R * Qw + 63) / 64 * 64;
+            const dim3 grid((unsigned)wgs), block(lanes < 256 ? lanes : 256);
+            {
+                LaunchScope scope("col2im", 0.0, bytes);
+                if (th == 3 || tw == 3)
+                    hipLaunchKernelGGL((col2im_strided_kernel<3, 3>), grid, block, lds, s, col, im, g, R, Qw, qtiles,
+                                       FastDiv((uint32_t)Qw), FastDiv((uint32_t)qtiles));
+                else
+                    hipLaunchKernelGGL((col2im_strided_kernel<2, 2>), grid, block, lds, s, col, im, g, R, Qw, qtiles,
+                                       FastDiv((uint32_t)Qw), FastDiv((uint32_t)qtiles));
+            }
+            return check_launch("col2im");
+        }
     }
     {
         LaunchScope scope("col2im", 0.0, bytes);

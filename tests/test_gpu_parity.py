@@ -55,6 +55,9 @@ GEOMS = [
     (3, 2, 24, 28, 5, 5, 0, 0, 1, 1),
     (300, 2, 3, 4, 3, 3, 2, 2, 1, 1),       # planes much smaller than a workgroup
     (2, 3, 9, 7, 5, 5, 4, 4, 1, 1),         # padding as large as the window allows
+    (2, 3, 224, 224, 11, 11, 2, 2, 4, 4),   # first layer of the AlexNet-style stack
+    (1, 2, 70, 90, 5, 7, 2, 3, 2, 3),
+    (2, 2, 65, 131, 4, 6, 0, 5, 3, 2),
 ]
 
 
