@@ -266,6 +266,24 @@ void THLongTensor_copyGPU(THLongTensor *self, THGPUTensor *src);
 void THFloatTensor_copyGPU(THFloatTensor *self, THGPUTensor *src);
 void THDoubleTensor_copyGPU(THDoubleTensor *self, THGPUTensor *src);
 
+/* ---- tensor math on the GEMM (the classifier layers after a conv stack) ------ */
+
+/* self = src + value / src * value / src / value, self resized to src
+ * (gputorch/lib/THC/THCTensorMath.cpp:67-101). */
+void THGPUTensor_add(THGPUTensor *self, THGPUTensor *src, float value);
+void THGPUTensor_mul(THGPUTensor *self, THGPUTensor *src, float value);
+void THGPUTensor_div(THGPUTensor *self, THGPUTensor *src, float value);
+/* self = src1 + value * src2 (THCTensorMath.cpp:103-131). */
+void THGPUTensor_cadd(THGPUTensor *self, THGPUTensor *src1, float value, THGPUTensor *src2);
+/* self = beta*t + alpha * mat*vec, mat1*mat2, vec1 (x) vec2; self is resized to t and
+ * takes its values when they differ; views contiguous along either dimension are used
+ * in place (THCTensorMath.cpp:624-829; CPU twin TH/generic/THTensorMath.c:458-620). */
+void THGPUTensor_addmv(THGPUTensor *self, float beta, THGPUTensor *t, float alpha, THGPUTensor *mat, THGPUTensor *vec);
+void THGPUTensor_addmm(THGPUTensor *self, float beta, THGPUTensor *t, float alpha, THGPUTensor *mat1,
+                       THGPUTensor *mat2);
+void THGPUTensor_addr(THGPUTensor *self, float beta, THGPUTensor *t, float alpha, THGPUTensor *vec1,
+                      THGPUTensor *vec2);
+
 /* ---- BLAS ------------------------------------------------------------------ */
 
 /* Column-major C = beta*C + alpha*op(A)*op(B) on DEVICE pointers: the generic

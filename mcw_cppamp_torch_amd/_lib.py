@@ -154,6 +154,13 @@ _SIGNATURES = {
     "THGPUTensor_copy": (None, [TensorP, TensorP]),
     "THGPUTensor_copyGPU": (None, [TensorP, TensorP]),
     # blas
+    "THGPUTensor_add": (None, [TensorP, TensorP, c_float]),
+    "THGPUTensor_mul": (None, [TensorP, TensorP, c_float]),
+    "THGPUTensor_div": (None, [TensorP, TensorP, c_float]),
+    "THGPUTensor_cadd": (None, [TensorP, TensorP, c_float, TensorP]),
+    "THGPUTensor_addmv": (None, [TensorP, c_float, TensorP, c_float, TensorP, TensorP]),
+    "THGPUTensor_addmm": (None, [TensorP, c_float, TensorP, c_float, TensorP, TensorP]),
+    "THGPUTensor_addr": (None, [TensorP, c_float, TensorP, c_float, TensorP, TensorP]),
     "THGPUBlas_gemm": (None, [c_char, c_char, c_long, c_long, c_long, c_float, f32p, c_long, f32p, c_long,
                               c_float, f32p, c_long]),
     # flat operators

@@ -1,0 +1,199 @@
+// THGPUTensor BLAS-level math on the MFMA GEMM: addmm, addmv, addr, and the
+// scalar/axpy elementwise operations nn.Linear is written with
+// (mcw_nn/Linear.lua:34-101).  The view handling follows the reference
+// dispatcher (gputorch/lib/THC/THCTensorMath.cpp:624-829, the same logic as
+// TH/generic/THTensorMath.c:458-561): a result or operand that is contiguous
+// along either of its two dimensions is used in place through the transpose
+// flags of THGPUBlas_gemm, anything else goes through a dense copy.
+#include "common.h"
+
+using namespace thgpu;
+
+namespace {
+
+// op 0: out = in + v; 1: out = in * v; 2: out = in / v; 3: out = out + v * in (axpy)
+__global__ __launch_bounds__(256) void scalar_op_kernel(const float *__restrict__ in, float *__restrict__ out, long n,
+                                                        float v, int op) {
+    const long stride = (long)gridDim.x * blockDim.x;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const float x = in[i];
+        // the axpy keeps the two roundings of y[i] += a*x[i] (TH/generic/THBlas.c:96-99): no fused multiply-add
+        out[i] = op == 0 ? x + v : op == 1 ? x * v : op == 2 ? x / v : __fadd_rn(out[i], __fmul_rn(v, x));
+    }
+}
+
+int scalar_op(const float *in, float *out, long n, float v, int op, const char *tag) {
+    hipStream_t s = stream();
+    if (!s) return 1;
+    if (n == 0) return 0;
+    long blocks = (n + 255) / 256;
+    if (blocks > 8L * 4 * num_cus()) blocks = 8L * 4 * num_cus();
+    {
+        LaunchScope scope(tag, 0.0, (op == 3 ? 12.0 : 8.0) * n);
+        hipLaunchKernelGGL(scalar_op_kernel, dim3((unsigned)blocks), dim3(256), 0, s, in, out, n, v, op);
+    }
+    return check_launch(tag);
+}
+
+// self = op(src, value) with the reference's resize / densify / copy-back sequence
+// (THCTensorMath.cpp:67-101).
+void unary_scalar(THGPUTensor *self_, THGPUTensor *src_, float value, int op, const char *tag) {
+    THGPUTensor_resizeAs(self_, src_);
+    THGPUTensor *self = THGPUTensor_newContiguous(self_);
+    THGPUTensor *src = THGPUTensor_newContiguous(src_);
+    if (scalar_op(THGPUTensor_data(src), THGPUTensor_data(self), THGPUTensor_nElement(self), value, op, tag))
+        raise("%s", thgpu_last_error());
+    THGPUTensor_free(src);
+    THGPUTensor_freeCopyTo(self, self_);
+}
+
+}  // namespace
+
+extern "C" {
+
+void THGPUTensor_add(THGPUTensor *self, THGPUTensor *src, float value) { unary_scalar(self, src, value, 0, "tensor_add"); }
+void THGPUTensor_mul(THGPUTensor *self, THGPUTensor *src, float value) { unary_scalar(self, src, value, 1, "tensor_mul"); }
+void THGPUTensor_div(THGPUTensor *self, THGPUTensor *src, float value) { unary_scalar(self, src, value, 2, "tensor_div"); }
+
+void THGPUTensor_cadd(THGPUTensor *self_, THGPUTensor *src1, float value, THGPUTensor *src2) {
+    THGPUTensor_resizeAs(self_, src1);
+    THGPU_ARGCHECK(THGPUTensor_nElement(src1) == THGPUTensor_nElement(src2), 3, "size do not match", );
+    THGPUTensor *self = THGPUTensor_newContiguous(self_);
+    if (self_ != src1) THGPUTensor_copy(self, src1);
+    THGPUTensor *s2 = THGPUTensor_newContiguous(src2);
+    if (scalar_op(THGPUTensor_data(s2), THGPUTensor_data(self), THGPUTensor_nElement(self), value, 3, "tensor_cadd"))
+        raise("%s", thgpu_last_error());
+    THGPUTensor_free(s2);
+    THGPUTensor_freeCopyTo(self, self_);
+}
+
+void THGPUTensor_addmm(THGPUTensor *r_, float beta, THGPUTensor *t, float alpha, THGPUTensor *m1, THGPUTensor *m2) {
+    if (m1->nDimension != 2 || m2->nDimension != 2) {
+        raise("matrix and matrix expected");
+        return;
+    }
+    if (t->nDimension != 2 || t->size[0] != m1->size[0] || t->size[1] != m2->size[1] || m1->size[1] != m2->size[0]) {
+        raise("size mismatch");
+        return;
+    }
+    if (t != r_) {
+        THGPUTensor_resizeAs(r_, t);
+        THGPUTensor_copy(r_, t);
+    }
+    // In column-major terms the result is used as it lies when its first
+    // dimension is contiguous; when its second is, the product is formed
+    // transposed (operands swapped); otherwise through a dense transposed copy.
+    char tr;
+    THGPUTensor *r__;
+    if (r_->stride[0] == 1 && r_->stride[1] != 0) {
+        tr = 'n';
+        r__ = r_;
+    } else if (r_->stride[1] == 1 && r_->stride[0] != 0) {
+        THGPUTensor *swap = m2;
+        m2 = m1;
+        m1 = swap;
+        tr = 't';
+        r__ = r_;
+    } else {
+        tr = 'n';
+        THGPUTensor *dense = THGPUTensor_newWithSize2d(r_->size[1], r_->size[0]);
+        r__ = THGPUTensor_newTranspose(dense, 0, 1);  // shape of r_, first dimension contiguous
+        THGPUTensor_free(dense);
+        THGPUTensor_copy(r__, r_);
+    }
+    const int d0 = tr == 'n' ? 0 : 1, d1 = tr == 'n' ? 1 : 0;
+    char t1, t2;
+    THGPUTensor *m1_, *m2_;
+    if (m1->stride[d0] == 1 && m1->stride[d1] != 0) {
+        t1 = 'n';
+        m1_ = m1;
+    } else if (m1->stride[d1] == 1 && m1->stride[d0] != 0) {
+        t1 = 't';
+        m1_ = m1;
+    } else {
+        t1 = tr == 'n' ? 't' : 'n';
+        m1_ = THGPUTensor_newClone(m1);
+    }
+    if (m2->stride[d0] == 1 && m2->stride[d1] != 0) {
+        t2 = 'n';
+        m2_ = m2;
+    } else if (m2->stride[d1] == 1 && m2->stride[d0] != 0) {
+        t2 = 't';
+        m2_ = m2;
+    } else {
+        t2 = tr == 'n' ? 't' : 'n';
+        m2_ = THGPUTensor_newClone(m2);
+    }
+    const long mm = r__->size[d0], nn = r__->size[d1], kk = m1_->size[d1];
+    THGPUBlas_gemm(t1, t2, mm, nn, kk, alpha, THGPUTensor_data(m1_), t1 == 'n' ? m1_->stride[d1] : m1_->stride[d0],
+                   THGPUTensor_data(m2_), t2 == 'n' ? m2_->stride[d1] : m2_->stride[d0], beta, THGPUTensor_data(r__),
+                   r__->stride[d1]);
+    if (m1_ != m1) THGPUTensor_free(m1_);
+    if (m2_ != m2) THGPUTensor_free(m2_);
+    if (r__ != r_) THGPUTensor_freeCopyTo(r__, r_);
+}
+
+void THGPUTensor_addmv(THGPUTensor *r_, float beta, THGPUTensor *t, float alpha, THGPUTensor *mat, THGPUTensor *vec) {
+    if (mat->nDimension != 2 || vec->nDimension != 1) {
+        raise("matrix and vector expected");
+        return;
+    }
+    if (mat->size[1] != vec->size[0] || t->nDimension != 1 || t->size[0] != mat->size[0]) {
+        raise("size mismatch");
+        return;
+    }
+    if (r_ != t) {
+        THGPUTensor_resizeAs(r_, t);
+        THGPUTensor_copy(r_, t);
+    }
+    // y = beta*y + alpha*op(A)*x as a GEMM with one column; x and y must be dense for that.
+    THGPUTensor *x = THGPUTensor_newContiguous(vec);
+    THGPUTensor *y = THGPUTensor_newContiguous(r_);
+    THGPUTensor *a = mat;
+    char ta;
+    long lda;
+    if (mat->stride[0] == 1 && mat->stride[1] != 0) {
+        ta = 'n';
+        lda = mat->stride[1];
+    } else if (mat->stride[1] == 1 && mat->stride[0] != 0) {
+        ta = 't';
+        lda = mat->stride[0];
+    } else {
+        a = THGPUTensor_newClone(mat);  // row-major dense: the transposed case
+        ta = 't';
+        lda = a->stride[0];
+    }
+    THGPUBlas_gemm(ta, 'n', mat->size[0], 1, mat->size[1], alpha, THGPUTensor_data(a), lda, THGPUTensor_data(x),
+                   mat->size[1], beta, THGPUTensor_data(y), mat->size[0]);
+    if (a != mat) THGPUTensor_free(a);
+    THGPUTensor_free(x);
+    THGPUTensor_freeCopyTo(y, r_);
+}
+
+void THGPUTensor_addr(THGPUTensor *r_, float beta, THGPUTensor *t, float alpha, THGPUTensor *vec1, THGPUTensor *vec2) {
+    if (vec1->nDimension != 1 || vec2->nDimension != 1) {
+        raise("vector and vector expected");
+        return;
+    }
+    if (t->nDimension != 2 || t->size[0] != vec1->size[0] || t->size[1] != vec2->size[0]) {
+        raise("size mismatch");
+        return;
+    }
+    if (r_ != t) {
+        THGPUTensor_resizeAs(r_, t);
+        THGPUTensor_copy(r_, t);
+    }
+    // r = beta*r + alpha * vec1 (x) vec2: a GEMM with a reduction of length one on a dense row-major r.
+    THGPUTensor *r = THGPUTensor_newContiguous(r_);
+    THGPUTensor *x = THGPUTensor_newContiguous(vec1);
+    THGPUTensor *y = THGPUTensor_newContiguous(vec2);
+    const long m = vec1->size[0], n = vec2->size[0];
+    // column-major view of row-major r is n x m: r'(j, i) = alpha * y(j) * x(i)
+    THGPUBlas_gemm('n', 't', n, m, 1, alpha, THGPUTensor_data(y), n, THGPUTensor_data(x), m, beta, THGPUTensor_data(r),
+                   n);
+    THGPUTensor_free(x);
+    THGPUTensor_free(y);
+    THGPUTensor_freeCopyTo(r, r_);
+}
+
+}  // extern "C"

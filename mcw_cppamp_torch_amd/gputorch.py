@@ -312,6 +312,59 @@ class GPUTensor(object):
         _lib.check()
         return self
 
+    # ---- math (the overloads of the Lua methods, gputorch/TensorMath.cpp wrap of THCTensorMath.h) ----
+    def t(self):
+        assert self.dim() == 2, "t() expects a matrix"
+        return self.transpose(0, 1)
+
+    def add(self, *args):
+        """x:add(value) | x:add(y) | x:add(value, y)  (value defaults to 1)."""
+        if len(args) == 1 and not isinstance(args[0], GPUTensor):
+            lib.THGPUTensor_add(self._p, self._p, float(args[0]))
+        else:
+            value, other = (1.0, args[0]) if len(args) == 1 else (float(args[0]), args[1])
+            lib.THGPUTensor_cadd(self._p, self._p, value, other._p)
+        _lib.check()
+        return self
+
+    def mul(self, value):
+        lib.THGPUTensor_mul(self._p, self._p, float(value))
+        _lib.check()
+        return self
+
+    def div(self, value):
+        lib.THGPUTensor_div(self._p, self._p, float(value))
+        _lib.check()
+        return self
+
+    @staticmethod
+    def _blas_args(args, ntensors):
+        """([beta,] [alpha,] [t,] a, b) -> beta, alpha, t-or-None, a, b as the Lua methods accept them."""
+        nums = [float(a) for a in args if not isinstance(a, GPUTensor)]
+        tens = [a for a in args if isinstance(a, GPUTensor)]
+        assert len(nums) <= 2 and len(tens) in (ntensors, ntensors + 1), "bad arguments"
+        beta, alpha = (1.0, 1.0) if not nums else (1.0, nums[0]) if len(nums) == 1 else (nums[0], nums[1])
+        t = tens[0] if len(tens) == ntensors + 1 else None
+        return beta, alpha, t, tens[-2], tens[-1]
+
+    def addmm(self, *args):
+        beta, alpha, t, m1, m2 = self._blas_args(args, 2)
+        lib.THGPUTensor_addmm(self._p, beta, (t or self)._p, alpha, m1._p, m2._p)
+        _lib.check()
+        return self
+
+    def addmv(self, *args):
+        beta, alpha, t, mat, vec = self._blas_args(args, 2)
+        lib.THGPUTensor_addmv(self._p, beta, (t or self)._p, alpha, mat._p, vec._p)
+        _lib.check()
+        return self
+
+    def addr(self, *args):
+        beta, alpha, t, v1, v2 = self._blas_args(args, 2)
+        lib.THGPUTensor_addr(self._p, beta, (t or self)._p, alpha, v1._p, v2._p)
+        _lib.check()
+        return self
+
     def __getitem__(self, idx):  # 0-based element access (slow, blocking)
         if np.isscalar(idx):
             idx = (idx,)

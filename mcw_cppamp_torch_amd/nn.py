@@ -6,6 +6,7 @@ to the C ABI the way the Lua modules dispatch to `input.nn.<Op>_<method>`:
   nn.SpatialConvolutionMM  mcw_nn/SpatialConvolutionMM.lua:1-60
   nn.SpatialMaxPooling     mcw_nn/SpatialMaxPooling.lua:1-34
   nn.Threshold / nn.ReLU   mcw_nn/Threshold.lua:1-21, mcw_nn/ReLU.lua:1-5
+  nn.Linear                mcw_nn/Linear.lua:1-104 (the classifier after a conv stack)
 
 Same constructor arguments, field names and call order.  Modules are created
 with host tensors (numpy float32, like torch.Tensor) and moved with :gpu();
@@ -226,6 +227,76 @@ class SpatialConvolutionMM(Module):
         _lib.check_status(lib.thgpu_SpatialConvolutionMM_accGradParameters(
             input._p, gradOutput._p, self.gradWeight._p, self.gradBias._p, self.finput._p, self.fgradInput._p,
             *(self._geom() + (float(scale),))))
+
+
+class Linear(Module):
+    """nn.Linear(inputSize, outputSize): the statement-for-statement mirror of mcw_nn/Linear.lua:3-101 on GPU tensors
+    (addmv / addr / addmm of the tensor library; 1-D and 2-D inputs, the nunit == 1 special case included)."""
+
+    _assign = SpatialConvolutionMM._assign
+
+    def __init__(self, inputSize, outputSize, rng=None):
+        Module.__init__(self)
+        self.weight = FloatTensor(outputSize, inputSize)
+        self.bias = FloatTensor(outputSize)
+        self.gradWeight = FloatTensor(outputSize, inputSize)
+        self.gradBias = FloatTensor(outputSize)
+        self._rng = rng if rng is not None else np.random.default_rng()
+        self.reset()
+
+    def reset(self, stdv=None):
+        # mcw_nn/Linear.lua:15-32
+        shape = tuple(self.weight.size()) if isinstance(self.weight, GPUTensor) else self.weight.shape
+        stdv = stdv * math.sqrt(3) if stdv else 1.0 / math.sqrt(shape[1])
+        self._assign("weight", self._rng.uniform(-stdv, stdv, size=shape))
+        self._assign("bias", self._rng.uniform(-stdv, stdv, size=(shape[0],)))
+
+    def updateOutput(self, input):
+        _require_gpu(input, self.weight, self.bias, self.output)
+        if input.dim() == 1:
+            self.output.resize(self.bias.size(0))
+            self.output.copy(self.bias)
+            self.output.addmv(1, self.weight, input)
+        elif input.dim() == 2:
+            nframe, nunit = input.size(0), self.bias.size(0)
+            self.output.resize(nframe, nunit)
+            if nunit == 1:
+                self.output.zero().add(self.bias[0])
+                self.output.select(1, 0).addmv(1, input, self.weight.select(0, 0))
+            else:
+                self.output.zero().addr(1, GPUTensor(nframe).fill(1), self.bias)
+                self.output.addmm(1, input, self.weight.t())
+        else:
+            raise ValueError("input must be vector or matrix")
+        return self.output
+
+    def updateGradInput(self, input, gradOutput):
+        if self.gradInput is None:
+            return None
+        _require_gpu(input, gradOutput, self.weight, self.gradInput)
+        n = self.gradInput.nElement()
+        self.gradInput.resizeAs(input)
+        if self.gradInput.nElement() != n:
+            self.gradInput.zero()
+        if input.dim() == 1:
+            self.gradInput.addmv(0, 1, self.weight.t(), gradOutput)
+        elif input.dim() == 2:
+            self.gradInput.addmm(0, 1, gradOutput, self.weight)
+        return self.gradInput
+
+    def accGradParameters(self, input, gradOutput, scale=1):
+        _require_gpu(input, gradOutput, self.gradWeight, self.gradBias)
+        if input.dim() == 1:
+            self.gradWeight.addr(scale, gradOutput, input)
+            self.gradBias.add(scale, gradOutput)
+        elif input.dim() == 2:
+            nframe, nunit = input.size(0), self.bias.size(0)
+            ones = GPUTensor(nframe).fill(1)
+            if nunit == 1:
+                self.gradWeight.select(0, 0).addmv(scale, input.t(), gradOutput.select(1, 0))
+            else:
+                self.gradWeight.addmm(scale, gradOutput.t(), input)
+            self.gradBias.addmv(scale, gradOutput.t(), ones)
 
 
 class SpatialMaxPooling(Module):

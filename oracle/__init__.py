@@ -40,6 +40,9 @@ def _load():
     lib.oracle_get_threads.restype = _c_int
     lib.oracle_sgemm.argtypes = [ctypes.c_char, ctypes.c_char, _c_long, _c_long, _c_long, _c_float,
                                  _f32p, _c_long, _f32p, _c_long, _c_float, _f32p, _c_long]
+    lib.oracle_sgemv.argtypes = [ctypes.c_char, _c_long, _c_long, _c_float, _f32p, _c_long, _f32p, _c_long, _c_float,
+                                 _f32p, _c_long]
+    lib.oracle_sger.argtypes = [_c_long, _c_long, _c_float, _f32p, _c_long, _f32p, _c_long, _f32p, _c_long]
     lib.oracle_im2col.argtypes = [_f32p, _c_long] + ints(9) + [_f32p]
     lib.oracle_col2im.argtypes = [_f32p, _c_long] + ints(9) + [_f32p]
     lib.oracle_conv_updateOutput.argtypes = [_f32p, _c_long] + ints(3) + [_f32p, _f32p] + ints(7) + [_f32p, _f32p]
@@ -110,6 +113,76 @@ def sgemm(transa, transb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc):
     """Column-major BLAS sgemm on flat float32 arrays; c is updated in place."""
     _lib.oracle_sgemm(transa.encode(), transb.encode(), m, n, k, alpha, _p(a), lda, _p(b), ldb, beta, _p(c), ldc)
     return c
+
+
+# ---- THTensor addmm / addmv / addr on row-major (C-contiguous) arrays -------------------------------
+# TH sees a C-contiguous matrix as one whose SECOND dimension is contiguous, i.e. as the transpose of a
+# column-major matrix; the dispatchers below make the BLAS calls TH/generic/THTensorMath.c makes for that case.
+def addmm(beta, t, alpha, m1, m2):
+    """r = beta*t + alpha*m1@m2 as THTensor_(addmm) (THTensorMath.c:458-561) computes it for contiguous
+    operands: r has stride[1] == 1, so the operands are swapped and r^T = m2^T m1^T goes to gemm('n','n')."""
+    t, m1, m2 = _f32(t), _f32(m1), _f32(m2)
+    m, k = m1.shape
+    k2, n = m2.shape
+    assert k == k2 and t.shape == (m, n)
+    r = t.copy()
+    _lib.oracle_sgemm(b"n", b"n", n, m, k, alpha, _p(m2), n, _p(m1), k, beta, _p(r), n)
+    return r
+
+
+def addmv(beta, t, alpha, mat, vec):
+    """r = beta*t + alpha*mat@vec as THTensor_(addmv) (THTensorMath.c:369-420): a C-contiguous mat has
+    stride[1] == 1 and goes to gemv('t', n, m, ...)."""
+    t, mat, vec = _f32(t), _f32(mat), _f32(vec)
+    m, n = mat.shape
+    assert vec.shape == (n,) and t.shape == (m,)
+    r = t.copy()
+    _lib.oracle_sgemv(b"t", n, m, alpha, _p(mat), n, _p(vec), 1, beta, _p(r), 1)
+    return r
+
+
+def addmv_t(beta, t, alpha, mat, vec):
+    """r = beta*t + alpha*mat.T@vec for a C-contiguous mat: the transposed view has stride[0] == 1 and
+    goes to gemv('n', ...) (THTensorMath.c:389-394)."""
+    t, mat, vec = _f32(t), _f32(mat), _f32(vec)
+    m, n = mat.shape
+    assert vec.shape == (m,) and t.shape == (n,)
+    r = t.copy()
+    _lib.oracle_sgemv(b"n", n, m, alpha, _p(mat), n, _p(vec), 1, beta, _p(r), 1)
+    return r
+
+
+def addr(beta, t, alpha, vec1, vec2):
+    """r = beta*t + alpha*outer(vec1, vec2) as THTensor_(addr) (THTensorMath.c:563-610): r scaled by beta
+    first unless beta == 1, then ger with the vectors swapped because r has stride[1] == 1."""
+    t, vec1, vec2 = _f32(t), _f32(vec1), _f32(vec2)
+    m, n = vec1.shape[0], vec2.shape[0]
+    assert t.shape == (m, n)
+    r = t.copy()
+    if beta != 1:
+        r *= np.float32(beta)
+    _lib.oracle_sger(n, m, alpha, _p(vec2), 1, _p(vec1), 1, _p(r), n)
+    return r
+
+
+# ---- nn.Linear on 2-D inputs, statement by statement (mcw_nn/Linear.lua:34-101) ------------------------
+def linear_updateOutput(inp, weight, bias):
+    inp, weight, bias = _f32(inp), _f32(weight), _f32(bias)
+    nframe = inp.shape[0]
+    out = addr(1.0, np.zeros((nframe, bias.shape[0]), np.float32), 1.0, np.ones(nframe, np.float32), bias)
+    return addmm(1.0, out, 1.0, inp, np.ascontiguousarray(weight.T))
+
+
+def linear_updateGradInput(gradOutput, weight):
+    gradOutput, weight = _f32(gradOutput), _f32(weight)
+    return addmm(0.0, np.zeros((gradOutput.shape[0], weight.shape[1]), np.float32), 1.0, gradOutput, weight)
+
+
+def linear_accGradParameters(inp, gradOutput, gradWeight, gradBias, scale=1.0):
+    """Accumulates into gradWeight / gradBias in place."""
+    inp, gradOutput = _f32(inp), _f32(gradOutput)
+    gradWeight[...] = addmm(1.0, gradWeight, scale, np.ascontiguousarray(gradOutput.T), inp)
+    gradBias[...] = addmv_t(1.0, gradBias, scale, gradOutput, np.ones(inp.shape[0], np.float32))
 
 
 def im2col(im, kH, kW, pH, pW, sH, sW):

@@ -19,6 +19,8 @@
  *       torch.nn.functional.conv2d + autograd on the CPU.
  *   sgemm fallback loops: float64 numpy product, exact small-integer matrices,
  *       all four transpose variants with ragged leading dimensions.
+ *   sgemv / sger fallback loops (the classifier's addmv / addr): float64 numpy
+ *       products, exact small-integer cases, both gemv orientations.
  *   max-pool fwd/bwd: reference known answers with overlapping windows and
  *       ties, brute force, torch max_pool2d(return_indices=True).
  *   threshold: closed form.
@@ -117,6 +119,49 @@ void oracle_sgemm(char transa, char transb, long m, long n, long k, float alpha,
         return;
     }
     sgemm_loops(transa, transb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+}
+
+/* ------------------------------------------------------------------------- */
+/* Column-major y = beta*y + alpha*op(A)*x, the TH fallback loops:
+ * TH/generic/THBlas.c:181-235.  't': one float accumulator per output, j
+ * ascending, then beta*y + alpha*sum (:214-222); 'n': y scaled by beta first
+ * unless beta == 1, then columns added j ascending with z = alpha*x[j]
+ * (:225-234). */
+void oracle_sgemv(char trans, long m, long n, float alpha, const float *a, long lda,
+                  const float *x, long incx, float beta, float *y, long incy)
+{
+    long i, j;
+    if (n == 1) lda = m;
+    if (trans == 't' || trans == 'T') {
+        for (i = 0; i < n; i++) {
+            float sum = 0;
+            const float *row_ = a + lda * i;
+            for (j = 0; j < m; j++) sum += x[j * incx] * row_[j];
+            y[i * incy] = beta * y[i * incy] + alpha * sum;
+        }
+    } else {
+        if (beta != 1)
+            for (i = 0; i < m; i++) y[i * incy] *= beta;
+        for (j = 0; j < n; j++) {
+            const float *column_ = a + lda * j;
+            float z = alpha * x[j * incx];
+            for (i = 0; i < m; i++) y[i * incy] += z * column_[i];
+        }
+    }
+}
+
+/* Column-major A += alpha * x * y^T, the TH fallback loops:
+ * TH/generic/THBlas.c:237-268 (z = alpha*y[j], then column_[i] += z*x[i]). */
+void oracle_sger(long m, long n, float alpha, const float *x, long incx, const float *y,
+                 long incy, float *a, long lda)
+{
+    long i, j;
+    if (n == 1) lda = m;
+    for (j = 0; j < n; j++) {
+        float *column_ = a + j * lda;
+        float z = alpha * y[j * incy];
+        for (i = 0; i < m; i++) column_[i] += z * x[i * incx];
+    }
 }
 
 /* ------------------------------------------------------------------------- */

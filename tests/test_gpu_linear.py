@@ -1,0 +1,207 @@
+"""GPU parity of the tensor math behind nn.Linear (THGPUTensor_addmm / addmv / addr / add / mul / div / cadd)
+and of nn.Linear itself, through the C ABI, against the CPU oracle.
+
+Bars: exact on small-integer data (every product and sum is exact in fp32, so any summation order must give
+the same bits); otherwise max error relative to the largest reference magnitude below 1e-4*sqrt(reduction
+length).
+"""
+import numpy as np
+import pytest
+
+from helpers import gemm_tol, rel_err, rng_for, uniform
+
+pytestmark = pytest.mark.gpu
+
+import oracle  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def gt():
+    import mcw_cppamp_torch_amd as pkg
+    assert pkg._lib.lib.thgpu_init() == 0, pkg._lib.lib.thgpu_last_error()
+    return pkg
+
+
+def dev(gt, a):
+    return gt.GPUTensor.from_numpy(np.ascontiguousarray(a, np.float32))
+
+
+def ints(rng, shape):
+    return rng.integers(-3, 4, shape).astype(np.float32)
+
+
+def view_of(gt, a, kind):
+    """A device tensor with the values of `a` laid out as `kind`: dense, the transpose of a dense transposed
+    copy (first dimension contiguous), or a window of a larger buffer (neither dimension contiguous... the
+    column window keeps stride[1] == 1 but a row pitch larger than the row)."""
+    if kind == "dense":
+        return dev(gt, a)
+    if kind == "transposed":
+        return dev(gt, a.T).t()
+    if kind == "window":
+        big = np.full((a.shape[0] + 2, a.shape[1] + 3), 7.0, np.float32)
+        big[1:1 + a.shape[0], 2:2 + a.shape[1]] = a
+        return dev(gt, big).narrow(0, 1, a.shape[0]).narrow(1, 2, a.shape[1])
+    if kind == "strided":            # every second column of a wider buffer: no dimension contiguous
+        big = np.full((a.shape[0], 2 * a.shape[1]), 7.0, np.float32)
+        big[:, ::2] = a
+        wide = dev(gt, big)
+        t = gt.GPUTensor(_ptr=gt._lib.lib.THGPUTensor_newWithStorage2d(
+            gt._lib.lib.THGPUTensor_storage(wide._p), 0, a.shape[0], 2 * a.shape[1], a.shape[1], 2))
+        t._keep = wide
+        return t
+    raise ValueError(kind)
+
+
+KINDS = ["dense", "transposed", "window", "strided"]
+
+
+@pytest.mark.parametrize("kr", KINDS)
+@pytest.mark.parametrize("k1", KINDS)
+@pytest.mark.parametrize("k2", ["dense", "transposed", "strided"])
+def test_addmm_every_view_combination_exact(gt, kr, k1, k2):
+    rng = rng_for(81)
+    m, k, n = 9, 13, 7
+    t, m1, m2 = ints(rng, (m, n)), ints(rng, (m, k)), ints(rng, (k, n))
+    r = view_of(gt, t, kr)
+    r.addmm(2.0, 3.0, view_of(gt, m1, k1), view_of(gt, m2, k2))
+    assert np.array_equal(r.float(), 2 * t + 3 * (m1 @ m2))
+
+
+@pytest.mark.parametrize("mnk", [(130, 70, 300), (64, 256, 100), (1, 9, 33), (257, 1, 17), (128, 4096, 1024)])
+def test_addmm_tolerance_and_separate_result(gt, mnk):
+    m, n, k = mnk
+    rng = rng_for(82)
+    t, m1, m2 = uniform(rng, (m, n)), uniform(rng, (m, k)), uniform(rng, (k, n))
+    r = gt.GPUTensor()
+    r.addmm(0.5, dev(gt, t), 1.5, dev(gt, m1), dev(gt, m2))          # r is resized to t and takes its values
+    assert r.size() == (m, n)
+    ref = 0.5 * t.astype(np.float64) + 1.5 * (m1.astype(np.float64) @ m2.astype(np.float64))
+    assert rel_err(r.float(), ref) < gemm_tol(k)
+    oracle.use_blas(k >= 1024)
+    try:
+        assert rel_err(r.float(), oracle.addmm(0.5, t, 1.5, m1, m2)) < gemm_tol(k)
+    finally:
+        oracle.use_blas(False)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("vstride", [1, 3])
+def test_addmv_views_exact(gt, kind, vstride):
+    rng = rng_for(83)
+    m, n = 11, 6
+    mat, vec, t = ints(rng, (m, n)), ints(rng, (n,)), ints(rng, (m,))
+    buf = np.full(n * vstride, 9.0, np.float32)
+    buf[::vstride] = vec
+    dvec = dev(gt, buf)
+    if vstride != 1:
+        v = gt.GPUTensor(_ptr=gt._lib.lib.THGPUTensor_newWithStorage1d(
+            gt._lib.lib.THGPUTensor_storage(dvec._p), 0, n, vstride))
+    else:
+        v = dvec
+    r = dev(gt, t)
+    r.addmv(2.0, 3.0, view_of(gt, mat, kind), v)
+    assert np.array_equal(r.float(), 2 * t + 3 * (mat @ vec))
+    assert np.array_equal(r.float(), oracle.addmv(2.0, t, 3.0, mat, vec))
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_addr_views_exact(gt, kind):
+    rng = rng_for(84)
+    m, n = 8, 5
+    t, v1, v2 = ints(rng, (m, n)), ints(rng, (m,)), ints(rng, (n,))
+    r = view_of(gt, t, kind)
+    r.addr(2.0, 3.0, dev(gt, v1), dev(gt, v2))
+    assert np.array_equal(r.float(), 2 * t + 3 * np.outer(v1, v2))
+    assert np.array_equal(r.float(), oracle.addr(2.0, t, 3.0, v1, v2))
+
+
+def test_scalar_ops_and_cadd_exact(gt):
+    rng = rng_for(85)
+    a, b = uniform(rng, (7, 33)), uniform(rng, (7, 33))
+    x = dev(gt, a)
+    assert np.array_equal(x.add(0.25).float(), a + np.float32(0.25))
+    assert np.array_equal(x.mul(3.0).float(), (a + np.float32(0.25)) * np.float32(3.0))
+    assert np.array_equal(x.div(7.0).float(), ((a + np.float32(0.25)) * np.float32(3.0)) / np.float32(7.0))
+    y = dev(gt, a)
+    y.add(0.5, dev(gt, b))
+    assert np.array_equal(y.float(), a + np.float32(0.5) * b)        # a + value*b, one rounding each (no fma)
+    z = view_of(gt, a, "transposed")
+    z.add(dev(gt, b))
+    assert np.array_equal(z.float(), a + b)
+
+
+def test_math_argument_errors(gt):
+    a, b = dev(gt, np.zeros((3, 4), np.float32)), dev(gt, np.zeros((5, 6), np.float32))
+    with pytest.raises(gt.THGPUError, match="size mismatch"):
+        dev(gt, np.zeros((3, 6), np.float32)).addmm(a, b)
+    with pytest.raises(gt.THGPUError, match="matrix and vector expected"):
+        dev(gt, np.zeros(3, np.float32)).addmv(a, a)
+    with pytest.raises(gt.THGPUError, match="vector and vector expected"):
+        a.addr(a, a)
+
+
+@pytest.mark.parametrize("shape", [(6, 11, 5), (128, 300, 64), (3, 20, 1)])
+def test_linear_fwd_bwd_matches_oracle(gt, shape):
+    B, I, O = shape
+    rng = rng_for(86)
+    m = gt.nn.Linear(I, O, rng=np.random.default_rng(5))
+    w, b = np.array(m.weight), np.array(m.bias)
+    x, go = uniform(rng, (B, I)), uniform(rng, (B, O))
+    gw0, gb0 = uniform(rng, (O, I)), uniform(rng, (O,))
+    m.gpu()
+    m.gradWeight.copy(gw0)
+    m.gradBias.copy(gb0)
+    dx, dgo = dev(gt, x), dev(gt, go)
+    out = m.forward(dx).float()
+    gi = m.backward(dx, dgo, 0.5).float()
+    assert rel_err(out, oracle.linear_updateOutput(x, w, b)) < gemm_tol(I)
+    assert rel_err(gi, oracle.linear_updateGradInput(go, w)) < gemm_tol(O)
+    gw, gb = gw0.copy(), gb0.copy()
+    oracle.linear_accGradParameters(x, go, gw, gb, 0.5)
+    assert rel_err(m.gradWeight.float(), gw) < gemm_tol(B)
+    assert rel_err(m.gradBias.float(), gb) < gemm_tol(B)
+
+
+def test_linear_vector_input(gt):
+    I, O = 17, 9
+    rng = rng_for(87)
+    m = gt.nn.Linear(I, O, rng=np.random.default_rng(6))
+    w, b = np.array(m.weight), np.array(m.bias)
+    x, go = uniform(rng, (I,)), uniform(rng, (O,))
+    m.gpu()
+    m.zeroGradParameters()
+    out = m.forward(dev(gt, x)).float()
+    gi = m.backward(dev(gt, x), dev(gt, go)).float()
+    assert rel_err(out, oracle.addmv(1.0, b, 1.0, w, x)) < gemm_tol(I)
+    assert rel_err(gi, oracle.addmv_t(0.0, np.zeros(I, np.float32), 1.0, w, go)) < gemm_tol(O)
+    assert rel_err(m.gradWeight.float(), np.outer(go, x)) < 1e-6
+    assert np.array_equal(m.gradBias.float(), go)
+
+
+def test_alexnet_classifier_sizes(gt):
+    """The classifier that follows the AlexNet-style conv stack at batch 128: 9216 -> 4096 -> 4096 -> 1000."""
+    rng = rng_for(88)
+    B = 128
+    x = uniform(rng, (B, 9216))
+    oracle.use_blas(True)
+    try:
+        for I, O in ((9216, 4096), (4096, 4096), (4096, 1000)):
+            m = gt.nn.Linear(I, O, rng=np.random.default_rng(I + O))
+            w, b = np.array(m.weight), np.array(m.bias)
+            go = uniform(rng, (B, O))
+            m.gpu()
+            m.zeroGradParameters()
+            dx = dev(gt, x)
+            out = m.forward(dx).float()
+            gi = m.backward(dx, dev(gt, go)).float()
+            ref = oracle.linear_updateOutput(x, w, b)
+            assert rel_err(out, ref) < gemm_tol(I)
+            assert rel_err(gi, oracle.linear_updateGradInput(go, w)) < gemm_tol(O)
+            gw, gb = np.zeros_like(w), np.zeros_like(b)
+            oracle.linear_accGradParameters(x, go, gw, gb, 1.0)
+            assert rel_err(m.gradWeight.float(), gw) < gemm_tol(B)
+            assert rel_err(m.gradBias.float(), gb) < gemm_tol(B)
+            x = np.maximum(ref, 0)
+    finally:
+        oracle.use_blas(False)

@@ -244,3 +244,44 @@ def test_threshold_closed_form():
     assert np.array_equal(oracle.threshold_updateOutput(x), np.array([0, 0, 0, 1e-30, 2, np.inf, 0], np.float32))
     assert np.array_equal(oracle.threshold_updateGradInput(x, g), np.array([0, 0, 0, 4, 5, 6, 0], np.float32))
     assert np.array_equal(oracle.threshold_updateOutput(x, 1.0, -7.0), np.array([-7, -7, -7, -7, 2, np.inf, -7], np.float32))
+
+
+# ---- THTensor addmm / addmv / addr and nn.Linear (the classifier after a conv stack) -----------------
+def test_oracle_addmm_addmv_addr_exact_on_small_integers():
+    rng = rng_for(71)
+    m1 = rng.integers(-3, 4, (5, 7)).astype(np.float32)
+    m2 = rng.integers(-3, 4, (7, 4)).astype(np.float32)
+    t = rng.integers(-3, 4, (5, 4)).astype(np.float32)
+    assert np.array_equal(oracle.addmm(2.0, t, 3.0, m1, m2), 2 * t + 3 * (m1 @ m2))
+    assert np.array_equal(oracle.addmm(0.0, np.full_like(t, np.nan), 1.0, m1, m2), m1 @ m2)   # beta 0 ignores t
+    v7, v5, v4 = (rng.integers(-3, 4, n).astype(np.float32) for n in (7, 5, 4))
+    assert np.array_equal(oracle.addmv(2.0, v5, 3.0, m1, v7), 2 * v5 + 3 * (m1 @ v7))
+    assert np.array_equal(oracle.addmv_t(2.0, v7, 3.0, m1, v5), 2 * v7 + 3 * (m1.T @ v5))
+    assert np.array_equal(oracle.addr(2.0, t, 3.0, v5, v4), 2 * t + 3 * np.outer(v5, v4))
+
+
+def test_oracle_gemv_orders_follow_the_th_loops():
+    # 't' (row-major mat @ vec): one accumulator, j ascending -> (1*1 + 1e8) - 1e8 = 0 in fp32, not 1
+    mat = np.array([[1.0, 1e8, -1e8]], np.float32)
+    assert oracle.addmv(0.0, np.zeros(1, np.float32), 1.0, mat, np.ones(3, np.float32))[0] == 0.0
+    mat = np.array([[1e8, -1e8, 1.0]], np.float32)
+    assert oracle.addmv(0.0, np.zeros(1, np.float32), 1.0, mat, np.ones(3, np.float32))[0] == 1.0
+    # 'n' (mat.T @ vec): columns added j ascending into y
+    mat = np.array([[1.0], [1e8], [-1e8]], np.float32)
+    assert oracle.addmv_t(1.0, np.zeros(1, np.float32), 1.0, mat, np.ones(3, np.float32))[0] == 0.0
+
+
+def test_oracle_linear_matches_torch_linear_and_autograd():
+    torch = pytest.importorskip("torch")
+    rng = rng_for(72)
+    B, I, O = 6, 11, 5
+    x, w, b, go = uniform(rng, (B, I)), uniform(rng, (O, I)), uniform(rng, (O,)), uniform(rng, (B, O))
+    tx, tw, tb = (torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in (x, w, b))
+    out = torch.nn.functional.linear(tx, tw, tb)
+    out.backward(torch.tensor(go, dtype=torch.float64))
+    assert rel_err(oracle.linear_updateOutput(x, w, b), out.detach().numpy()) < 1e-6
+    assert rel_err(oracle.linear_updateGradInput(go, w), tx.grad.numpy()) < 1e-6
+    gw, gb = np.zeros_like(w), np.zeros_like(b)
+    oracle.linear_accGradParameters(x, go, gw, gb, 0.5)
+    assert rel_err(gw, 0.5 * tw.grad.numpy()) < 1e-6
+    assert rel_err(gb, 0.5 * tb.grad.numpy()) < 1e-6
