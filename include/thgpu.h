@@ -133,6 +133,10 @@ long thgpu_prof_report(char *buf, long cap); /* returns the length needed */
  * division against the C operators over a sweep of divisors and dividends).
  * Needs no GPU.  Returns the number of mismatches. */
 long thgpu_selftest_index_math(void);
+/* Host-only check of the im2col strip planner and the max-pool backward tile planner over a grid of
+ * geometries (LDS budgets, coverage, index ranges); returns the number of violations (no counterpart in the
+ * reference). */
+long thgpu_selftest_launch_plans(void);
 
 /* ---- THGPUStorage: TH/generic/THStorage.h:33-65 instantiated for GPU,
  *      implementation replaced: gputorch/lib/THC/THCStorage.cpp:7-198 -------- */

@@ -71,6 +71,7 @@ _SIGNATURES = {
     "thgpu_prof_reset": (c_int, []),
     "thgpu_prof_report": (c_long, [c_char_p, c_long]),
     "thgpu_selftest_index_math": (c_long, []),
+    "thgpu_selftest_launch_plans": (c_long, []),
     # storage
     "THGPUStorage_data": (f32p, [StorageP]),
     "THGPUStorage_size": (c_long, [StorageP]),

@@ -655,6 +655,43 @@ int im2col_launch(const float *im, long B, int C, int H, int W, int kH, int kW, 
     return 0;
 }
 
+// Host check of the strip planner over a grid of geometries: every plan must keep the LDS tile within
+// its budget, cover the plane exactly, and keep every LDS index of the kernel inside the tile.
+long im2col_plan_selftest() {
+    long bad = 0;
+    const int sizes[] = {1, 2, 5, 6, 7, 12, 13, 14, 24, 27, 28, 55, 56, 57, 112, 224, 231, 300, 1000, 5000};
+    const int kernels[] = {1, 2, 3, 5, 7, 11};
+    for (int H : sizes)
+        for (int W : sizes)
+            for (int k : kernels)
+                for (int st = 1; st <= 4; st += (st == 1 ? 1 : 2))
+                    for (int pad = 0; pad <= k / 2; pad += (k / 2 > 0 ? k / 2 : 1)) {
+                        ConvGeom g;
+                        if (H + 2 * pad < k || W + 2 * pad < k) continue;
+                        if (make_geom(g, 4, 3, H, W, k, k, pad, pad, st, st)) continue;
+                        for (long planes : {1L, 7L, 4096L}) {
+                            StripPlan p;
+                            if (!plan_strips(g, planes, p)) continue;
+                            const long LP = (long)p.LH * p.LW;
+                            const long positions = (long)p.G * p.TR * g.Wo;
+                            const long slots = (positions + p.PL - 1) / p.PL;
+                            bool ok = p.G >= 1 && p.TR >= 1 && p.TR <= g.Ho && (p.G == 1 || p.TR == g.Ho) &&
+                                      p.G <= planes && p.G * LP * 4 <= 32 * 1024 &&
+                                      p.LW == (g.Wo - 1) * g.sW + g.kW && p.LH == (p.TR - 1) * g.sH + g.kH &&
+                                      p.PL % 64 == 0 && p.PL >= 64 && p.TG >= 1 && p.PL * p.TG <= 256 &&
+                                      (slots <= 4 || p.PL == 256) && (long)p.tiles * p.TR >= g.Ho &&
+                                      (long)(p.tiles - 1) * p.TR < g.Ho &&
+                                      (long)p.G * g.kH * g.kW * g.N * 4 < (1L << 32);
+                            // largest LDS index the column loop forms: last plane, last row and column, last tap
+                            const long last = (p.G - 1) * LP + (long)(p.TR - 1) * g.sH * p.LW + (long)(g.Wo - 1) * g.sW +
+                                              (long)(g.kH - 1) * p.LW + (g.kW - 1);
+                            ok = ok && last < p.G * LP;
+                            if (!ok) ++bad;
+                        }
+                    }
+    return bad;
+}
+
 int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW,
                   float *im) {
     ConvGeom g;

@@ -18,4 +18,8 @@ int threshold_fwd_launch(const float *in, float *out, long n, float th, float va
 int threshold_bwd_launch(const float *in, const float *gout, float *gin, long n, float th);
 int gradbias_launch(const float *gout, float *gbias, long B, int M, long N, float scale);
 
+// Host-only checks of the launch planners (no GPU needed); each returns the number of violations.
+long im2col_plan_selftest();
+long pool_plan_selftest();
+
 }  // namespace thgpu

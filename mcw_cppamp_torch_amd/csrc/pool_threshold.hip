@@ -389,6 +389,38 @@ int maxpool_fwd_launch(const float *in, long planes, int H, int W, int kH, int k
     return check_launch("maxpool_fwd");
 }
 
+// Host check of the backward tile planner: the window rows and columns a strip's pixels look up must
+// lie inside the staged tile, which must fit its LDS budget.
+long pool_plan_selftest() {
+    long bad = 0;
+    const int sizes[] = {2, 3, 6, 7, 12, 13, 14, 24, 27, 28, 55, 56, 112, 224, 231, 1000, 5000};
+    for (int H : sizes)
+        for (int W : sizes)
+            for (int k = 1; k <= 4; ++k)
+                for (int d = 1; d <= 4; ++d) {
+                    const int th = (k + d - 1) / d;
+                    if (H < k || W < k || !(th == 1 || th == 2)) continue;
+                    PoolGeom g;
+                    g.H = H; g.W = W; g.kH = k; g.kW = k; g.dH = d; g.dW = d;
+                    g.Ho = (H - k) / d + 1;
+                    g.Wo = (W - k) / d + 1;
+                    for (long planes : {1L, 5L, 4096L}) {
+                        PoolBwdPlan p;
+                        if (!plan_pool_bwd(g, planes, th, th, p)) continue;
+                        bool ok = p.G >= 1 && p.G <= planes && p.PR >= 1 && p.PR <= H && (p.G == 1 || p.PR == H) &&
+                                  (long)p.G * p.RW * p.CW * 8 <= kPoolBwdLdsBytes && (long)p.tiles * p.PR >= H &&
+                                  (long)(p.tiles - 1) * p.PR < H && p.CW >= (W - 1) / d + th;
+                        for (int t = 0; t < p.tiles && ok; ++t) {
+                            const int h0 = t * p.PR, h1 = (h0 + p.PR < H ? h0 + p.PR : H) - 1;
+                            const int i_first = h0 / d - (th - 1);
+                            ok = h1 / d - i_first < p.RW;  // the last pixel row's newest window row
+                        }
+                        if (!ok) ++bad;
+                    }
+                }
+    return bad;
+}
+
 int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int H, int W, int Ho, int Wo, int kH,
                        int kW, int dH, int dW, float *gin) {
     hipStream_t s = stream();

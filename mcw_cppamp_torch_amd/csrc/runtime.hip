@@ -1,6 +1,7 @@
 // Runtime plumbing of libthgpu: error reporting, the library stream, the
 // split-reduction workspace, event timing and per-kernel profiling.
 #include "common.h"
+#include "kernels.h"
 
 #include <cstdlib>
 #include <cstring>
@@ -223,6 +224,8 @@ long thgpu_selftest_index_math(void) {
     }
     return bad;
 }
+
+long thgpu_selftest_launch_plans(void) { return im2col_plan_selftest() + pool_plan_selftest(); }
 
 int thgpu_prof_enable(int on) {
     g_prof_on = on != 0;

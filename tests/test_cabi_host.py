@@ -68,6 +68,11 @@ def test_index_math_selftest(pkg):
     assert pkg._lib.lib.thgpu_selftest_index_math() == 0
 
 
+def test_launch_plan_selftest(pkg):
+    # im2col strip shapes and max-pool backward tiles over a grid of geometries, checked on the host
+    assert pkg._lib.lib.thgpu_selftest_launch_plans() == 0
+
+
 def test_metadata_only_tensor_ops_and_error_handler(pkg):
     # Views and argument errors need no device memory.
     t = pkg.GPUTensor()
