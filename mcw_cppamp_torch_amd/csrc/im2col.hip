@@ -725,7 +725,6 @@ int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW,
     if (!(generic && generic[0] == '1') && (sW > 1 || sH > 1) && W >= 64 && th <= 3 && tw <= 3) {
         // R quotient rows per workgroup: about 256 (qh, qw) pairs, image rows within the LDS budget
         int R = 256 / Qw;
-        if (const char *e = std::getenv("THGPU_COL2IM_R")) R = atoi(e);
         if (R < 1) R = 1;
         if (R > Qh) R = Qh;
         while (R > 1 && (long)R * sH * W * 4 > 48 * 1024) --R;
