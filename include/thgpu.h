@@ -214,6 +214,7 @@ THGPUTensor *THGPUTensor_newContiguous(THGPUTensor *tensor);          /* THCTens
 THGPUTensor *THGPUTensor_newSelect(THGPUTensor *tensor, int dimension, long sliceIndex);
 THGPUTensor *THGPUTensor_newNarrow(THGPUTensor *tensor, int dimension, long firstIndex, long size);
 THGPUTensor *THGPUTensor_newTranspose(THGPUTensor *tensor, int dimension1, int dimension2);
+THGPUTensor *THGPUTensor_newUnfold(THGPUTensor *tensor, int dimension, long size, long step);
 
 void THGPUTensor_resize(THGPUTensor *tensor, THLongStorage *size, THLongStorage *stride);
 void THGPUTensor_resizeAs(THGPUTensor *tensor, THGPUTensor *src);
@@ -226,9 +227,19 @@ void THGPUTensor_resize5d(THGPUTensor *tensor, long size0, long size1, long size
 void THGPUTensor_set(THGPUTensor *self, THGPUTensor *src);
 void THGPUTensor_setStorage(THGPUTensor *self, THGPUStorage *storage, long storageOffset, THLongStorage *size,
                             THLongStorage *stride);
+void THGPUTensor_setStorage1d(THGPUTensor *self, THGPUStorage *storage, long storageOffset, long size0, long stride0);
+void THGPUTensor_setStorage2d(THGPUTensor *self, THGPUStorage *storage, long storageOffset, long size0, long stride0,
+                              long size1, long stride1);
+void THGPUTensor_setStorage3d(THGPUTensor *self, THGPUStorage *storage, long storageOffset, long size0, long stride0,
+                              long size1, long stride1, long size2, long stride2);
+void THGPUTensor_setStorage4d(THGPUTensor *self, THGPUStorage *storage, long storageOffset, long size0, long stride0,
+                              long size1, long stride1, long size2, long stride2, long size3, long stride3);
 void THGPUTensor_narrow(THGPUTensor *self, THGPUTensor *src, int dimension, long firstIndex, long size);
 void THGPUTensor_select(THGPUTensor *self, THGPUTensor *src, int dimension, long sliceIndex);
 void THGPUTensor_transpose(THGPUTensor *self, THGPUTensor *src, int dimension1, int dimension2);
+void THGPUTensor_unfold(THGPUTensor *self, THGPUTensor *src, int dimension, long size, long step);   /* THCTensor.h:92; TH/generic/THTensor.c:418-460 */
+void THGPUTensor_squeeze(THGPUTensor *self, THGPUTensor *src);                                         /* TH/generic/THTensor.c:462-493 */
+void THGPUTensor_squeeze1d(THGPUTensor *self, THGPUTensor *src, int dimension);                        /* TH/generic/THTensor.c:495-513 */
 
 int THGPUTensor_isContiguous(const THGPUTensor *self);                /* THCTensor.cpp:510-525 */
 int THGPUTensor_isSameSizeAs(const THGPUTensor *self, const THGPUTensor *src);

@@ -123,6 +123,7 @@ _SIGNATURES = {
     "THGPUTensor_newSelect": (TensorP, [TensorP, c_int, c_long]),
     "THGPUTensor_newNarrow": (TensorP, [TensorP, c_int, c_long, c_long]),
     "THGPUTensor_newTranspose": (TensorP, [TensorP, c_int, c_int]),
+    "THGPUTensor_newUnfold": (TensorP, [TensorP, c_int, c_long, c_long]),
     "THGPUTensor_resize": (None, [TensorP, ctypes.POINTER(THLongStorage), ctypes.POINTER(THLongStorage)]),
     "THGPUTensor_resizeAs": (None, [TensorP, TensorP]),
     "THGPUTensor_resize1d": (None, [TensorP] + [c_long]),
@@ -136,6 +137,13 @@ _SIGNATURES = {
     "THGPUTensor_narrow": (None, [TensorP, TensorP, c_int, c_long, c_long]),
     "THGPUTensor_select": (None, [TensorP, TensorP, c_int, c_long]),
     "THGPUTensor_transpose": (None, [TensorP, TensorP, c_int, c_int]),
+    "THGPUTensor_unfold": (None, [TensorP, TensorP, c_int, c_long, c_long]),
+    "THGPUTensor_squeeze": (None, [TensorP, TensorP]),
+    "THGPUTensor_squeeze1d": (None, [TensorP, TensorP, c_int]),
+    "THGPUTensor_setStorage1d": (None, [TensorP, StorageP, c_long] + [c_long] * 2),
+    "THGPUTensor_setStorage2d": (None, [TensorP, StorageP, c_long] + [c_long] * 4),
+    "THGPUTensor_setStorage3d": (None, [TensorP, StorageP, c_long] + [c_long] * 6),
+    "THGPUTensor_setStorage4d": (None, [TensorP, StorageP, c_long] + [c_long] * 8),
     "THGPUTensor_isContiguous": (c_int, [TensorP]),
     "THGPUTensor_isSameSizeAs": (c_int, [TensorP, TensorP]),
     "THGPUTensor_nElement": (c_long, [TensorP]),

@@ -322,6 +322,24 @@ void THGPUTensor_setStorage(THGPUTensor *self, THGPUStorage *storage, long stora
             size ? size->data : nullptr, stride ? stride->data : nullptr);
 }
 
+void THGPUTensor_setStorage4d(THGPUTensor *self, THGPUStorage *storage, long storageOffset, long size0, long stride0,
+                              long size1, long stride1, long size2, long stride2, long size3, long stride3) {
+    long size[4] = {size0, size1, size2, size3};
+    long stride[4] = {stride0, stride1, stride2, stride3};
+    raw_set(self, storage, storageOffset, 4, size, stride);
+}
+void THGPUTensor_setStorage1d(THGPUTensor *self, THGPUStorage *storage, long storageOffset, long size0, long stride0) {
+    THGPUTensor_setStorage4d(self, storage, storageOffset, size0, stride0, -1, -1, -1, -1, -1, -1);
+}
+void THGPUTensor_setStorage2d(THGPUTensor *self, THGPUStorage *storage, long storageOffset, long size0, long stride0,
+                              long size1, long stride1) {
+    THGPUTensor_setStorage4d(self, storage, storageOffset, size0, stride0, size1, stride1, -1, -1, -1, -1);
+}
+void THGPUTensor_setStorage3d(THGPUTensor *self, THGPUStorage *storage, long storageOffset, long size0, long stride0,
+                              long size1, long stride1, long size2, long stride2) {
+    THGPUTensor_setStorage4d(self, storage, storageOffset, size0, stride0, size1, stride1, size2, stride2, -1, -1);
+}
+
 void THGPUTensor_narrow(THGPUTensor *self, THGPUTensor *src, int dimension, long firstIndex, long size) {
     if (!src) src = self;
     THGPU_ARGCHECK((dimension >= 0) && (dimension < src->nDimension), 3, "out of range", );
@@ -358,6 +376,78 @@ void THGPUTensor_transpose(THGPUTensor *self, THGPUTensor *src, int dimension1, 
     z = self->size[dimension1];
     self->size[dimension1] = self->size[dimension2];
     self->size[dimension2] = z;
+}
+
+// A new last dimension of length `size` walks along `dimension` with its stride; `dimension`
+// itself keeps every `step`-th start (TH/generic/THTensor.c:418-460).
+void THGPUTensor_unfold(THGPUTensor *self, THGPUTensor *src, int dimension, long size, long step) {
+    if (!src) src = self;
+    THGPU_ARGCHECK(src->nDimension > 0, 1, "cannot unfold an empty tensor", );
+    THGPU_ARGCHECK(dimension >= 0 && dimension < src->nDimension, 2, "out of range", );
+    THGPU_ARGCHECK(size <= src->size[dimension], 3, "out of range", );
+    THGPU_ARGCHECK(step > 0, 4, "invalid step", );
+    THGPUTensor_set(self, src);
+    const int nd = self->nDimension;
+    std::vector<long> new_size(nd + 1), new_stride(nd + 1);
+    new_size[nd] = size;
+    new_stride[nd] = self->stride[dimension];
+    for (int d = 0; d < nd; d++) {
+        if (d == dimension) {
+            new_size[d] = (self->size[d] - size) / step + 1;
+            new_stride[d] = step * self->stride[d];
+        } else {
+            new_size[d] = self->size[d];
+            new_stride[d] = self->stride[d];
+        }
+    }
+    self->size = static_cast<long *>(std::realloc(self->size, sizeof(long) * (nd + 1)));
+    self->stride = static_cast<long *>(std::realloc(self->stride, sizeof(long) * (nd + 1)));
+    for (int d = 0; d <= nd; d++) {
+        self->size[d] = new_size[d];
+        self->stride[d] = new_stride[d];
+    }
+    self->nDimension = nd + 1;
+}
+
+THGPUTensor *THGPUTensor_newUnfold(THGPUTensor *tensor, int dimension, long size, long step) {
+    THGPUTensor *self = THGPUTensor_newWithTensor(tensor);
+    THGPUTensor_unfold(self, nullptr, dimension, size, step);
+    return self;
+}
+
+// Drops the dimensions of length one (all of them: TH/generic/THTensor.c:462-493; one: :495-513).
+void THGPUTensor_squeeze(THGPUTensor *self, THGPUTensor *src) {
+    if (!src) src = self;
+    THGPUTensor_set(self, src);
+    int ndim = 0;
+    for (int d = 0; d < src->nDimension; d++) {
+        if (src->size[d] != 1) {
+            if (d != ndim) {
+                self->size[ndim] = src->size[d];
+                self->stride[ndim] = src->stride[d];
+            }
+            ndim++;
+        }
+    }
+    if (ndim == 0 && src->nDimension > 0) {  // no 0-dimensional tensors
+        self->size[0] = 1;
+        self->stride[0] = 1;
+        ndim = 1;
+    }
+    self->nDimension = ndim;
+}
+
+void THGPUTensor_squeeze1d(THGPUTensor *self, THGPUTensor *src, int dimension) {
+    if (!src) src = self;
+    THGPU_ARGCHECK(dimension >= 0 && dimension < src->nDimension, 3, "dimension out of range", );
+    THGPUTensor_set(self, src);
+    if (src->size[dimension] == 1 && src->nDimension > 1) {
+        for (int d = dimension; d < self->nDimension - 1; d++) {
+            self->size[d] = self->size[d + 1];
+            self->stride[d] = self->stride[d + 1];
+        }
+        self->nDimension--;
+    }
 }
 
 int THGPUTensor_isContiguous(const THGPUTensor *self) {

@@ -277,6 +277,18 @@ class GPUTensor(object):
     def transpose(self, d1, d2):
         return self._view(lib.THGPUTensor_newTranspose(self._p, int(d1), int(d2)))
 
+    def unfold(self, dim, size, step):
+        return self._view(lib.THGPUTensor_newUnfold(self._p, int(dim), int(size), int(step)))
+
+    def squeeze(self, dim=None):
+        t = self._view(lib.THGPUTensor_newWithTensor(self._p))
+        if dim is None:
+            lib.THGPUTensor_squeeze(t._p, None)
+        else:
+            lib.THGPUTensor_squeeze1d(t._p, None, int(dim))
+        _lib.check()
+        return t
+
     def contiguous(self):
         return self._view(lib.THGPUTensor_newContiguous(self._p))
 

@@ -205,3 +205,27 @@ def test_alexnet_classifier_sizes(gt):
             x = np.maximum(ref, 0)
     finally:
         oracle.use_blas(False)
+
+
+def test_unfold_squeeze_setstorage_views(gt):
+    rng = rng_for(89)
+    a = uniform(rng, (3, 1, 10, 1))
+    t = dev(gt, a)
+    assert t.squeeze().size() == (3, 10) and np.array_equal(t.squeeze().float(), a.reshape(3, 10))
+    assert t.squeeze(1).size() == (3, 10, 1) and t.squeeze(0).size() == (3, 1, 10, 1)
+    assert dev(gt, np.ones((1, 1), np.float32)).squeeze().size() == (1,)
+    v = dev(gt, np.arange(10, dtype=np.float32))
+    u = v.unfold(0, 4, 3)                      # windows [0..3], [3..6], [6..9]
+    assert u.size() == (3, 4) and u.stride() == (3, 1)
+    assert np.array_equal(u.float(), np.array([[0, 1, 2, 3], [3, 4, 5, 6], [6, 7, 8, 9]], np.float32))
+    m = dev(gt, a.reshape(3, 10))
+    u2 = m.unfold(1, 2, 4)                     # (3, 3, 2): columns {0,1}, {4,5}, {8,9}
+    assert u2.size() == (3, 3, 2)
+    assert np.array_equal(u2.float(), np.stack([a.reshape(3, 10)[:, [0, 1]], a.reshape(3, 10)[:, [4, 5]],
+                                                a.reshape(3, 10)[:, [8, 9]]], axis=1))
+    w = gt.GPUTensor()
+    lib = gt._lib.lib
+    lib.THGPUTensor_setStorage2d(w._p, lib.THGPUTensor_storage(m._p), 1, 3, 10, 4, 2)   # rows, every 2nd column from 1
+    assert w.size() == (3, 4) and np.array_equal(w.float(), a.reshape(3, 10)[:, 1:9:2])
+    with pytest.raises(gt.THGPUError, match="invalid step"):
+        v.unfold(0, 2, 0)
