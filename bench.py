@@ -13,6 +13,8 @@ Beside the throughput the line carries
                 GEMM launches of a step / their summed HIP-event durations,
                 measured in a second, instrumented run of the same K steps;
   kernels       the same for every kernel family (HBM-bound ones in GB/s);
+  gemm_shapes   every GEMM of the stack on its own (shape, chosen tile and split,
+                TFLOP/s): the small-K GEMMs of first layers are HBM-bound themselves;
   cpu_baseline  the CPU oracle (a port of the reference CPU nn path, OpenMP over
                 the batch + an optimised BLAS sgemm where one is found) timed
                 on this host on a reduced batch of the same stack.
@@ -33,7 +35,7 @@ PEAK_HBM_GBS = 8000.0
 # script (FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0, the factors a plain copy kernel of known size gives);
 # the summary with the commands is profiles/hbm_traffic_alexnet_b128_pmc.txt.  Counters cannot be read
 # from inside the timed process, so the figure is carried here for the configuration it was measured on.
-MEASURED_GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("alexnet", 128): 6.061e8}
+MEASURED_GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("alexnet", 128): 6.066e8}
 
 
 def cpu_baseline(workload, sample_batch, budget_s=20.0):
@@ -160,7 +162,7 @@ def main():
     d2h_ms = (time.perf_counter() - t1) * 1e3
 
     w = stacks.work(name, B)
-    kernels, roofline = {}, None
+    kernels, roofline, gemm_shapes = {}, None, []
     if not args.no_kernel_timing:
         gputorch.prof_reset()
         gputorch.prof_enable(True)
@@ -172,19 +174,34 @@ def main():
         gputorch.prof_reset()
         g_ms = g_fl = 0.0
         g_calls = 0
+        gemm_shapes = []
         for kname, r in sorted(rep.items()):
             ms = r["ms"] / args.steps
-            ent = {"launches_per_step": r["calls"] / args.steps, "ms_per_step": round(ms, 4)}
-            if kname.startswith("gemm_conv") or kname == "gemm_blas":
+            family = kname.split(" ")[0]          # GEMM records are labelled "<family> M=.. J=.. R=.. tile=.. split=.."
+            if family.startswith("gemm_conv") or family == "gemm_blas":
                 fl = r["flops"] / args.steps
-                ent.update(bound="mfma", tflops=round(fl / ms / 1e9, 2), frac=round(fl / ms / 1e9 / PEAK_MFMA_F32_TFLOPS, 4))
+                ent = kernels.setdefault(family, {"launches_per_step": 0.0, "ms_per_step": 0.0, "bound": "mfma",
+                                                  "flops_per_step": 0.0})
+                ent["launches_per_step"] += r["calls"] / args.steps
+                ent["ms_per_step"] += ms
+                ent["flops_per_step"] += fl
+                gemm_shapes.append({"gemm": kname, "launches_per_step": r["calls"] / args.steps,
+                                    "ms_per_step": round(ms, 4), "tflops": round(fl / ms / 1e9, 2),
+                                    "frac": round(fl / ms / 1e9 / PEAK_MFMA_F32_TFLOPS, 4)})
                 g_ms += ms
                 g_fl += fl
                 g_calls += r["calls"]
-            elif r["bytes"] > 0:
+                continue
+            ent = {"launches_per_step": r["calls"] / args.steps, "ms_per_step": round(ms, 4)}
+            if r["bytes"] > 0:
                 by = r["bytes"] / args.steps
                 ent.update(bound="hbm", gbs=round(by / ms / 1e6, 1), frac=round(by / ms / 1e6 / PEAK_HBM_GBS, 4))
             kernels[kname] = ent
+        for ent in kernels.values():
+            if ent.get("bound") == "mfma":
+                fl, ms = ent.pop("flops_per_step"), ent["ms_per_step"]
+                ent.update(ms_per_step=round(ms, 4), tflops=round(fl / ms / 1e9, 2),
+                           frac=round(fl / ms / 1e9 / PEAK_MFMA_F32_TFLOPS, 4))
         if g_ms > 0:
             roofline = {
                 "bound": "mfma", "kernel": "gemm_fast_kernel<...> (all conv GEMM launches of a step)",
@@ -210,7 +227,7 @@ def main():
         "transfers": {"h2d_input_ms": round(h2d_ms, 3), "d2h_gradinput_ms": round(d2h_ms, 3),
                       "images_per_s_including_transfers": round(B / ((ms_per_step + h2d_ms + d2h_ms) / 1e3), 1)},
         "gemm_tflops_over_whole_step": round(w["gemm_flops"] / (ms_per_step / 1e3) / 1e12, 2),
-        "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels,
+        "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels, "gemm_shapes": gemm_shapes,
     }
     print(json.dumps(line))
 

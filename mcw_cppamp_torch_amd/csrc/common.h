@@ -62,6 +62,11 @@ struct LaunchScope {
     int slot;
 };
 
+// Per-kernel timing on?  And a label for one record that is formatted only then (interned; the
+// report groups records by label), so that e.g. every GEMM shape of a network is listed on its own.
+bool prof_enabled();
+const char *prof_label(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+
 // Checks the launch itself (bad configuration shows up here, not at sync).
 int check_launch(const char *name);
 

@@ -200,7 +200,11 @@ int gemm_launch(const GemmProblem &p) {
 
     int rc;
     {
-        LaunchScope scope(p.tag, 2.0 * p.M * p.J * (double)p.R * (red ? p.nb : 1), 0.0);
+        const char *label = p.tag;
+        if (prof_enabled())
+            label = prof_label("%s M=%d J=%d R=%ld tile=%s split=%d", p.tag, p.M, p.J, (long)p.R * (red ? p.nb : 1),
+                               best ? best->name : "generic", g.nsplit);
+        LaunchScope scope(label, 2.0 * p.M * p.J * (double)p.R * (red ? p.nb : 1), 0.0);
         rc = best ? best->launch(g, la, lb, red, s) : gemm_generic_64x64(g, p.a_rc, p.b_rc, red, s);
     }
     if (rc) return rc;

@@ -6,6 +6,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <set>
 #include <string>
 #include <vector>
 
@@ -120,6 +121,18 @@ static hipEvent_t pool_event() {
     hipEvent_t e = nullptr;
     (void)hipEventCreate(&e);
     return e;
+}
+
+bool prof_enabled() { return g_prof_on; }
+
+const char *prof_label(const char *fmt, ...) {
+    static std::set<std::string> labels;  // node addresses stay valid: the returned pointer lives as long as the process
+    char buf[256];
+    va_list ap;
+    va_start(ap, fmt);
+    std::vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    return labels.insert(buf).first->c_str();
 }
 
 LaunchScope::LaunchScope(const char *name, double flops, double bytes) : slot(-1) {
