@@ -309,6 +309,15 @@ void THGPUTensor_addr(THGPUTensor *self, float beta, THGPUTensor *t, float alpha
 void THGPUBlas_gemm(char transa, char transb, long m, long n, long k, float alpha, float *a, long lda, float *b,
                     long ldb, float beta, float *c, long ldc);
 
+/* The same product for `batch` problems whose operands and results are `stride_*` floats apart
+ * (stride 0 shares an operand).  New: the reference multiplies image by image (gpunn-impl/
+ * SpatialConvolutionMM.cpp:168-217 calls THGPUBlas_gemm once per image); here a shared op(B) with
+ * transa == 'n' -- the convolution's forward and gradInput products -- runs as one launch.  Returns
+ * 0 or a status with thgpu_last_error() set. */
+int thgpu_gemm_strided_batched(char transa, char transb, long m, long n, long k, float alpha, const float *a, long lda,
+                               long stride_a, const float *b, long ldb, long stride_b, float beta, float *c, long ldc,
+                               long stride_c, long batch);
+
 /* ---- flat operator entry points -------------------------------------------- */
 
 /* Batched im2col: im [B,C,H,W] -> col [B, C*kH*kW, Ho*Wo] (device pointers).

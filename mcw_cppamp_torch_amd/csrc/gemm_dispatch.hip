@@ -269,3 +269,57 @@ extern "C" void THGPUBlas_gemm(char transa, char transb, long m, long n, long k,
     p.tag = "gemm_blas";
     if (gemm_launch(p)) raise("%s", thgpu_last_error());
 }
+
+extern "C" int thgpu_gemm_strided_batched(char transa, char transb, long m, long n, long k, float alpha, const float *a,
+                                          long lda, long stride_a, const float *b, long ldb, long stride_b, float beta,
+                                          float *c, long ldc, long stride_c, long batch) {
+    const bool ta = (transa == 't' || transa == 'T');
+    const bool tb = (transb == 't' || transb == 'T');
+    if (batch <= 0 || !m || !n) return 0;
+    if (m >= (1L << 31) || n >= (1L << 31) || k >= (1L << 31)) return fail("gemm_strided_batched: dimension exceeds 2^31");
+    if (stride_c == 0 && batch > 1) return fail("gemm_strided_batched: the results of a batch must not overlap");
+    // One launch for the whole batch when op(B) is shared, op(A) = A and the batch's columns fit the
+    // kernel's 32-bit tile indexing: the batch index then simply extends the columns of the (row-major,
+    // transposed) product, as in the convolution's forward and gradInput GEMMs.
+    if (!ta && stride_b == 0 && batch > 1 && m * batch < (1L << 31) && n * m * batch < (1L << 31)) {
+        GemmProblem p;
+        p.A = b;
+        p.B = a;
+        p.C = c;
+        p.M = (int)n;
+        p.J = (int)(m * batch);
+        p.R = alpha == 0 ? 0 : (int)k;
+        p.N = (int)m;
+        p.a_rc = !tb;
+        p.sA = ldb;
+        p.b_rc = false;
+        p.sB = lda;
+        p.sC = ldc;
+        p.bsB = stride_a;
+        p.bsC = stride_c;
+        p.alpha = alpha;
+        p.beta = beta;
+        p.tag = "gemm_blas_batched";
+        return gemm_launch(p);
+    }
+    for (long i = 0; i < batch; ++i) {
+        GemmProblem p;
+        p.A = b + i * stride_b;
+        p.B = a + i * stride_a;
+        p.C = c + i * stride_c;
+        p.M = (int)n;
+        p.J = (int)m;
+        p.R = alpha == 0 ? 0 : (int)k;
+        p.N = (int)m;
+        p.a_rc = !tb;
+        p.sA = ldb;
+        p.b_rc = ta;
+        p.sB = lda;
+        p.sC = ldc;
+        p.alpha = alpha;
+        p.beta = beta;
+        p.tag = "gemm_blas_batched";
+        if (gemm_launch(p)) return 1;
+    }
+    return 0;
+}

@@ -229,3 +229,28 @@ def test_unfold_squeeze_setstorage_views(gt):
     assert w.size() == (3, 4) and np.array_equal(w.float(), a.reshape(3, 10)[:, 1:9:2])
     with pytest.raises(gt.THGPUError, match="invalid step"):
         v.unfold(0, 2, 0)
+
+
+@pytest.mark.parametrize("ta,tb", [("n", "n"), ("n", "t"), ("t", "n"), ("t", "t")])
+@pytest.mark.parametrize("shared_b", [True, False])
+def test_gemm_strided_batched(gt, ta, tb, shared_b):
+    """Column-major C_i = beta*C_i + alpha*op(A_i)*op(B_i) for a batch; a shared B with op(A) = A takes the
+    single-launch path of the convolution products, everything else one launch per problem."""
+    rng = rng_for(90)
+    m, n, k, batch = 70, 33, 129, 5
+    A = ints(rng, (batch, k, m) if ta == "n" else (batch, m, k))       # column-major m x k (or k x m) per problem
+    B = ints(rng, (1 if shared_b else batch, n, k) if tb == "n" else (1 if shared_b else batch, k, n))
+    C = ints(rng, (batch, n, m))                                       # column-major m x n per problem
+    dA, dB, dC = dev(gt, A), dev(gt, B), dev(gt, C)
+    lib = gt._lib.lib
+    rc = lib.thgpu_gemm_strided_batched(ta.encode(), tb.encode(), m, n, k, 2.0, lib.THGPUTensor_data(dA._p),
+                                        m if ta == "n" else k, A[0].size, lib.THGPUTensor_data(dB._p),
+                                        k if tb == "n" else n, 0 if shared_b else B[0].size, 3.0,
+                                        lib.THGPUTensor_data(dC._p), m, m * n, batch)
+    gt._lib.check_status(rc)
+    got = dC.float()
+    for i in range(batch):
+        opA = A[i].T if ta == "n" else A[i]                            # m x k
+        Bi = B[0 if shared_b else i]
+        opB = Bi.T if tb == "n" else Bi                                # k x n
+        assert np.array_equal(got[i].T, 3 * C[i].T + 2 * (opA @ opB)), i
