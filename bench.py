@@ -114,7 +114,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the path is built and measured on a single MI355X "
-                 "(--gpus %d is not supported; batch sharding is described in DESIGN.md)" % args.gpus)
+                 "(--gpus %d is not supported: every GPU box of this build has one GPU, and the value reported "
+                 "is that GPU's throughput)" % args.gpus)
 
     import numpy as np
 
