@@ -87,12 +87,15 @@ struct PoolBwdPlan {
     int RW;     // window rows kept per strip (with TH-1 rows of history)
     int CW;     // window columns kept per row (with TW-1 columns of history and the uncovered right edge)
     FastDiv divTiles, divEnt, divCW, divPix;
+    FastDiv divW2, divPix2;  // pixel pairs (dW == 2): pairs per row, pairs per plane
 };
 
 // TH x TW = the most windows that can cover one pixel.  Pixel (h, w) can only
 // be the argmax of windows (i_hi - a, j_hi - b), i_hi = h / dH, j_hi = w / dW,
 // a < TH, b < TW; visiting a and b downwards is (i ascending, j ascending).
-template <int TH, int TW>
+// PAIRS (horizontal stride 2): a lane takes the two pixels (h, 2k) and (h, 2k+1), which share j_hi = k and
+// with it all their candidate windows, so each staged pair is read once for both.
+template <int TH, int TW, bool PAIRS>
 __global__ __launch_bounds__(256) void maxpool_bwd_tile_kernel(const float *__restrict__ gout,
                                                                const float *__restrict__ indy,
                                                                const float *__restrict__ indx,
@@ -142,6 +145,33 @@ __global__ __launch_bounds__(256) void maxpool_bwd_tile_kernel(const float *__re
     __syncthreads();
 
     // ---- pixels ----------------------------------------------------------------------------------
+    if (PAIRS) {
+        const int W2 = (g.W + 1) / 2;
+        const int P2 = nh * W2;
+        const int total2 = np * P2;
+        for (int q = tid; q < total2; q += nthr) {
+            unsigned pl = 0, r = (unsigned)q, hh, w2;
+            if (p.G > 1) p.divPix2.divmod(r, pl, r);  // grouped planes are whole: P2 == H*W2
+            p.divW2.divmod(r, hh, w2);
+            const int h = h0 + (int)hh, w = 2 * (int)w2;
+            const int i_hi = (int)g.divDH.div((unsigned)h), j_hi = (int)w2;
+            const int2 *e = ent + (int)pl * per_plane + (i_hi - i_first) * p.CW + j_hi + (TW - 1);
+            const int pix = h * g.W + w;
+            float acc0 = 0.0f, acc1 = 0.0f;
+#pragma unroll
+            for (int a = TH - 1; a >= 0; --a)
+#pragma unroll
+                for (int b = TW - 1; b >= 0; --b) {
+                    const int2 c = e[-a * p.CW - b];
+                    acc0 += c.x == pix ? __int_as_float(c.y) : 0.0f;
+                    acc1 += c.x == pix + 1 ? __int_as_float(c.y) : 0.0f;
+                }
+            float *out = gin + (long)(plane0 + pl) * g.H * g.W + pix;
+            out[0] = acc0;
+            if (w + 1 < g.W) out[1] = acc1;
+        }
+        return;
+    }
     const int P = nh * g.W;
     const int total = np * P;
     for (int q = tid; q < total; q += nthr) {
@@ -196,6 +226,8 @@ bool plan_pool_bwd(const PoolGeom &g, long planes, int TH, int TW, PoolBwdPlan &
     p.divEnt = FastDiv((uint32_t)(p.RW * p.CW));
     p.divCW = FastDiv((uint32_t)p.CW);
     p.divPix = FastDiv((uint32_t)(g.H * g.W));
+    p.divW2 = FastDiv((uint32_t)((g.W + 1) / 2));
+    p.divPix2 = FastDiv((uint32_t)(g.H * ((g.W + 1) / 2)));
     return true;
 }
 
@@ -448,12 +480,16 @@ int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int
             const size_t lds = sizeof(int2) * (size_t)plan.G * plan.RW * plan.CW;
             {
                 LaunchScope scope("maxpool_bwd", 0.0, bytes);
-                if (th == 2)
-                    hipLaunchKernelGGL((maxpool_bwd_tile_kernel<2, 2>), dim3((unsigned)blocks), dim3(256), lds, s, gout,
-                                       indices, indices + ototal, gin, g, plan, (unsigned)planes);
-                else
-                    hipLaunchKernelGGL((maxpool_bwd_tile_kernel<1, 1>), dim3((unsigned)blocks), dim3(256), lds, s, gout,
-                                       indices, indices + ototal, gin, g, plan, (unsigned)planes);
+                const dim3 grid((unsigned)blocks), block(256);
+                float *ix = const_cast<float *>(indices) + ototal;
+#define THGPU_POOL_BWD(TH_, TW_, PAIRS_)                                                                          \
+    hipLaunchKernelGGL((maxpool_bwd_tile_kernel<TH_, TW_, PAIRS_>), grid, block, lds, s, gout, indices, ix, gin, g, \
+                       plan, (unsigned)planes)
+                if (th == 2 && dW == 2) THGPU_POOL_BWD(2, 2, true);
+                else if (th == 2) THGPU_POOL_BWD(2, 2, false);
+                else if (dW == 2) THGPU_POOL_BWD(1, 1, true);
+                else THGPU_POOL_BWD(1, 1, false);
+#undef THGPU_POOL_BWD
             }
             return check_launch("maxpool_bwd");
         }
