@@ -42,7 +42,7 @@ struct __attribute__((packed, aligned(4))) float4u {
 // accumulators take (BM/WGM)*(BN/WGN)/64 registers of the 512 a lane has.
 template <int BM, int BN, int WGM, int WGN>
 constexpr int gemm_min_waves() {
-    return (BM / WGM) * (BN / WGN) / 64 >= 128 ? 2 : 3;
+    return (BM / WGM) * (BN / WGN) / 64 >= 96 ? 2 : 3;
 }
 
 // DBG is 0 in the library; experiments switch phases off with it (1: no global
@@ -57,7 +57,8 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     constexpr int NA = BM * BK / NT, NB = BN * BK / NT;
     static_assert(BM % (WGM * 32) == 0 && BN % (WGN * 32) == 0, "wave tile must be whole 32x32 blocks");
     static_assert(NT % 16 == 0 && NA >= 4 && NB >= 4 && NA % 4 == 0 && NB % 4 == 0, "loader shape");
-    static_assert(NT % BM == 0 && NT % BN == 0, "x-contiguous loaders give every thread one row/column");
+    static_assert((LA != LD_XC_SCALAR || NT % BM == 0) && (LB != LD_XC_SCALAR || NT % BN == 0),
+                  "x-contiguous loaders give every thread one row/column");
     static_assert(!RED || (LA != LD_XC_SCALAR && LB != LD_XC_SCALAR), "reduction batching needs r-contiguous operands");
 
     __shared__ __attribute__((aligned(16))) float As[2][BM][LDK];
@@ -373,15 +374,20 @@ int gemm_fast_go(const GemmArgs &g, hipStream_t s) {
 // Dispatch over the loader kinds for one tile configuration.
 template <int BM, int BN, int WGM, int WGN>
 int gemm_fast_dispatch(const GemmArgs &g, int la, int lb, bool red, hipStream_t s) {
-#define THGPU_CASE(LA_, LB_)                                                          \
-    if (la == LA_ && lb == LB_) {                                                     \
-        if (red) {                                                                    \
-            if constexpr (LA_ != LD_XC_SCALAR && LB_ != LD_XC_SCALAR)                 \
-                return gemm_fast_go<BM, BN, WGM, WGN, LA_, LB_, true>(g, s);          \
-            else                                                                      \
-                return fail("gemm: reduction batching needs r-contiguous operands");  \
-        }                                                                             \
-        return gemm_fast_go<BM, BN, WGM, WGN, LA_, LB_, false>(g, s);                 \
+#define THGPU_CASE(LA_, LB_)                                                           \
+    if (la == LA_ && lb == LB_) {                                                      \
+        if constexpr ((LA_ == LD_XC_SCALAR && (WGM * WGN * 64) % BM != 0) ||           \
+                      (LB_ == LD_XC_SCALAR && (WGM * WGN * 64) % BN != 0)) {           \
+            return fail("gemm: this tile has no x-contiguous loader for that side");   \
+        } else {                                                                       \
+            if (red) {                                                                 \
+                if constexpr (LA_ != LD_XC_SCALAR && LB_ != LD_XC_SCALAR)              \
+                    return gemm_fast_go<BM, BN, WGM, WGN, LA_, LB_, true>(g, s);       \
+                else                                                                   \
+                    return fail("gemm: reduction batching needs r-contiguous operands"); \
+            }                                                                          \
+            return gemm_fast_go<BM, BN, WGM, WGN, LA_, LB_, false>(g, s);              \
+        }                                                                              \
     }
     THGPU_CASE(LD_RC_VEC, LD_RC_VEC)
     THGPU_CASE(LD_RC_VEC, LD_RC_SCALAR)

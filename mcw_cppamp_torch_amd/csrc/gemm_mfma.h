@@ -89,6 +89,7 @@ enum Loader {
 // Launch one tile configuration of the fast kernel (gemm_fast.h).  la/lb are
 // Loader values; returns 0 or a recorded error.
 int gemm_fast_128x128(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
+int gemm_fast_192x128(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
 int gemm_fast_128x256(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
 int gemm_fast_256x128(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
 int gemm_fast_64x64(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);

@@ -244,6 +244,52 @@ def test_blas_gemm_integer_exact_beta0_ignores_nan_and_quick_returns(gt):
     assert np.array_equal(dc.float(), before * 3.0)
 
 
+GEMM_TILES = ["128x128", "192x128", "64x256", "128x256", "256x128", "64x64"]
+
+
+@pytest.mark.parametrize("split", [1, 3])
+@pytest.mark.parametrize("ta,tb", list(itertools.product("nt", "nt")))
+@pytest.mark.parametrize("tile", GEMM_TILES)
+def test_blas_gemm_every_tile_configuration_exact(gt, tile, ta, tb, split, monkeypatch):
+    """Every tile configuration of the fast kernel is forced in turn on a ragged problem (edge tiles shifted back in
+    both directions, a partial last reduction step) with small integers, where any summation order is exact.  The
+    profiler label tells which kernel ran: a configuration without a loader for the operand layout at hand must
+    have gone to the bounds-checked kernel, never to another fast tile."""
+    monkeypatch.setenv("THGPU_GEMM_TILE", tile)
+    monkeypatch.setenv("THGPU_GEMM_SPLIT", str(split))
+    rng = rng_for(43)
+    m, n, k = 300, 421, 601
+    lda = (m if ta == "n" else k) + 1
+    ldb = (k if tb == "n" else n) + 3
+    ldc = m + 2
+    a = rng.integers(-3, 4, size=(lda * (k if ta == "n" else m),)).astype(np.float32)
+    b = rng.integers(-3, 4, size=(ldb * (n if tb == "n" else k),)).astype(np.float32)
+    c0 = rng.integers(-3, 4, size=(ldc * n,)).astype(np.float32)
+    A = a.reshape(-1, lda)[:, :(m if ta == "n" else k)].astype(np.int64)      # column-major: [col][row]
+    Bm = b.reshape(-1, ldb)[:, :(k if tb == "n" else n)].astype(np.int64)
+    opA = A.T if ta == "n" else A                                              # m x k
+    opB = Bm.T if tb == "n" else Bm                                            # k x n
+    ref = c0.reshape(n, ldc).copy()
+    ref[:, :m] = (2 * (opA @ opB).T + 3 * ref[:, :m].astype(np.int64)).astype(np.float32)
+    da, db, dc = dev(gt, a), dev(gt, b), dev(gt, c0)
+    gt.gputorch.synchronize()
+    gt.gputorch.prof_reset()
+    gt.gputorch.prof_enable(True)
+    try:
+        gt.gputorch.gemm(ta, tb, m, n, k, 2.0, da, lda, db, ldb, 3.0, dc, ldc)
+        gt.gputorch.synchronize()
+        labels = [key for key in gt.gputorch.prof_report() if "tile=" in key]
+    finally:
+        gt.gputorch.prof_enable(False)
+        gt.gputorch.prof_reset()
+    assert np.array_equal(dc.float().reshape(n, ldc), ref)
+    assert len(labels) == 1
+    ran = labels[0].split("tile=")[1].split(" ")[0]
+    # the 192x128 tile only loads a first operand that is contiguous along the reduction index: op(B) = B here
+    assert ran == (tile if tile != "192x128" or tb == "n" else "generic"), labels
+    assert ("split=%d" % split) in labels[0] or ran == "generic", labels
+
+
 POOLS = [(2, 3, 7, 7, 3, 3, 2, 2), (3, 2, 9, 8, 2, 2, 2, 2), (2, 2, 10, 11, 3, 2, 1, 3), (1, 1, 6, 6, 4, 4, 1, 1),
          (4, 16, 55, 55, 3, 3, 2, 2), (2, 8, 13, 13, 3, 3, 2, 2), (2, 4, 24, 24, 2, 2, 2, 2),
          (2, 3, 11, 12, 2, 2, 3, 3),       # windows smaller than the stride: uncovered pixels
