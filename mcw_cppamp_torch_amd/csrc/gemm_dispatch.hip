@@ -52,18 +52,20 @@ struct TileCfg {
     int resident;  // workgroups that fit a CU at once (registers / LDS)
     // Fraction of the MFMA rate the inner loop sustains with a full CU, by operand layout (measured
     // on the AlexNet layer shapes): [0] A along r, B along j (forward); [1] both along their free
-    // index (gradInput); [2] both along r (gradWeight); [3] A along i, B along r.
+    // index (gradInput); [2] both along r (gradWeight); [3] A along i, B along r.  The figures are fitted to
+    // measured launch times together with kOcc below, so a two-resident tile that loses nothing to its
+    // lower occupancy carries a figure above 1.
     double eff[4];
     bool a_xc;  // has a loader for a first operand that is contiguous along i
     int (*launch)(const GemmArgs &, int, int, bool, hipStream_t);
 };
 
 const TileCfg kCfgs[] = {
-    {"128x128", 128, 128, 4, {0.90, 0.90, 0.86, 0.86}, true, gemm_fast_128x128},
+    {"128x128", 128, 128, 4, {0.90, 0.90, 0.88, 0.86}, true, gemm_fast_128x128},
     {"192x128", 192, 128, 3, {0.90, 0.0, 0.90, 0.0}, false, gemm_fast_192x128},
     {"64x256", 64, 256, 3, {0.76, 0.74, 0.90, 0.74}, true, gemm_fast_64x256},
-    {"128x256", 128, 256, 2, {0.85, 0.87, 0.90, 0.85}, true, gemm_fast_128x256},
-    {"256x128", 256, 128, 2, {0.90, 0.75, 0.90, 0.75}, true, gemm_fast_256x128},
+    {"128x256", 128, 256, 2, {0.85, 0.87, 1.06, 0.85}, true, gemm_fast_128x256},
+    {"256x128", 256, 128, 2, {0.90, 0.75, 1.06, 0.75}, true, gemm_fast_256x128},
     {"64x64", 64, 64, 4, {0.68, 0.60, 0.74, 0.60}, true, gemm_fast_64x64},
 };
 

@@ -12,12 +12,16 @@
 //     is zeroed on its way to LDS.  Needs M >= BM, J >= BN, R >= 16; smaller
 //     problems take the bounds-checked generic kernel.
 //   * LDS holds both operand tiles as [x][r] (x the free index, r the
-//     reduction index, 16 + 4 floats per row).  Each lane fetches its MFMA
-//     operands with 128-bit LDS reads: lane (x, h) reads r = 8h .. 8h+7, and
-//     MFMA step s takes r = s from the lower half-wave and r = 8 + s from the
-//     upper one.  A and B use the same permutation of r, so the sum over r is
-//     unchanged.  The row pitch of 20 floats makes 8 consecutive lanes hit 32
-//     distinct banks.
+//     reduction index).  Each lane fetches its MFMA operands with 128-bit LDS
+//     reads: lane (x, h) reads r = 8h .. 8h+7, and MFMA step s takes r = s from
+//     the lower half-wave and r = 8 + s from the upper one.  A and B use the
+//     same permutation of r, so the sum over r is unchanged.  The row layout
+//     follows the operand's loader, so that its 128-bit LDS writes and the
+//     operand reads are both free of bank conflicts (the LDS conflict counter
+//     reads zero for either): a tile written a column at a time (consecutive
+//     lanes = consecutive rows) has rows of 16 + 4 floats; a tile written a row
+//     at a time (four lanes per row) has rows of 16 floats whose four 16-byte
+//     quarters are stored at quarter (r/4) xor ((x/4) mod 4).
 //   * LDS is double buffered; the next tile's global loads are issued before
 //     the current tile's MFMAs and written to the other buffer afterwards: one
 //     barrier per reduction step.
@@ -29,7 +33,15 @@
 
 namespace thgpu {
 
-constexpr int LDK = GEMM_BK + 4;  // LDS row pitch in floats
+// LDS row layout by loader kind: pitch in floats, and the column at which element r of row x is stored.
+template <int KIND>
+struct LdsRow {
+    static constexpr bool kSwizzled = KIND == LD_RC_VEC;
+    static constexpr int kPitch = kSwizzled ? GEMM_BK : GEMM_BK + 4;
+    __device__ static __forceinline__ int col(int x, int r) {
+        return kSwizzled ? ((r & 3) | ((((r >> 2) ^ (x >> 2)) & 3) << 2)) : r;
+    }
+};
 
 // Four floats at a 4-byte aligned address: the hardware handles the
 // misalignment of a 128-bit global load; the type only keeps the compiler from
@@ -47,7 +59,11 @@ constexpr int gemm_min_waves() {
 
 // DBG is 0 in the library; experiments switch phases off with it (1: no global
 // fetch in the loop, 2: no LDS operand reads, 4: no LDS stores, 8: no barrier,
-// 16: epilogue stores only one value per lane).
+// 16: epilogue stores only one value per lane) or instrument the kernel (128:
+// each workgroup writes its shader-clock and wall-clock duration to g.ws; 256:
+// each wavefront accumulates the cycles it spends per step waiting for its LDS
+// operands / issuing MFMAs and loads / waiting for the loads / storing to LDS /
+// at the barrier, and writes the five sums to g.ws past the first 8 MiB).
 template <int BM, int BN, int WGM, int WGN, int LA, int LB, bool RED, int DBG = 0>
 __global__ __launch_bounds__(WGM *WGN * 64)
     __attribute__((amdgpu_waves_per_eu(gemm_min_waves<BM, BN, WGM, WGN>()))) void gemm_fast_kernel(const GemmArgs g) {
@@ -61,9 +77,16 @@ __global__ __launch_bounds__(WGM *WGN * 64)
                   "x-contiguous loaders give every thread one row/column");
     static_assert(!RED || (LA != LD_XC_SCALAR && LB != LD_XC_SCALAR), "reduction batching needs r-contiguous operands");
 
-    __shared__ __attribute__((aligned(16))) float As[2][BM][LDK];
-    __shared__ __attribute__((aligned(16))) float Bs[2][BN][LDK];
+    using RowA = LdsRow<LA>;
+    using RowB = LdsRow<LB>;
+    __shared__ __attribute__((aligned(16))) float As[2][BM][RowA::kPitch];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BN][RowB::kPitch];
 
+    long dbg_c0 = 0, dbg_w0 = 0;
+    if (DBG & 128) {
+        dbg_c0 = (long)clock64();
+        dbg_w0 = (long)wall_clock64();
+    }
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: row bases stay uniform
     const int wm = wave / WGN, wn = wave % WGN;
@@ -183,21 +206,22 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         }
     };
 
-    auto stash_one = [&](auto kind_tag, float (*tile)[LDK], int t_x, int t_r, const float *src, auto count_tag) {
+    auto stash_one = [&](auto kind_tag, auto tile, int t_x, int t_r, const float *src, auto count_tag) {
         constexpr int KIND = decltype(kind_tag)::value;
+        using Row = LdsRow<KIND>;
         constexpr int CNT = decltype(count_tag)::value;
         if (KIND == LD_RC_VEC) {
 #pragma unroll
             for (int q = 0; q < CNT / 4; ++q)
-                *reinterpret_cast<float4 *>(&tile[t_x + q * (NT / 4)][t_r]) =
+                *reinterpret_cast<float4 *>(&tile[t_x + q * (NT / 4)][Row::col(t_x + q * (NT / 4), t_r)]) =
                     make_float4(src[q * 4], src[q * 4 + 1], src[q * 4 + 2], src[q * 4 + 3]);
         } else if (KIND == LD_RC_SCALAR) {
 #pragma unroll
-            for (int q = 0; q < CNT; ++q) tile[t_x + q * (NT / 16)][t_r] = src[q];
+            for (int q = 0; q < CNT; ++q) tile[t_x + q * (NT / 16)][Row::col(t_x + q * (NT / 16), t_r)] = src[q];
         } else {
 #pragma unroll
             for (int w = 0; w < CNT / 4; ++w)
-                *reinterpret_cast<float4 *>(&tile[t_x][t_r + 4 * w]) =
+                *reinterpret_cast<float4 *>(&tile[t_x][Row::col(t_x, t_r + 4 * w)]) =
                     make_float4(src[w * 4], src[w * 4 + 1], src[w * 4 + 2], src[w * 4 + 3]);
         }
     };
@@ -209,16 +233,6 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         stash_one(std::integral_constant<int, LA>{}, As[buf], a_x, a_r, ra, std::integral_constant<int, NA>{});
         stash_one(std::integral_constant<int, LB>{}, Bs[buf], b_x, b_r, rb, std::integral_constant<int, NB>{});
     };
-
-    if (DBG & 32) {
-        // experiment: stagger the first generation of workgroups
-        if (blockIdx.x < 1024u) {
-            const unsigned phase = (blockIdx.x * 2654435761u >> 13) & 3u;
-            const long wait = (long)phase * nsteps * (2048L * 4 / 4);
-            const long t0 = (long)__builtin_readcyclecounter();
-            while ((long)__builtin_readcyclecounter() - t0 < wait) __builtin_amdgcn_s_sleep(32);
-        }
-    }
 
     // ---- prologue: first step ---------------------------------------------------------
     const char *ga = tileA, *gb = tileB;
@@ -239,6 +253,14 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     // in slices between its MFMAs (a steady trickle of requests; a burst at the
     // head of the step would hold the wavefront, and with it its MFMAs, in the
     // memory pipeline's queue) and written to the other buffer afterwards.
+    long ph[5] = {0, 0, 0, 0, 0};
+    long tprev = (DBG & 256) ? (long)__builtin_readcyclecounter() : 0;
+#define THGPU_PHASE(k)                                        \
+    if (DBG & 256) {                                          \
+        const long tn = (long)__builtin_readcyclecounter();   \
+        ph[k] += tn - tprev;                                  \
+        tprev = tn;                                           \
+    }
     for (int s = 0; s < nsteps; ++s) {
         const int buf = s & 1;
         const bool more = !(DBG & 1) && s + 1 < nsteps;
@@ -258,10 +280,16 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         for (int h2 = 0; h2 < 2 && !(DBG & 2); ++h2) {
 #pragma unroll
             for (int a = 0; a < TM; ++a)
-                av[a][h2] = *reinterpret_cast<const float4 *>(&As[buf][wm * (TM * 32) + a * 32 + l32][8 * half + 4 * h2]);
+                av[a][h2] = *reinterpret_cast<const float4 *>(
+                    &As[buf][wm * (TM * 32) + a * 32 + l32][RowA::col(l32, 8 * half + 4 * h2)]);
 #pragma unroll
             for (int b = 0; b < TN; ++b)
-                bv[b][h2] = *reinterpret_cast<const float4 *>(&Bs[buf][wn * (TN * 32) + b * 32 + l32][8 * half + 4 * h2]);
+                bv[b][h2] = *reinterpret_cast<const float4 *>(
+                    &Bs[buf][wn * (TN * 32) + b * 32 + l32][RowB::col(l32, 8 * half + 4 * h2)]);
+        }
+        if (DBG & 256) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            THGPU_PHASE(0)  // LDS operand reads
         }
 #pragma unroll
         for (int h2 = 0; h2 < 2; ++h2) {
@@ -292,11 +320,28 @@ __global__ __launch_bounds__(WGM *WGN * 64)
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        THGPU_PHASE(1)  // MFMA and load issue
+        if (DBG & 256) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            THGPU_PHASE(2)  // waiting for the loads
+        }
         if (more) {
             if (!(DBG & 4)) stash(buf ^ 1, shift);
             advance();
         }
+        if (DBG & 256) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            THGPU_PHASE(3)  // stash
+        }
         if (!(DBG & 8)) __syncthreads();
+        THGPU_PHASE(4)  // barrier
+    }
+#undef THGPU_PHASE
+    if (DBG & 256) {
+        if (lane == 0) {
+            long *o = reinterpret_cast<long *>(g.ws) + (1L << 20) + ((long)blockIdx.x * 4 + wave) * 5;
+            for (int k = 0; k < 5; ++k) o[k] = ph[k];
+        }
     }
 
     // ---- epilogue ----------------------------------------------------------------------
@@ -353,6 +398,12 @@ __global__ __launch_bounds__(WGM *WGN * 64)
             }
         }
     };
+    if (DBG & 128) {
+        if (tid == 0) {
+            reinterpret_cast<long *>(g.ws)[2 * blockIdx.x] = (long)clock64() - dbg_c0;
+            reinterpret_cast<long *>(g.ws)[2 * blockIdx.x + 1] = (long)wall_clock64() - dbg_w0;
+        }
+    }
     using std::integral_constant;
     if (g.nsplit > 1) {
         if (rows_shifted) write_out(integral_constant<int, 0>{}, integral_constant<bool, true>{});
