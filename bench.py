@@ -15,6 +15,7 @@ Beside the throughput the line carries
   kernels       the same for every kernel family (HBM-bound ones in GB/s);
   gemm_shapes   every GEMM of the stack on its own (shape, chosen tile and split,
                 TFLOP/s): the small-K GEMMs of first layers are HBM-bound themselves;
+  hbm_shapes    every im2col / col2im / pooling launch geometry on its own (GB/s);
   cpu_baseline  the CPU oracle (a port of the reference CPU nn path, OpenMP over
                 the batch + an optimised BLAS sgemm where one is found) timed
                 on this host on a reduced batch of the same stack.
@@ -163,7 +164,7 @@ def main():
     d2h_ms = (time.perf_counter() - t1) * 1e3
 
     w = stacks.work(name, B)
-    kernels, roofline, gemm_shapes = {}, None, []
+    kernels, roofline, gemm_shapes, hbm_shapes = {}, None, [], []
     if not args.no_kernel_timing:
         gputorch.prof_reset()
         gputorch.prof_enable(True)
@@ -193,16 +194,26 @@ def main():
                 g_fl += fl
                 g_calls += r["calls"]
                 continue
-            ent = {"launches_per_step": r["calls"] / args.steps, "ms_per_step": round(ms, 4)}
-            if r["bytes"] > 0:
+            # HBM-bound kernels: im2col / col2im / pooling records carry their geometry after the family name
+            ent = kernels.setdefault(family, {"launches_per_step": 0.0, "ms_per_step": 0.0, "bytes_per_step": 0.0})
+            ent["launches_per_step"] += r["calls"] / args.steps
+            ent["ms_per_step"] += ms
+            ent["bytes_per_step"] += r["bytes"] / args.steps
+            if family != kname and r["bytes"] > 0:
                 by = r["bytes"] / args.steps
-                ent.update(bound="hbm", gbs=round(by / ms / 1e6, 1), frac=round(by / ms / 1e6 / PEAK_HBM_GBS, 4))
-            kernels[kname] = ent
+                hbm_shapes.append({"kernel": kname, "launches_per_step": r["calls"] / args.steps,
+                                   "ms_per_step": round(ms, 4), "gbs": round(by / ms / 1e6, 1),
+                                   "frac": round(by / ms / 1e6 / PEAK_HBM_GBS, 4)})
         for ent in kernels.values():
             if ent.get("bound") == "mfma":
                 fl, ms = ent.pop("flops_per_step"), ent["ms_per_step"]
                 ent.update(ms_per_step=round(ms, 4), tflops=round(fl / ms / 1e9, 2),
                            frac=round(fl / ms / 1e9 / PEAK_MFMA_F32_TFLOPS, 4))
+            else:
+                by, ms = ent.pop("bytes_per_step"), ent["ms_per_step"]
+                ent["ms_per_step"] = round(ms, 4)
+                if by > 0:
+                    ent.update(bound="hbm", gbs=round(by / ms / 1e6, 1), frac=round(by / ms / 1e6 / PEAK_HBM_GBS, 4))
         if g_ms > 0:
             roofline = {
                 "bound": "mfma", "kernel": "gemm_fast_kernel<...> (all conv GEMM launches of a step)",
@@ -229,6 +240,7 @@ def main():
                       "images_per_s_including_transfers": round(B / ((ms_per_step + h2d_ms + d2h_ms) / 1e3), 1)},
         "gemm_tflops_over_whole_step": round(w["gemm_flops"] / (ms_per_step / 1e3) / 1e12, 2),
         "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels, "gemm_shapes": gemm_shapes,
+        "hbm_shapes": hbm_shapes,
     }
     print(json.dumps(line))
 

@@ -48,6 +48,13 @@ struct ConvGeom {
     FastDiv divW, divHW, divSH, divSW, divH;  // col2im decomposition
 };
 
+// Timing label: the kernel family alone, or with the layer geometry while per-kernel timing is on.
+inline const char *geom_label(const char *family, const ConvGeom &g, long B) {
+    if (!prof_enabled()) return family;
+    return prof_label("%s B=%ld C=%d %dx%d k=%dx%d s=%dx%d p=%dx%d", family, B, g.C, g.H, g.W, g.kH, g.kW, g.sH, g.sW, g.pH,
+                      g.pW);
+}
+
 // Four floats at a 4-byte aligned address (the hardware handles the
 // misalignment; the type only tells the compiler not to assume 16 bytes).
 struct __attribute__((packed, aligned(4))) float4u {
@@ -583,7 +590,7 @@ int im2col_launch(const float *im, long B, int C, int H, int W, int kH, int kW, 
         const long positions = planes * g.N;
         const unsigned blocks = (unsigned)((positions + 255) / 256);
         {
-            LaunchScope scope("im2col", 0.0, bytes);
+            LaunchScope scope(geom_label("im2col", g, B), 0.0, bytes);
             if (kH == 3)
                 hipLaunchKernelGGL((im2col_unit_kernel<3, 3>), dim3(blocks), dim3(256), 0, s, im, col, g,
                                    (unsigned)positions);
@@ -599,7 +606,7 @@ int im2col_launch(const float *im, long B, int C, int H, int W, int kH, int kW, 
         if (blocks < (1L << 31) && planes < (1L << 31)) {
             const size_t lds = sizeof(float) * (size_t)plan.G * plan.LH * plan.LW;
             {
-                LaunchScope scope("im2col", 0.0, bytes);
+                LaunchScope scope(geom_label("im2col", g, B), 0.0, bytes);
                 const long positions = (long)plan.G * plan.TR * g.Wo;
                 const long slots = (positions + plan.PL - 1) / plan.PL;
                 const dim3 grid((unsigned)blocks), block(plan.PL * plan.TG);
@@ -625,7 +632,7 @@ int im2col_launch(const float *im, long B, int C, int H, int W, int kH, int kW, 
             const long nthr = threads - t0 < max_threads ? threads - t0 : max_threads;
             const unsigned blocks = (unsigned)((nthr + 255) / 256);
             {
-                LaunchScope scope("im2col", 0.0, bytes * ((double)nthr / threads));
+                LaunchScope scope(geom_label("im2col", g, B), 0.0, bytes * ((double)nthr / threads));
                 if (vec)
                     hipLaunchKernelGGL(im2col_flat_kernel<true>, dim3(blocks), dim3(256), 0, s, im, col, g, total,
                                        t0 * 4);
@@ -647,7 +654,7 @@ int im2col_launch(const float *im, long B, int C, int H, int W, int kH, int kW, 
         const float *im0 = im + (p0 / kH) * (long)H * W;
         float *col0 = col + p0 * (long)kW * g.N;
         {
-            LaunchScope scope("im2col", 0.0, bytes * ((double)np / prows));
+            LaunchScope scope(geom_label("im2col", g, B), 0.0, bytes * ((double)np / prows));
             hipLaunchKernelGGL(im2col_tapvec_kernel, dim3(blocks), dim3(256), 0, s, im0, col0, g, threads);
         }
         if (check_launch("im2col")) return 1;
@@ -710,7 +717,7 @@ int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW,
     if (!(generic && generic[0] == '1') && sH == 1 && sW == 1 && kH == kW && (kH == 3 || kH == 5) &&
         span_planes * kH * kW * g.N * 4 < (1L << 32) && total < (1L << 32)) {
         {
-            LaunchScope scope("col2im", 0.0, bytes);
+            LaunchScope scope(geom_label("col2im", g, B), 0.0, bytes);
             if (kH == 3)
                 hipLaunchKernelGGL((col2im_unit_kernel<3, 3>), dim3((unsigned)blocks), dim3(256), 0, s, col, im, g,
                                    (unsigned)total);
@@ -735,7 +742,7 @@ int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW,
             const int lanes = (R * Qw + 63) / 64 * 64;
             const dim3 grid((unsigned)wgs), block(lanes < 256 ? lanes : 256);
             {
-                LaunchScope scope("col2im", 0.0, bytes);
+                LaunchScope scope(geom_label("col2im", g, B), 0.0, bytes);
                 if (th == 3 || tw == 3)
                     hipLaunchKernelGGL((col2im_strided_kernel<3, 3>), grid, block, lds, s, col, im, g, R, Qw, qtiles,
                                        FastDiv((uint32_t)Qw), FastDiv((uint32_t)qtiles));
@@ -747,7 +754,7 @@ int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW,
         }
     }
     {
-        LaunchScope scope("col2im", 0.0, bytes);
+        LaunchScope scope(geom_label("col2im", g, B), 0.0, bytes);
         hipLaunchKernelGGL(col2im_kernel, dim3((unsigned)blocks), dim3(256), 0, s, col, im, g, total,
                            (kH + sH - 1) / sH, (kW + sW - 1) / sW);
     }

@@ -31,6 +31,12 @@ struct PoolGeom {
     FastDiv divWo, divHoWo, divW, divHW, divDH, divDW;
 };
 
+// Timing label: the kernel family alone, or with the geometry while per-kernel timing is on.
+inline const char *pool_label(const char *family, const PoolGeom &g, long planes) {
+    if (!prof_enabled()) return family;
+    return prof_label("%s planes=%ld %dx%d k=%dx%d s=%dx%d", family, planes, g.H, g.W, g.kH, g.kW, g.dH, g.dW);
+}
+
 // KH, KW > 0 fix the window at compile time (fully unrolled: all loads of a
 // window are in flight before the compare chain); 0 takes the run-time sizes.
 template <int KH, int KW>
@@ -406,7 +412,7 @@ int maxpool_fwd_launch(const float *in, long planes, int H, int W, int kH, int k
     g.divW = FastDiv((uint32_t)W);
     g.divHW = FastDiv((uint32_t)(H * W));
     {
-        LaunchScope scope("maxpool_fwd", 0.0, 4.0 * (planes * (double)H * W + 3.0 * total));
+        LaunchScope scope(pool_label("maxpool_fwd", g, planes), 0.0, 4.0 * (planes * (double)H * W + 3.0 * total));
         const dim3 grid((unsigned)((total + 255) / 256)), block(256);
         if (kH == 3 && kW == 3)
             hipLaunchKernelGGL((maxpool_fwd_kernel<3, 3>), grid, block, 0, s, in, out, indices, indices + total, g,
@@ -479,7 +485,7 @@ int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int
         if (blocks < (1L << 31)) {
             const size_t lds = sizeof(int2) * (size_t)plan.G * plan.RW * plan.CW;
             {
-                LaunchScope scope("maxpool_bwd", 0.0, bytes);
+                LaunchScope scope(pool_label("maxpool_bwd", g, planes), 0.0, bytes);
                 const dim3 grid((unsigned)blocks), block(256);
                 float *ix = const_cast<float *>(indices) + ototal;
 #define THGPU_POOL_BWD(TH_, TW_, PAIRS_)                                                                          \
@@ -495,7 +501,7 @@ int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int
         }
     }
     {
-        LaunchScope scope("maxpool_bwd", 0.0, bytes);
+        LaunchScope scope(pool_label("maxpool_bwd", g, planes), 0.0, bytes);
         const dim3 grid((unsigned)((total + 255) / 256)), block(256);
         if (th == 2 && tw == 2)
             hipLaunchKernelGGL((maxpool_bwd_kernel<2, 2>), grid, block, 0, s, gout, indices, indices + ototal, gin, g,
