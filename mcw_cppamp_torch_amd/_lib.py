@@ -184,6 +184,11 @@ _SIGNATURES = {
     "thgpu_SpatialMaxPooling_updateGradInput": (c_int, [TensorP] * 4 + [c_int] * 4),
     "thgpu_Threshold_updateOutput": (c_int, [TensorP] * 2 + [c_float] * 2),
     "thgpu_Threshold_updateGradInput": (c_int, [TensorP] * 3 + [c_float]),
+    "thgpu_SpatialAveragePooling_updateOutput": (c_int, [TensorP] * 2 + [c_int] * 4),
+    "thgpu_SpatialAveragePooling_updateGradInput": (c_int, [TensorP] * 3 + [c_int] * 4),
+    "thgpu_SpatialSubSampling_updateOutput": (c_int, [TensorP] * 4 + [c_int] * 4),
+    "thgpu_SpatialSubSampling_updateGradInput": (c_int, [TensorP] * 4 + [c_int] * 4),
+    "thgpu_SpatialSubSampling_accGradParameters": (c_int, [TensorP] * 4 + [c_int] * 4 + [c_float]),
 }
 for _k in HOST_TYPES:
     _SIGNATURES["THGPUStorage_copy%s" % _k] = (None, [StorageP, ctypes.POINTER(HostStorage[_k])])

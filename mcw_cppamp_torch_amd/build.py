@@ -21,6 +21,9 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
     # Keep the compiler from forming packed-FP32 instructions.
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # a*b + c stays two roundings, as in the CPU modules the results are compared with bit for bit (hipcc's
+    # default contracts them into fused multiply-adds, and its __fmul_rn / __fadd_rn are plain operators).
+    "-ffp-contract=off",
 ]
 
 

@@ -7,6 +7,8 @@ to the C ABI the way the Lua modules dispatch to `input.nn.<Op>_<method>`:
   nn.SpatialMaxPooling     mcw_nn/SpatialMaxPooling.lua:1-34
   nn.Threshold / nn.ReLU   mcw_nn/Threshold.lua:1-21, mcw_nn/ReLU.lua:1-5
   nn.Linear                mcw_nn/Linear.lua:1-104 (the classifier after a conv stack)
+  nn.SpatialAveragePooling mcw_nn/SpatialAveragePooling.lua:1-20
+  nn.SpatialSubSampling    mcw_nn/SpatialSubSampling.lua:1-54
 
 Same constructor arguments, field names and call order.  Modules are created
 with host tensors (numpy float32, like torch.Tensor) and moved with :gpu();
@@ -320,6 +322,72 @@ class SpatialMaxPooling(Module):
         _lib.check_status(lib.thgpu_SpatialMaxPooling_updateGradInput(
             input._p, gradOutput._p, self.gradInput._p, self.indices._p, self.kW, self.kH, self.dW, self.dH))
         return self.gradInput
+
+
+class SpatialAveragePooling(Module):
+    """nn.SpatialAveragePooling(kW, kH, dW, dH); dW, dH default to 1 (mcw_nn/SpatialAveragePooling.lua:3-20).
+    The module returns the window sum, as the reference's does."""
+
+    def __init__(self, kW, kH, dW=None, dH=None):
+        Module.__init__(self)
+        self.kW, self.kH = kW, kH
+        self.dW = dW or 1
+        self.dH = dH or 1
+
+    def updateOutput(self, input):
+        _require_gpu(input, self.output)
+        _lib.check_status(lib.thgpu_SpatialAveragePooling_updateOutput(
+            input._p, self.output._p, self.kW, self.kH, self.dW, self.dH))
+        return self.output
+
+    def updateGradInput(self, input, gradOutput):
+        _require_gpu(input, gradOutput, self.gradInput)
+        _lib.check_status(lib.thgpu_SpatialAveragePooling_updateGradInput(
+            input._p, gradOutput._p, self.gradInput._p, self.kW, self.kH, self.dW, self.dH))
+        return self.gradInput
+
+
+class SpatialSubSampling(Module):
+    """nn.SpatialSubSampling(nInputPlane, kW, kH, dW, dH); dW, dH default to 1; weight and bias drawn from
+    U(-1/sqrt(kW*kH), 1/sqrt(kW*kH)) (mcw_nn/SpatialSubSampling.lua:3-54)."""
+
+    _assign = SpatialConvolutionMM._assign
+
+    def __init__(self, nInputPlane, kW, kH, dW=None, dH=None, rng=None):
+        Module.__init__(self)
+        self.nInputPlane = nInputPlane
+        self.kW, self.kH = kW, kH
+        self.dW = dW or 1
+        self.dH = dH or 1
+        self.weight = FloatTensor(nInputPlane)
+        self.bias = FloatTensor(nInputPlane)
+        self.gradWeight = FloatTensor(nInputPlane)
+        self.gradBias = FloatTensor(nInputPlane)
+        self._rng = rng if rng is not None else np.random.default_rng()
+        self.reset()
+
+    def reset(self, stdv=None):
+        stdv = stdv * math.sqrt(3) if stdv else 1.0 / math.sqrt(self.kW * self.kH)
+        self._assign("weight", self._rng.uniform(-stdv, stdv, size=(self.nInputPlane,)))
+        self._assign("bias", self._rng.uniform(-stdv, stdv, size=(self.nInputPlane,)))
+
+    def updateOutput(self, input):
+        _require_gpu(input, self.weight, self.bias, self.output)
+        _lib.check_status(lib.thgpu_SpatialSubSampling_updateOutput(
+            input._p, self.weight._p, self.bias._p, self.output._p, self.kW, self.kH, self.dW, self.dH))
+        return self.output
+
+    def updateGradInput(self, input, gradOutput):
+        _require_gpu(input, gradOutput, self.weight, self.gradInput)
+        _lib.check_status(lib.thgpu_SpatialSubSampling_updateGradInput(
+            input._p, gradOutput._p, self.weight._p, self.gradInput._p, self.kW, self.kH, self.dW, self.dH))
+        return self.gradInput
+
+    def accGradParameters(self, input, gradOutput, scale=1.0):
+        _require_gpu(input, gradOutput, self.gradWeight, self.gradBias)
+        _lib.check_status(lib.thgpu_SpatialSubSampling_accGradParameters(
+            input._p, gradOutput._p, self.gradWeight._p, self.gradBias._p, self.kW, self.kH, self.dW, self.dH,
+            float(scale)))
 
 
 class Threshold(Module):

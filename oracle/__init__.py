@@ -30,9 +30,17 @@ def build(force=False):
     return _LIB_PATH
 
 
+def _stale():
+    """True when oracle.c was edited after liboracle.so was built."""
+    src = os.path.join(_HERE, "oracle.c")
+    return os.path.exists(src) and os.path.getmtime(src) > os.path.getmtime(_LIB_PATH)
+
+
 def _load():
     if not os.path.exists(_LIB_PATH):
         build()
+    elif _stale():
+        build(force=True)
     lib = ctypes.CDLL(_LIB_PATH)
     ints = lambda n: [_c_int] * n
     lib.oracle_set_blas.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
@@ -51,6 +59,9 @@ def _load():
                                                   _f32p, _f32p]
     lib.oracle_maxpool_updateOutput.argtypes = [_f32p, _c_long] + ints(7) + [_f32p, _f32p]
     lib.oracle_maxpool_updateGradInput.argtypes = [_f32p, _f32p, _c_long] + ints(7) + [_f32p]
+    lib.oracle_subsample_updateOutput.argtypes = [_f32p, _f32p, _f32p, _c_long] + ints(7) + [_f32p]
+    lib.oracle_subsample_updateGradInput.argtypes = [_f32p, _f32p, _c_long] + ints(7) + [_f32p]
+    lib.oracle_subsample_accGradParameters.argtypes = [_f32p, _f32p, _c_long] + ints(7) + [_c_float, _f32p, _f32p]
     lib.oracle_threshold_updateOutput.argtypes = [_f32p, _c_long, _c_float, _c_float, _f32p]
     lib.oracle_threshold_updateGradInput.argtypes = [_f32p, _f32p, _c_long, _c_float, _f32p]
     return lib
@@ -258,6 +269,38 @@ def maxpool_updateGradInput(gradOutput, indices, in_shape, dH, dW):
     gi = np.empty((B, C, H, W), np.float32)
     _lib.oracle_maxpool_updateGradInput(_p(gradOutput), _p(indices), B, C, H, W, Ho, Wo, dH, dW, _p(gi))
     return gi
+
+
+def subsample_updateOutput(inp, weight, bias, kH, kW, dH, dW):
+    """nn.SpatialSubSampling forward; weight=None gives nn.SpatialAveragePooling (a window sum)."""
+    inp = _f32(inp)
+    B, C, H, W = inp.shape
+    Ho, Wo = (H - kH) // dH + 1, (W - kW) // dW + 1
+    out = np.empty((B, C, Ho, Wo), np.float32)
+    w = None if weight is None else _f32(weight)
+    b = None if weight is None else _f32(bias)
+    _lib.oracle_subsample_updateOutput(_p(inp), None if w is None else _p(w), None if b is None else _p(b),
+                                       B, C, H, W, kH, kW, dH, dW, _p(out))
+    return out
+
+
+def subsample_updateGradInput(gradOutput, weight, in_shape, kH, kW, dH, dW):
+    gradOutput = _f32(gradOutput)
+    B, C, H, W = in_shape
+    gi = np.empty((B, C, H, W), np.float32)
+    w = None if weight is None else _f32(weight)
+    _lib.oracle_subsample_updateGradInput(_p(gradOutput), None if w is None else _p(w), B, C, H, W, kH, kW, dH, dW,
+                                          _p(gi))
+    return gi
+
+
+def subsample_accGradParameters(inp, gradOutput, gradWeight, gradBias, kH, kW, dH, dW, scale=1.0):
+    """Accumulates into gradWeight / gradBias (float32 vectors of C elements) in place."""
+    inp, gradOutput = _f32(inp), _f32(gradOutput)
+    B, C, H, W = inp.shape
+    assert gradWeight.dtype == np.float32 and gradBias.dtype == np.float32
+    _lib.oracle_subsample_accGradParameters(_p(inp), _p(gradOutput), B, C, H, W, kH, kW, dH, dW, scale,
+                                            _p(gradWeight), _p(gradBias))
 
 
 def threshold_updateOutput(inp, threshold=0.0, val=0.0):

@@ -393,6 +393,99 @@ void oracle_maxpool_updateGradInput(const float *gradOutput, const float *indice
 }
 
 /* ------------------------------------------------------------------------- */
+/* nn.SpatialSubSampling and nn.SpatialAveragePooling.
+ * forward: mcw_nn/generic/SpatialSubSampling.c:48-96 -- the output plane is
+ * filled with bias[k] (:66-69), then every window adds weight[k] * sum, the sum
+ * taken ky ascending, kx ascending from zero (:78-89).  SpatialAveragePooling
+ * (mcw_nn/generic/SpatialAveragePooling.c:54-92) is the same loop with a zero
+ * fill and no weight: it returns the window SUM, there is no division.
+ * weight == NULL selects the average-pooling form. */
+void oracle_subsample_updateOutput(const float *input, const float *weight, const float *bias, long B, int C,
+                                   int H, int W, int kH, int kW, int dH, int dW, float *output)
+{
+    int Ho = (H - kH) / dH + 1, Wo = (W - kW) / dW + 1;
+    long planes = B * C, p;
+#pragma omp parallel for num_threads(nthreads())
+    for (p = 0; p < planes; p++) {
+        int k = (int)(p % C), yy, xx, ky, kx;
+        const float *ip = input + p * (long)H * W;
+        float *op = output + p * (long)Ho * Wo;
+        float z = weight ? bias[k] : 0.0f;
+        for (yy = 0; yy < Ho * Wo; yy++) op[yy] = z;
+        for (yy = 0; yy < Ho; yy++)
+            for (xx = 0; xx < Wo; xx++) {
+                const float *win = ip + (long)yy * dH * W + (long)xx * dW;
+                float sum = 0;
+                for (ky = 0; ky < kH; ky++) {
+                    for (kx = 0; kx < kW; kx++) sum += win[kx];
+                    win += W;
+                }
+                if (weight) *op++ += weight[k] * sum;
+                else *op++ += sum;
+            }
+    }
+}
+
+/* backward: SpatialSubSampling.c:150-178 / SpatialAveragePooling.c:148-174 --
+ * gradInput is zeroed, then every window (yy ascending, xx ascending) adds
+ * z = gradOutput * weight[k] (or gradOutput alone) to each of its pixels. */
+void oracle_subsample_updateGradInput(const float *gradOutput, const float *weight, long B, int C, int H, int W,
+                                      int kH, int kW, int dH, int dW, float *gradInput)
+{
+    int Ho = (H - kH) / dH + 1, Wo = (W - kW) / dW + 1;
+    long planes = B * C, p;
+#pragma omp parallel for num_threads(nthreads())
+    for (p = 0; p < planes; p++) {
+        int k = (int)(p % C), yy, xx, ky, kx;
+        float *gi = gradInput + p * (long)H * W;
+        const float *go = gradOutput + p * (long)Ho * Wo;
+        for (yy = 0; yy < H * W; yy++) gi[yy] = 0.0f;
+        for (yy = 0; yy < Ho; yy++)
+            for (xx = 0; xx < Wo; xx++) {
+                float *win = gi + (long)yy * dH * W + (long)xx * dW;
+                float z = weight ? *go++ * weight[k] : *go++;
+                for (ky = 0; ky < kH; ky++) {
+                    for (kx = 0; kx < kW; kx++) win[kx] += z;
+                    win += W;
+                }
+            }
+    }
+}
+
+/* accGradParameters: SpatialSubSampling.c:236-264 -- per plane, image after
+ * image: gradBias[k] += scale * (sum of the gradOutput plane), gradWeight[k] +=
+ * scale * (sum over windows and taps of gradOutput * input), all in float. */
+void oracle_subsample_accGradParameters(const float *input, const float *gradOutput, long B, int C, int H, int W,
+                                        int kH, int kW, int dH, int dW, float scale, float *gradWeight,
+                                        float *gradBias)
+{
+    int Ho = (H - kH) / dH + 1, Wo = (W - kW) / dW + 1, k;
+#pragma omp parallel for num_threads(nthreads())
+    for (k = 0; k < C; k++) {
+        long b;
+        for (b = 0; b < B; b++) {
+            const float *go = gradOutput + (b * C + k) * (long)Ho * Wo;
+            const float *ip = input + (b * C + k) * (long)H * W;
+            float sum = 0;
+            int i, yy, xx, ky, kx;
+            for (i = 0; i < Ho * Wo; i++) sum += go[i];
+            gradBias[k] += scale * sum;
+            sum = 0;
+            for (yy = 0; yy < Ho; yy++)
+                for (xx = 0; xx < Wo; xx++) {
+                    const float *win = ip + (long)yy * dH * W + (long)xx * dW;
+                    float z = *go++;
+                    for (ky = 0; ky < kH; ky++) {
+                        for (kx = 0; kx < kW; kx++) sum += z * win[kx];
+                        win += W;
+                    }
+                }
+            gradWeight[k] += scale * sum;
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------- */
 /* nn.Threshold (nn.ReLU = Threshold(0,0), mcw_nn/ReLU.lua:1-5):
  * mcw_nn/generic/Threshold.c:5-32.  forward: x > threshold ? x : val;
  * backward uses the forward INPUT: x > threshold ? gradOutput : 0. */
