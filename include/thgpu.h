@@ -374,8 +374,8 @@ int thgpu_Threshold_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput,
                                     float threshold);
 
 /* nn.SpatialAveragePooling.  Replace gpunn_SpatialAveragePooling_updateOutput /
- * _updateGradInput (gpunn-impl/SpatialAveragePooling.cpp:68-133, 135-236; CPU twin
- * mcw_nn/generic/SpatialAveragePooling.c:5-96, 98-176).  Despite the name the
+ * _updateGradInput (gpunn-impl/SpatialAveragePooling.cpp:67-124, 185-233; CPU twin
+ * mcw_nn/generic/SpatialAveragePooling.c:5-94, 96-174).  Despite the name the
  * module returns the window SUM (neither implementation divides).  No padding,
  * Ho = (H - kH) / dH + 1.  Results are bit-identical to the CPU module's;
  * backward accepts overlapping windows (the reference GPU code requires
@@ -386,9 +386,9 @@ int thgpu_SpatialAveragePooling_updateGradInput(THGPUTensor *input, THGPUTensor 
 
 /* nn.SpatialSubSampling: output = bias[k] + weight[k] * sum(window), one weight
  * and one bias per plane.  Replace gpunn_SpatialSubSampling_updateOutput /
- * _updateGradInput / _accGradParameters (gpunn-impl/SpatialSubSampling.cpp:243-311,
- * 313-374, 376-440; CPU twin mcw_nn/generic/SpatialSubSampling.c:5-100, 102-180,
- * 182-268).  weight, bias, gradWeight, gradBias: contiguous vectors of
+ * _updateGradInput / _accGradParameters (gpunn-impl/SpatialSubSampling.cpp:246-317,
+ * 319-373, 375-440; CPU twin mcw_nn/generic/SpatialSubSampling.c:5-100, 102-185,
+ * 187-275).  weight, bias, gradWeight, gradBias: contiguous vectors of
  * nInputPlane elements.  output and gradInput are bit-identical to the CPU
  * module's; gradWeight and gradBias are deterministic and agree to rounding. */
 int thgpu_SpatialSubSampling_updateOutput(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias,

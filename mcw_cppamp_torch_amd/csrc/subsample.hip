@@ -2,19 +2,19 @@
 //
 // Both walk kH x kW windows with strides dH x dW and no padding, Ho = (H - kH) / dH + 1.
 //   SpatialAveragePooling  out = 0 + sum(window)            -- a window SUM: neither the CPU module
-//                          (mcw_nn/generic/SpatialAveragePooling.c:58-90) nor the GPU one
-//                          (gpunn-impl/SpatialAveragePooling.cpp:45-62) divides by the window size
+//                          (mcw_nn/generic/SpatialAveragePooling.c:56-90) nor the GPU one
+//                          (gpunn-impl/SpatialAveragePooling.cpp:46-61) divides by the window size
 //   SpatialSubSampling     out = bias[k] + weight[k] * sum(window), one weight and bias per plane
-//                          (mcw_nn/generic/SpatialSubSampling.c:60-94)
+//                          (mcw_nn/generic/SpatialSubSampling.c:58-96)
 // The window sum is taken ky ascending, kx ascending into a float that starts at zero, as the CPU
 // loops do, and product and sum are rounded separately, so the forward results are bit-identical
 // to the CPU modules'.  The backward pass is a gather: a thread owns one input pixel and adds the
 // gradients of the windows that cover it in the order the CPU's scatter reaches that pixel (window
 // row ascending, window column ascending, starting from the zero fill;
-// SpatialAveragePooling.c:150-174, SpatialSubSampling.c:150-176) -- bit-identical again, with
+// SpatialAveragePooling.c:151-170, SpatialSubSampling.c:161-180) -- bit-identical again, with
 // overlapping windows allowed (the reference GPU code insists on dW == kW, dH == kH:
 // SpatialAveragePooling.cpp:194-195, SpatialSubSampling.cpp:329-330) and without atomics.
-// accGradParameters (SpatialSubSampling.c:236-262) sums whole planes; the per-image sums are block
+// accGradParameters (SpatialSubSampling.c:236-270) sums whole planes; the per-image sums are block
 // reductions in a fixed order and the images are then added one after another as on the CPU, so the
 // result is deterministic and agrees with the CPU to rounding.
 #include "common.h"
@@ -148,7 +148,7 @@ struct SubShape {
     bool batched;
 };
 
-// Argument checks with the reference's messages (SpatialSubSampling.c:32-47, SpatialAveragePooling.c:33-50).
+// Argument checks with the reference's messages (SpatialSubSampling.c:34-48, SpatialAveragePooling.c:31-46).
 int sub_shape(const char *name, SubShape &s, SubGeom &g, const THGPUTensor *input, int kW, int kH, int dW, int dH) {
     if (!input) return fail("%s: null tensor", name);
     if (!(input->nDimension == 3 || input->nDimension == 4)) return fail("3D or 4D(batch mode) tensor expected");

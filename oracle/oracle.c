@@ -394,10 +394,10 @@ void oracle_maxpool_updateGradInput(const float *gradOutput, const float *indice
 
 /* ------------------------------------------------------------------------- */
 /* nn.SpatialSubSampling and nn.SpatialAveragePooling.
- * forward: mcw_nn/generic/SpatialSubSampling.c:48-96 -- the output plane is
- * filled with bias[k] (:66-69), then every window adds weight[k] * sum, the sum
- * taken ky ascending, kx ascending from zero (:78-89).  SpatialAveragePooling
- * (mcw_nn/generic/SpatialAveragePooling.c:54-92) is the same loop with a zero
+ * forward: mcw_nn/generic/SpatialSubSampling.c:58-96 -- the output plane is
+ * filled with bias[k] (:70-74), then every window adds weight[k] * sum, the sum
+ * taken ky ascending, kx ascending from zero (:82-92).  SpatialAveragePooling
+ * (mcw_nn/generic/SpatialAveragePooling.c:56-90) is the same loop with a zero
  * fill and no weight: it returns the window SUM, there is no division.
  * weight == NULL selects the average-pooling form. */
 void oracle_subsample_updateOutput(const float *input, const float *weight, const float *bias, long B, int C,
@@ -426,7 +426,7 @@ void oracle_subsample_updateOutput(const float *input, const float *weight, cons
     }
 }
 
-/* backward: SpatialSubSampling.c:150-178 / SpatialAveragePooling.c:148-174 --
+/* backward: SpatialSubSampling.c:151-181 / SpatialAveragePooling.c:142-171 --
  * gradInput is zeroed, then every window (yy ascending, xx ascending) adds
  * z = gradOutput * weight[k] (or gradOutput alone) to each of its pixels. */
 void oracle_subsample_updateGradInput(const float *gradOutput, const float *weight, long B, int C, int H, int W,
@@ -452,7 +452,7 @@ void oracle_subsample_updateGradInput(const float *gradOutput, const float *weig
     }
 }
 
-/* accGradParameters: SpatialSubSampling.c:236-264 -- per plane, image after
+/* accGradParameters: SpatialSubSampling.c:236-270 -- per plane, image after
  * image: gradBias[k] += scale * (sum of the gradOutput plane), gradWeight[k] +=
  * scale * (sum over windows and taps of gradOutput * input), all in float. */
 void oracle_subsample_accGradParameters(const float *input, const float *gradOutput, long B, int C, int H, int W,

@@ -1,10 +1,10 @@
 """Pins the oracle's nn.SpatialSubSampling / nn.SpatialAveragePooling restatements (CPU only).
 
 What pins them: a brute-force restatement written from the loop structure of
-mcw_nn/generic/SpatialSubSampling.c:48-96,150-178,236-264 in pure Python (same float32 operation order, so equality is
+mcw_nn/generic/SpatialSubSampling.c:58-96,151-181,236-270 in pure Python (same float32 operation order, so equality is
 bit-for-bit); torch's CPU avg_pool2d and grouped conv2d with autograd as an independent library routine (tolerance);
 and closed forms on integer data: a plane of ones must give kH*kW everywhere -- the reference module returns the window
-SUM, it never divides (mcw_nn/generic/SpatialAveragePooling.c:75-88).
+SUM, it never divides (mcw_nn/generic/SpatialAveragePooling.c:75-86).
 """
 import numpy as np
 import pytest
