@@ -398,6 +398,26 @@ int thgpu_SpatialSubSampling_updateGradInput(THGPUTensor *input, THGPUTensor *gr
 int thgpu_SpatialSubSampling_accGradParameters(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *gradWeight,
                                                THGPUTensor *gradBias, int kW, int kH, int dW, int dH, float scale);
 
+/* nn.LogSoftMax on a vector or a matrix of frames.  Replace gpunn_LogSoftMax_updateOutput /
+ * _updateGradInput (gpunn-impl/LogSoftMax.cpp:115-146, 148-181).  The arithmetic is the CPU
+ * module's (mcw_nn/generic/LogSoftMax.c:37-53, 85-97: double accumulation and the polynomial
+ * THExpMinusApprox of TH/THLogAdd.c:56-86 in the forward sum), so results agree with it to the
+ * rounding of the float output.  updateGradInput reads the module's output, not its input. */
+int thgpu_LogSoftMax_updateOutput(THGPUTensor *input, THGPUTensor *output);
+int thgpu_LogSoftMax_updateGradInput(THGPUTensor *gradOutput, THGPUTensor *output, THGPUTensor *gradInput);
+
+/* nn.ClassNLLCriterion without class weights.  Replace gpunn_ClassNLLCriterion_updateOutput /
+ * _updateGradInput (gpunn-impl/ClassNLLCriterion.cpp:96-135, 137-184).  target holds 1-based class
+ * numbers as floats, one per frame ([nframe] or [nframe, ntarget]); outputTensor is the module's
+ * one-element tensor and receives -(sum of input[i][target[i]-1]) [/ nframe when sizeAverage and the
+ * input is a matrix].  updateGradInput writes -1 [/ nframe] at the target positions of gradInput, which
+ * the caller has sized like the input and zeroed (mcw_nn/ClassNLLCriterion.lua:43-51).  Targets outside
+ * 1..ndim are skipped. */
+int thgpu_ClassNLLCriterion_updateOutput(THGPUTensor *input, THGPUTensor *target, THGPUTensor *outputTensor,
+                                         int sizeAverage);
+int thgpu_ClassNLLCriterion_updateGradInput(THGPUTensor *input, THGPUTensor *target, THGPUTensor *gradInput,
+                                            int sizeAverage);
+
 #ifdef __cplusplus
 }
 #endif

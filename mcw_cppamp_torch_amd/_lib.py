@@ -189,6 +189,10 @@ _SIGNATURES = {
     "thgpu_SpatialSubSampling_updateOutput": (c_int, [TensorP] * 4 + [c_int] * 4),
     "thgpu_SpatialSubSampling_updateGradInput": (c_int, [TensorP] * 4 + [c_int] * 4),
     "thgpu_SpatialSubSampling_accGradParameters": (c_int, [TensorP] * 4 + [c_int] * 4 + [c_float]),
+    "thgpu_LogSoftMax_updateOutput": (c_int, [TensorP] * 2),
+    "thgpu_LogSoftMax_updateGradInput": (c_int, [TensorP] * 3),
+    "thgpu_ClassNLLCriterion_updateOutput": (c_int, [TensorP] * 3 + [c_int]),
+    "thgpu_ClassNLLCriterion_updateGradInput": (c_int, [TensorP] * 3 + [c_int]),
 }
 for _k in HOST_TYPES:
     _SIGNATURES["THGPUStorage_copy%s" % _k] = (None, [StorageP, ctypes.POINTER(HostStorage[_k])])

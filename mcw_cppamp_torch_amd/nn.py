@@ -9,6 +9,8 @@ to the C ABI the way the Lua modules dispatch to `input.nn.<Op>_<method>`:
   nn.Linear                mcw_nn/Linear.lua:1-104 (the classifier after a conv stack)
   nn.SpatialAveragePooling mcw_nn/SpatialAveragePooling.lua:1-20
   nn.SpatialSubSampling    mcw_nn/SpatialSubSampling.lua:1-54
+  nn.LogSoftMax            mcw_nn/LogSoftMax.lua:1-9
+  nn.Criterion, nn.ClassNLLCriterion   mcw_nn/Criterion.lua:1-44, mcw_nn/ClassNLLCriterion.lua:1-72
 
 Same constructor arguments, field names and call order.  Modules are created
 with host tensors (numpy float32, like torch.Tensor) and moved with :gpu();
@@ -416,3 +418,70 @@ class Threshold(Module):
 class ReLU(Threshold):
     def __init__(self):
         Threshold.__init__(self, 0, 0)
+
+
+class LogSoftMax(Module):
+    """nn.LogSoftMax() (mcw_nn/LogSoftMax.lua:1-9): vector or matrix of frames."""
+
+    def updateOutput(self, input):
+        _require_gpu(input, self.output)
+        _lib.check_status(lib.thgpu_LogSoftMax_updateOutput(input._p, self.output._p))
+        return self.output
+
+    def updateGradInput(self, input, gradOutput):
+        _require_gpu(gradOutput, self.output, self.gradInput)
+        _lib.check_status(lib.thgpu_LogSoftMax_updateGradInput(gradOutput._p, self.output._p, self.gradInput._p))
+        return self.gradInput
+
+
+class Criterion(object):
+    """nn.Criterion (mcw_nn/Criterion.lua:1-44)."""
+
+    def __init__(self):
+        self.gradInput = FloatTensor()
+        self.output = 0
+
+    def forward(self, input, target):
+        return self.updateOutput(input, target)
+
+    def backward(self, input, target):
+        return self.updateGradInput(input, target)
+
+    def type(self, type_name):
+        for key, val in list(self.__dict__.items()):
+            self.__dict__[key] = _convert(val, type_name)
+        return self
+
+    def gpu(self):
+        return self.type("torch.GPUTensor")
+
+    def float(self):
+        return self.type("torch.FloatTensor")
+
+
+class ClassNLLCriterion(Criterion):
+    """nn.ClassNLLCriterion() on GPU tensors (mcw_nn/ClassNLLCriterion.lua:3-72): target holds 1-based class numbers,
+    one per frame; sizeAverage defaults to true.  Class weights have no GPU implementation in the reference (its Lua
+    falls back to element-by-element tensor indexing) and are not accepted here."""
+
+    def __init__(self, weights=None):
+        Criterion.__init__(self)
+        if weights is not None:
+            raise THGPUError("nn.ClassNLLCriterion: class weights are not supported on GPU tensors")
+        self.sizeAverage = True
+        self.outputTensor = FloatTensor(1)
+
+    def updateOutput(self, input, target):
+        _require_gpu(input, target, self.outputTensor)
+        _lib.check_status(lib.thgpu_ClassNLLCriterion_updateOutput(input._p, target._p, self.outputTensor._p,
+                                                                   1 if self.sizeAverage else 0))
+        self.output = float(self.outputTensor[0])
+        return self.output
+
+    def updateGradInput(self, input, target):
+        _require_gpu(input, target, self.gradInput)
+        self.gradInput.resizeAs(input)
+        self.gradInput.zero()
+        _lib.check_status(lib.thgpu_ClassNLLCriterion_updateGradInput(input._p, target._p, self.gradInput._p,
+                                                                      1 if self.sizeAverage else 0))
+        return self.gradInput

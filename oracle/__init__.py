@@ -62,6 +62,8 @@ def _load():
     lib.oracle_subsample_updateOutput.argtypes = [_f32p, _f32p, _f32p, _c_long] + ints(7) + [_f32p]
     lib.oracle_subsample_updateGradInput.argtypes = [_f32p, _f32p, _c_long] + ints(7) + [_f32p]
     lib.oracle_subsample_accGradParameters.argtypes = [_f32p, _f32p, _c_long] + ints(7) + [_c_float, _f32p, _f32p]
+    lib.oracle_logsoftmax_updateOutput.argtypes = [_f32p, _c_long, _c_long, _f32p]
+    lib.oracle_logsoftmax_updateGradInput.argtypes = [_f32p, _f32p, _c_long, _c_long, _f32p]
     lib.oracle_threshold_updateOutput.argtypes = [_f32p, _c_long, _c_float, _c_float, _f32p]
     lib.oracle_threshold_updateGradInput.argtypes = [_f32p, _f32p, _c_long, _c_float, _f32p]
     return lib
@@ -301,6 +303,56 @@ def subsample_accGradParameters(inp, gradOutput, gradWeight, gradBias, kH, kW, d
     assert gradWeight.dtype == np.float32 and gradBias.dtype == np.float32
     _lib.oracle_subsample_accGradParameters(_p(inp), _p(gradOutput), B, C, H, W, kH, kW, dH, dW, scale,
                                             _p(gradWeight), _p(gradBias))
+
+
+def logsoftmax_updateOutput(inp):
+    """nn.LogSoftMax forward on a vector or a matrix of frames."""
+    inp = _f32(inp)
+    assert inp.ndim in (1, 2)
+    nframe, dim = (1, inp.shape[0]) if inp.ndim == 1 else inp.shape
+    out = np.empty_like(inp)
+    _lib.oracle_logsoftmax_updateOutput(_p(inp), nframe, dim, _p(out))
+    return out
+
+
+def logsoftmax_updateGradInput(gradOutput, output):
+    gradOutput, output = _f32(gradOutput), _f32(output)
+    nframe, dim = (1, output.shape[0]) if output.ndim == 1 else output.shape
+    gi = np.empty_like(output)
+    _lib.oracle_logsoftmax_updateGradInput(_p(gradOutput), _p(output), nframe, dim, _p(gi))
+    return gi
+
+
+def classnll_updateOutput(inp, target, sizeAverage=True):
+    """nn.ClassNLLCriterion forward as the Lua module computes it on CPU tensors without class weights
+    (mcw_nn/ClassNLLCriterion.lua:21-41): a Lua number (a double) accumulated frame after frame; target holds
+    1-based class numbers."""
+    inp = _f32(inp)
+    target = np.asarray(target)
+    if inp.ndim == 1:
+        return -float(inp[int(target.ravel()[0]) - 1])
+    output = 0.0
+    for i in range(inp.shape[0]):
+        output = output - float(inp[i, int(target[i]) - 1])
+    if sizeAverage:
+        output = output / inp.shape[0]
+    return output
+
+
+def classnll_updateGradInput(inp, target, sizeAverage=True):
+    """mcw_nn/ClassNLLCriterion.lua:43-71: zeros with -1 (or -1/nframe) at the target positions."""
+    inp = _f32(inp)
+    target = np.asarray(target)
+    gi = np.zeros_like(inp)
+    if inp.ndim == 1:
+        gi[int(target.ravel()[0]) - 1] = -1
+        return gi
+    z = -1.0
+    if sizeAverage:
+        z = z / inp.shape[0]
+    for i in range(inp.shape[0]):
+        gi[i, int(target[i]) - 1] = z
+    return gi
 
 
 def threshold_updateOutput(inp, threshold=0.0, val=0.0):

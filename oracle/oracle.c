@@ -486,6 +486,55 @@ void oracle_subsample_accGradParameters(const float *input, const float *gradOut
 }
 
 /* ------------------------------------------------------------------------- */
+/* nn.LogSoftMax: mcw_nn/generic/LogSoftMax.c:37-53 (forward) and :85-97
+ * (backward).  accreal is double for float tensors; the forward sum uses
+ * THExpMinusApprox (mcw_torch7_core/lib/TH/THLogAdd.c:56-86), a polynomial
+ * raised to the eighth power that is exactly zero from 13 on -- not exp. */
+static double exp_minus_approx(double x)
+{
+    if (x < 13.0) {
+        double y = 1.0 + x * (0.125 + x * (0.0078125 + x * (0.00032552083 + x * 1.0172526e-5)));
+        y *= y;
+        y *= y;
+        y *= y;
+        return 1 / y;
+    }
+    return 0;
+}
+
+void oracle_logsoftmax_updateOutput(const float *input, long nframe, long dim, float *output)
+{
+    long t;
+#pragma omp parallel for num_threads(nthreads())
+    for (t = 0; t < nframe; t++) {
+        const float *in = input + dim * t;
+        float *out = output + dim * t;
+        double logsum = 0;
+        float maxInput = -INFINITY;
+        long d;
+        for (d = 0; d < dim; d++) maxInput = maxInput > in[d] ? maxInput : in[d];
+        for (d = 0; d < dim; d++) logsum += exp_minus_approx(maxInput - in[d]);
+        logsum = maxInput + log(logsum);
+        for (d = 0; d < dim; d++) out[d] = in[d] - logsum;
+    }
+}
+
+void oracle_logsoftmax_updateGradInput(const float *gradOutput, const float *output, long nframe, long dim,
+                                       float *gradInput)
+{
+    long t;
+#pragma omp parallel for num_threads(nthreads())
+    for (t = 0; t < nframe; t++) {
+        const float *go = gradOutput + dim * t, *out = output + dim * t;
+        float *gi = gradInput + dim * t;
+        double sum = 0;
+        long d;
+        for (d = 0; d < dim; d++) sum += go[d];
+        for (d = 0; d < dim; d++) gi[d] = go[d] - exp(out[d]) * sum;
+    }
+}
+
+/* ------------------------------------------------------------------------- */
 /* nn.Threshold (nn.ReLU = Threshold(0,0), mcw_nn/ReLU.lua:1-5):
  * mcw_nn/generic/Threshold.c:5-32.  forward: x > threshold ? x : val;
  * backward uses the forward INPUT: x > threshold ? gradOutput : 0. */
