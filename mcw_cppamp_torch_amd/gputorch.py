@@ -289,6 +289,30 @@ class GPUTensor(object):
         _lib.check()
         return t
 
+    def view(self, *sizes):
+        """tensor:view(sizes) (mcw_torch7_core/Tensor.lua: a new tensor on the same storage; the tensor must be
+        contiguous and the element count must match)."""
+        if len(sizes) == 1 and not np.isscalar(sizes[0]):
+            sizes = tuple(sizes[0])
+        sizes = [int(v) for v in sizes]
+        if sizes.count(-1) == 1:                  # one dimension may be left for view to work out
+            known = int(np.prod([v for v in sizes if v != -1], dtype=np.int64))
+            if known > 0 and self.nElement() % known == 0:
+                sizes[sizes.index(-1)] = self.nElement() // known
+        if not self.isContiguous():
+            raise THGPUError("expecting a contiguous tensor")
+        if int(np.prod(sizes, dtype=np.int64)) != self.nElement():
+            raise THGPUError("Wrong size for view. Input size: %d. Output size: %s" % (self.nElement(), "x".join(map(str, sizes))))
+        arr = (ctypes.c_long * len(sizes))(*sizes)
+        st = _lib.THLongStorage()
+        st.data = ctypes.cast(arr, _lib.longp)
+        st.size = len(sizes)
+        return self._view(lib.THGPUTensor_newWithStorage(lib.THGPUTensor_storage(self._p), self.storageOffset(),
+                                                         ctypes.byref(st), None))
+
+    def viewAs(self, other):
+        return self.view(*other.size())
+
     def contiguous(self):
         return self._view(lib.THGPUTensor_newContiguous(self._p))
 

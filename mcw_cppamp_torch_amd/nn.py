@@ -9,6 +9,7 @@ to the C ABI the way the Lua modules dispatch to `input.nn.<Op>_<method>`:
   nn.Linear                mcw_nn/Linear.lua:1-104 (the classifier after a conv stack)
   nn.SpatialAveragePooling mcw_nn/SpatialAveragePooling.lua:1-20
   nn.SpatialSubSampling    mcw_nn/SpatialSubSampling.lua:1-54
+  nn.View, nn.Reshape      mcw_nn/View.lua:1-47, mcw_nn/Reshape.lua:1-70 (between a conv stack and its classifier)
   nn.LogSoftMax            mcw_nn/LogSoftMax.lua:1-9
   nn.Criterion, nn.ClassNLLCriterion   mcw_nn/Criterion.lua:1-44, mcw_nn/ClassNLLCriterion.lua:1-72
 
@@ -93,6 +94,30 @@ class Module(object):
             else:
                 g[...] = 0
 
+    def updateParameters(self, learningRate):
+        # mcw_nn/Module.lua:75-82
+        params, grads = self.parameters()
+        for p, g in zip(params or [], grads or []):
+            if isinstance(p, GPUTensor):
+                p.add(-learningRate, g)
+            else:
+                p += np.float32(-learningRate) * g
+
+    def accUpdateGradParameters(self, input, gradOutput, lr):
+        # mcw_nn/Module.lua:49-57: accumulate straight into the parameters with scale -lr
+        gw, gb = getattr(self, "gradWeight", None), getattr(self, "gradBias", None)
+        self.gradWeight, self.gradBias = getattr(self, "weight", None), getattr(self, "bias", None)
+        try:
+            self.accGradParameters(input, gradOutput, -lr)
+        finally:
+            self.gradWeight, self.gradBias = gw, gb
+
+    def backwardUpdate(self, input, gradOutput, lr):
+        # mcw_nn/Module.lua:35-39
+        self.updateGradInput(input, gradOutput)
+        self.accUpdateGradParameters(input, gradOutput, lr)
+        return self.gradInput
+
     def type(self, type_name):
         for key, val in list(self.__dict__.items()):
             if key != "modules":
@@ -154,9 +179,42 @@ class Sequential(Module):
             cur = self.modules[i].gradInput
         self.modules[0].accGradParameters(input, cur, scale)
 
+    def accUpdateGradParameters(self, input, gradOutput, lr):
+        # mcw_nn/Sequential.lua:72-83
+        cur = gradOutput
+        for i in range(len(self.modules) - 1, 0, -1):
+            self.modules[i].accUpdateGradParameters(self.modules[i - 1].output, cur, lr)
+            cur = self.modules[i].gradInput
+        self.modules[0].accUpdateGradParameters(input, cur, lr)
+
     def zeroGradParameters(self):
         for m in self.modules:
             m.zeroGradParameters()
+
+    def updateParameters(self, learningRate):
+        # mcw_nn/Sequential.lua:91-95
+        for m in self.modules:
+            m.updateParameters(learningRate)
+
+    def parameters(self):
+        # mcw_nn/Sequential.lua:121-141: the modules' parameters and gradients, flattened in module order
+        w, gw = [], []
+        for m in self.modules:
+            mw, mgw = m.parameters()
+            if mw:
+                w.extend(mw)
+                gw.extend(mgw)
+        return w, gw
+
+    def insert(self, module, index=None):
+        # mcw_nn/Sequential.lua:17-25 (index counts from 0 here)
+        index = len(self.modules) if index is None else index
+        if index > len(self.modules):
+            raise THGPUError("index should be contiguous to existing modules")
+        self.modules.insert(index, module)
+        self.output = self.modules[-1].output
+        self.gradInput = self.modules[0].gradInput
+        return self
 
     def reset(self, stdv=None):
         for m in self.modules:
@@ -418,6 +476,85 @@ class Threshold(Module):
 class ReLU(Threshold):
     def __init__(self):
         Threshold.__init__(self, 0, 0)
+
+
+class View(Module):
+    """nn.View(sizes...) (mcw_nn/View.lua:1-47): a view of the input with the given sizes, keeping a leading batch
+    dimension when the input has one more dimension than setNumInputDims says, or when its per-sample element count
+    matches."""
+
+    def __init__(self, *sizes):
+        Module.__init__(self)
+        if len(sizes) == 1 and not np.isscalar(sizes[0]):
+            sizes = tuple(sizes[0])
+        self.size = tuple(int(v) for v in sizes)
+        self.numElements = int(np.prod(self.size, dtype=np.int64))
+        self.output = None
+        self.gradInput = None
+        self.numInputDims = None
+
+    def setNumInputDims(self, n):
+        self.numInputDims = n
+        return self
+
+    def _is_minibatch(self, input):
+        if self.numInputDims:
+            return input.dim() == self.numInputDims + 1
+        return input.dim() > 1 and input.nElement() // input.size(0) == self.numElements and \
+            input.nElement() % input.size(0) == 0
+
+    def updateOutput(self, input):
+        _require_gpu(input)
+        if self._is_minibatch(input):
+            self.output = input.view(input.size(0), *self.size)
+        else:
+            self.output = input.view(*self.size)
+        return self.output
+
+    def updateGradInput(self, input, gradOutput):
+        _require_gpu(input, gradOutput)
+        self.gradInput = gradOutput.view(*input.size())
+        return self.gradInput
+
+
+class Reshape(Module):
+    """nn.Reshape(sizes..., [batchMode]) (mcw_nn/Reshape.lua:1-70): like View, but a non-contiguous input or
+    gradOutput is copied into a dense buffer first."""
+
+    def __init__(self, *args):
+        Module.__init__(self)
+        args = list(args)
+        self.batchMode = None
+        if args and isinstance(args[-1], bool):
+            self.batchMode = args.pop()
+        if len(args) == 1 and not np.isscalar(args[0]):
+            args = list(args[0])
+        self.size = tuple(int(v) for v in args)
+        self.nelement = int(np.prod(self.size, dtype=np.int64))
+        self._input = FloatTensor()
+        self._gradOutput = FloatTensor()
+
+    def updateOutput(self, input):
+        _require_gpu(input, self._input)
+        if not input.isContiguous():
+            self._input.resizeAs(input)
+            self._input.copy(input)
+            input = self._input
+        if self.batchMode is False or (self.batchMode is None and input.nElement() == self.nelement and
+                                       input.size(0) != 1):
+            self.output = input.view(*self.size)
+        else:
+            self.output = input.view(input.size(0), *self.size)
+        return self.output
+
+    def updateGradInput(self, input, gradOutput):
+        _require_gpu(input, gradOutput, self._gradOutput)
+        if not gradOutput.isContiguous():
+            self._gradOutput.resizeAs(gradOutput)
+            self._gradOutput.copy(gradOutput)
+            gradOutput = self._gradOutput
+        self.gradInput = gradOutput.viewAs(input)
+        return self.gradInput
 
 
 class LogSoftMax(Module):
