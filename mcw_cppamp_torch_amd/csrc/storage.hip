@@ -124,6 +124,7 @@ THGPUStorage *THGPUStorage_newWithSize(long size) {
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&s->data), sizeof(float) * (size_t)size);
     if (e != hipSuccess) {
         std::free(s);
+        (void)hipGetLastError();  // the failure is reported here; later launch checks must not see it again
         raise("hipMalloc of %ld floats failed: %s", size, hipGetErrorString(e));
         return nullptr;
     }
@@ -198,6 +199,7 @@ void THGPUStorage_resize(THGPUStorage *self, long size) {
     }
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&fresh), sizeof(float) * (size_t)size);
     if (e != hipSuccess) {
+        (void)hipGetLastError();
         raise("hipMalloc of %ld floats failed: %s", size, hipGetErrorString(e));
         return;
     }

@@ -250,3 +250,17 @@ def test_copies_with_non_contiguous_host_and_device_tensors(gt):
     with pytest.raises(gt.THGPUError):
         gt.GPUTensor(3, 3).copy(base)             # sizes do not match
     assert d.double().dtype == np.float64 and np.array_equal(d.double(), ref.astype(np.float64))
+
+
+def test_allocation_failure_is_reported_and_leaves_the_library_usable(gt):
+    S = gt.gputorch.GPUStorage
+    with pytest.raises(gt.THGPUError, match="hipMalloc"):
+        S(1 << 46)                                # 256 TiB
+    s = S(8).fill(1.0)
+    with pytest.raises(gt.THGPUError, match="hipMalloc"):
+        s.resize(1 << 46)
+    assert s.size() == 8 and np.array_equal(s.float(), np.ones(8, np.float32))      # unchanged by the failed resize
+    t = gt.GPUTensor(3, 3).fill(2.0)              # kernels still launch and check clean
+    assert np.array_equal(t.float(), np.full((3, 3), 2.0, np.float32))
+    with pytest.raises(gt.THGPUError):
+        gt.GPUTensor(1 << 23, 1 << 23)
