@@ -62,7 +62,7 @@ struct TileCfg {
 
 const TileCfg kCfgs[] = {
     {"128x128", 128, 128, 4, {0.90, 0.90, 0.88, 0.86}, true, gemm_fast_128x128},
-    {"192x128", 192, 128, 3, {0.90, 0.0, 0.90, 0.0}, false, gemm_fast_192x128},
+    {"192x128", 192, 128, 3, {0.90, 0.90, 0.90, 0.86}, true, gemm_fast_192x128},
     {"64x256", 64, 256, 3, {0.76, 0.74, 0.90, 0.74}, true, gemm_fast_64x256},
     {"128x256", 128, 256, 2, {0.85, 0.87, 1.06, 0.85}, true, gemm_fast_128x256},
     {"256x128", 256, 128, 2, {0.90, 0.75, 1.06, 0.75}, true, gemm_fast_256x128},

@@ -33,6 +33,11 @@
 
 namespace thgpu {
 
+// Loader kind used inside the kernel only: an x-contiguous first operand whose row count the thread
+// count does not divide (192 rows, 256 threads).  Wavefront w takes r = 4w .. 4w+3 of every block of
+// 64 consecutive rows; lanes run along the rows.
+constexpr int LD_XC_BLOCK = 3;
+
 // LDS row layout by loader kind: pitch in floats, and the column at which element r of row x is stored.
 template <int KIND>
 struct LdsRow {
@@ -73,11 +78,13 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     constexpr int NA = BM * BK / NT, NB = BN * BK / NT;
     static_assert(BM % (WGM * 32) == 0 && BN % (WGN * 32) == 0, "wave tile must be whole 32x32 blocks");
     static_assert(NT % 16 == 0 && NA >= 4 && NB >= 4 && NA % 4 == 0 && NB % 4 == 0, "loader shape");
-    static_assert((LA != LD_XC_SCALAR || NT % BM == 0) && (LB != LD_XC_SCALAR || NT % BN == 0),
-                  "x-contiguous loaders give every thread one row/column");
+    // The kind the A loader really uses: x-contiguous with 192 rows goes block-wise.
+    constexpr int KA = (LA == LD_XC_SCALAR && NT % BM != 0) ? LD_XC_BLOCK : LA;
+    static_assert(KA != LD_XC_BLOCK || (NT == 256 && BM % 64 == 0 && NA == BM / 16), "block loader shape");
+    static_assert(LB != LD_XC_SCALAR || NT % BN == 0, "x-contiguous loaders give every thread one row/column");
     static_assert(!RED || (LA != LD_XC_SCALAR && LB != LD_XC_SCALAR), "reduction batching needs r-contiguous operands");
 
-    using RowA = LdsRow<LA>;
+    using RowA = LdsRow<KA>;
     using RowB = LdsRow<LB>;
     __shared__ __attribute__((aligned(16))) float As[2][BM][RowA::kPitch];
     __shared__ __attribute__((aligned(16))) float Bs[2][BN][RowB::kPitch];
@@ -118,13 +125,19 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     //   LD_RC_VEC     x = tid/4 (+64 per load), r = 4*(tid%4) .. +3   (one 128-bit load each)
     //   LD_RC_SCALAR  x = tid/16 (+16 per load), r = tid%16
     //   LD_XC_SCALAR  x = tid % X, r = (tid / X) * CNT .. + CNT-1     (CNT loads down the column)
+    //   LD_XC_BLOCK   x = lane (+64 per block of rows), r = 4*wave .. +3
     // A load address is a wave-uniform base (tile, image, step, load number: all
     // scalar) plus a per-thread byte offset that never changes, so the loop
     // spends no vector ALU work on addressing.
     int a_x, a_r, b_x, b_r;
     unsigned voffA, voffB;
     const char *tileA, *tileB;
-    if (LA == LD_XC_SCALAR) {
+    if (KA == LD_XC_BLOCK) {
+        a_x = lane;
+        a_r = 4 * wave;
+        voffA = (unsigned)(((long)a_r * g.sA + a_x) * 4);
+        tileA = reinterpret_cast<const char *>(g.A + i0);
+    } else if (LA == LD_XC_SCALAR) {
         a_x = tid % BM;
         a_r = (tid / BM) * NA;
         voffA = (unsigned)(((long)a_r * g.sA + a_x) * 4);
@@ -173,6 +186,8 @@ __global__ __launch_bounds__(WGM *WGN * 64)
             dst[u * 4 + 3] = v.w;
         } else if (KIND == LD_RC_SCALAR) {
             dst[u] = *reinterpret_cast<const float *>(base + (long)(u * (NT / 16)) * stride * 4 + voff);
+        } else if (KIND == LD_XC_BLOCK) {
+            dst[u] = *reinterpret_cast<const float *>(base + (long)(u & 3) * stride * 4 + (u >> 2) * 256 + voff);
         } else {
             dst[u] = *reinterpret_cast<const float *>(base + (long)u * stride * 4 + voff);
         }
@@ -201,7 +216,9 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         constexpr int CNT = decltype(count_tag)::value;
 #pragma unroll
         for (int q = 0; q < CNT; ++q) {
-            const int rel = KIND == LD_RC_VEC ? t_r + (q & 3) : KIND == LD_RC_SCALAR ? t_r : t_r + q;
+            const int rel = (KIND == LD_RC_VEC || KIND == LD_XC_BLOCK) ? t_r + (q & 3)
+                            : KIND == LD_RC_SCALAR                          ? t_r
+                                                                            : t_r + q;
             v[q] = rel < shift ? 0.0f : v[q];
         }
     };
@@ -218,6 +235,11 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         } else if (KIND == LD_RC_SCALAR) {
 #pragma unroll
             for (int q = 0; q < CNT; ++q) tile[t_x + q * (NT / 16)][Row::col(t_x + q * (NT / 16), t_r)] = src[q];
+        } else if (KIND == LD_XC_BLOCK) {
+#pragma unroll
+            for (int w = 0; w < CNT / 4; ++w)
+                *reinterpret_cast<float4 *>(&tile[t_x + 64 * w][Row::col(t_x + 64 * w, t_r)]) =
+                    make_float4(src[w * 4], src[w * 4 + 1], src[w * 4 + 2], src[w * 4 + 3]);
         } else {
 #pragma unroll
             for (int w = 0; w < CNT / 4; ++w)
@@ -227,10 +249,10 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     };
     auto stash = [&](int buf, int shift) {
         if (shift > 0) {  // uniform: only the last step of an image can be partial
-            mask_one(std::integral_constant<int, LA>{}, a_r, ra, std::integral_constant<int, NA>{}, shift);
+            mask_one(std::integral_constant<int, KA>{}, a_r, ra, std::integral_constant<int, NA>{}, shift);
             mask_one(std::integral_constant<int, LB>{}, b_r, rb, std::integral_constant<int, NB>{}, shift);
         }
-        stash_one(std::integral_constant<int, LA>{}, As[buf], a_x, a_r, ra, std::integral_constant<int, NA>{});
+        stash_one(std::integral_constant<int, KA>{}, As[buf], a_x, a_r, ra, std::integral_constant<int, NA>{});
         stash_one(std::integral_constant<int, LB>{}, Bs[buf], b_x, b_r, rb, std::integral_constant<int, NB>{});
     };
 
@@ -240,7 +262,7 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     if (nsteps > 0) {
         step_bases(ga, gb, shift);
 #pragma unroll
-        for (int u = 0; u < UA; ++u) load_unit(std::integral_constant<int, LA>{}, ga, g.sA, voffA, ra, u);
+        for (int u = 0; u < UA; ++u) load_unit(std::integral_constant<int, KA>{}, ga, g.sA, voffA, ra, u);
 #pragma unroll
         for (int u = 0; u < UB; ++u) load_unit(std::integral_constant<int, LB>{}, gb, g.sB, voffB, rb, u);
         stash(0, shift);
@@ -311,7 +333,7 @@ __global__ __launch_bounds__(WGM *WGN * 64)
 #pragma unroll
                     for (int u = 0; u < UA; ++u)
                         if (u * SLICES / UA == slice)
-                            load_unit(std::integral_constant<int, LA>{}, ga, g.sA, voffA, ra, u);
+                            load_unit(std::integral_constant<int, KA>{}, ga, g.sA, voffA, ra, u);
 #pragma unroll
                     for (int u = 0; u < UB; ++u)
                         if (u * SLICES / UB == slice)
@@ -427,7 +449,8 @@ template <int BM, int BN, int WGM, int WGN>
 int gemm_fast_dispatch(const GemmArgs &g, int la, int lb, bool red, hipStream_t s) {
 #define THGPU_CASE(LA_, LB_)                                                           \
     if (la == LA_ && lb == LB_) {                                                      \
-        if constexpr ((LA_ == LD_XC_SCALAR && (WGM * WGN * 64) % BM != 0) ||           \
+        if constexpr ((LA_ == LD_XC_SCALAR && (WGM * WGN * 64) % BM != 0 &&            \
+                       !((WGM * WGN * 64) == 256 && BM % 64 == 0)) ||                  \
                       (LB_ == LD_XC_SCALAR && (WGM * WGN * 64) % BN != 0)) {           \
             return fail("gemm: this tile has no x-contiguous loader for that side");   \
         } else {                                                                       \

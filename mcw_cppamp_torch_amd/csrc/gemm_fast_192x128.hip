@@ -1,5 +1,5 @@
 // Fast fp32 MFMA GEMM, 192 x 128 workgroup tile (2 x 2 wavefronts of 96 x 64): for row counts that are
-// multiples of 192 rather than 128.  Its first operand must be contiguous along the reduction index.
+// multiples of 192 rather than 128.
 #include "gemm_fast.h"
 
 #include <type_traits>

@@ -253,8 +253,7 @@ GEMM_TILES = ["128x128", "192x128", "64x256", "128x256", "256x128", "64x64"]
 def test_blas_gemm_every_tile_configuration_exact(gt, tile, ta, tb, split, monkeypatch):
     """Every tile configuration of the fast kernel is forced in turn on a ragged problem (edge tiles shifted back in
     both directions, a partial last reduction step) with small integers, where any summation order is exact.  The
-    profiler label tells which kernel ran: a configuration without a loader for the operand layout at hand must
-    have gone to the bounds-checked kernel, never to another fast tile."""
+    profiler label tells which kernel ran."""
     monkeypatch.setenv("THGPU_GEMM_TILE", tile)
     monkeypatch.setenv("THGPU_GEMM_SPLIT", str(split))
     rng = rng_for(43)
@@ -285,8 +284,7 @@ def test_blas_gemm_every_tile_configuration_exact(gt, tile, ta, tb, split, monke
     assert np.array_equal(dc.float().reshape(n, ldc), ref)
     assert len(labels) == 1
     ran = labels[0].split("tile=")[1].split(" ")[0]
-    # the 192x128 tile only loads a first operand that is contiguous along the reduction index: op(B) = B here
-    assert ran == (tile if tile != "192x128" or tb == "n" else "generic"), labels
+    assert ran == tile, labels
     assert ("split=%d" % split) in labels[0] or ran == "generic", labels
 
 
