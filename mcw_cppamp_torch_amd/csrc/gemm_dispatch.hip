@@ -56,17 +56,16 @@ struct TileCfg {
     // measured launch times together with kOcc below, so a two-resident tile that loses nothing to its
     // lower occupancy carries a figure above 1.
     double eff[4];
-    bool a_xc;  // has a loader for a first operand that is contiguous along i
     int (*launch)(const GemmArgs &, int, int, bool, hipStream_t);
 };
 
 const TileCfg kCfgs[] = {
-    {"128x128", 128, 128, 4, {0.90, 0.90, 0.88, 0.86}, true, gemm_fast_128x128},
-    {"192x128", 192, 128, 3, {0.90, 0.90, 0.90, 0.86}, true, gemm_fast_192x128},
-    {"64x256", 64, 256, 3, {0.76, 0.74, 0.90, 0.74}, true, gemm_fast_64x256},
-    {"128x256", 128, 256, 2, {0.85, 0.87, 1.06, 0.85}, true, gemm_fast_128x256},
-    {"256x128", 256, 128, 2, {0.90, 0.75, 1.06, 0.75}, true, gemm_fast_256x128},
-    {"64x64", 64, 64, 4, {0.68, 0.60, 0.74, 0.60}, true, gemm_fast_64x64},
+    {"128x128", 128, 128, 4, {0.90, 0.90, 0.88, 0.86}, gemm_fast_128x128},
+    {"192x128", 192, 128, 3, {0.90, 0.90, 0.90, 0.86}, gemm_fast_192x128},
+    {"64x256", 64, 256, 3, {0.76, 0.74, 0.90, 0.74}, gemm_fast_64x256},
+    {"128x256", 128, 256, 2, {0.85, 0.87, 1.06, 0.85}, gemm_fast_128x256},
+    {"256x128", 256, 128, 2, {0.90, 0.75, 1.06, 0.75}, gemm_fast_256x128},
+    {"64x64", 64, 64, 4, {0.68, 0.60, 0.74, 0.60}, gemm_fast_64x64},
 };
 
 inline long cdiv(long a, long b) { return (a + b - 1) / b; }
@@ -155,7 +154,7 @@ int gemm_launch(const GemmProblem &p) {
     const bool fast_ok = p.R == 0 || p.R >= GEMM_BK;
     const int layout = p.a_rc ? (p.b_rc ? 2 : 0) : (p.b_rc ? 3 : 1);
     for (const TileCfg &c : kCfgs) {
-        if (!fast_ok || p.M < c.bm || p.J < c.bn || !offsets_fit(c.bm, c.bn) || (!p.a_rc && !c.a_xc)) continue;
+        if (!fast_ok || p.M < c.bm || p.J < c.bn || !offsets_fit(c.bm, c.bn)) continue;
         if (force && std::strcmp(force, c.name) != 0) continue;
         const long tiles = cdiv(p.M, c.bm) * cdiv(p.J, c.bn);
         const int max_split = (int)(g.steps_total / 8 > 0 ? (g.steps_total / 8 < 256 ? g.steps_total / 8 : 256) : 1);
