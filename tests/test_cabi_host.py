@@ -128,3 +128,42 @@ def test_stack_bookkeeping_reproduces_the_benchmark_work(pkg):
     assert st.output_shape("alexnet") == (128, 256, 6, 6)
     assert st.output_shape("overfeat") == (128, 1024, 6, 6)
     assert st.output_shape("vgg_a") == (64, 512, 7, 7)
+
+
+def test_more_module_defaults_follow_the_lua_constructors(pkg):
+    nn = pkg.nn
+    a = nn.SpatialAveragePooling(3, 2)
+    assert (a.kW, a.kH, a.dW, a.dH) == (3, 2, 1, 1)                      # mcw_nn/SpatialAveragePooling.lua:8-9
+    s = nn.SpatialSubSampling(6, 2, 3)
+    assert (s.dW, s.dH) == (1, 1) and s.weight.shape == (6,) and s.gradBias.shape == (6,)
+    bound = 1 / np.sqrt(2 * 3)                                           # mcw_nn/SpatialSubSampling.lua:28
+    assert np.abs(s.weight).max() <= bound and np.abs(s.bias).max() <= bound
+    c = nn.ClassNLLCriterion()
+    assert c.sizeAverage is True and c.output == 0 and c.outputTensor.shape == (1,)
+    v = nn.View(4, 5)
+    assert v.size == (4, 5) and v.numElements == 20 and v.output is None and v.numInputDims is None
+    r = nn.Reshape(2, 3, True)
+    assert r.size == (2, 3) and r.nelement == 6 and r.batchMode is True
+    seq = nn.Sequential().add(nn.Linear(3, 2)).add(nn.ReLU()).add(nn.Linear(2, 2))
+    w, gw = seq.parameters()
+    assert len(w) == 4 and len(gw) == 4                                  # weight, bias of both Linear modules
+    seq.insert(nn.ReLU(), 0)
+    assert seq.size() == 4 and isinstance(seq.get(0), nn.ReLU)
+    with pytest.raises(pkg.THGPUError):
+        seq.insert(nn.ReLU(), 9)
+
+
+def test_product_never_imports_the_oracle_and_bench_refuses_more_than_one_gpu():
+    import glob
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for path in glob.glob(os.path.join(root, "mcw_cppamp_torch_amd", "**", "*.py"), recursive=True):
+        text = open(path).read()
+        assert "import oracle" not in text and "from oracle" not in text, path
+    for path in glob.glob(os.path.join(root, "mcw_cppamp_torch_amd", "csrc", "*")):
+        assert "oracle" not in open(path, errors="ignore").read(), path
+    proc = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], stdout=subprocess.PIPE,
+                          stderr=subprocess.PIPE, text=True, timeout=120)
+    assert proc.returncode != 0 and "one GPU" in (proc.stdout + proc.stderr)
