@@ -133,3 +133,41 @@ def test_pooling_random_geometry_bit_exact(gt, geo):
     assert np.array_equal(bits(out.float()), bits(oracle.subsample_updateOutput(x, w, b, kH, kW, dH, dW)))
     gt._lib.check_status(lib.thgpu_SpatialSubSampling_updateGradInput(dx._p, dgo._p, dw._p, gi._p, kW, kH, dW, dH))
     assert np.array_equal(bits(gi.float()), bits(oracle.subsample_updateGradInput(go, w, x.shape, kH, kW, dH, dW)))
+
+
+def gemm_cases(n, seed):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    out = []
+    for _ in range(n):
+        big = rng.integers(0, 3) == 0
+        hi = 700 if big else 90
+        m, nn_, k = int(rng.integers(1, hi)), int(rng.integers(1, hi)), int(rng.integers(1, hi))
+        out.append(("nt"[rng.integers(0, 2)], "nt"[rng.integers(0, 2)], m, nn_, k, int(rng.integers(0, 4)),
+                    int(rng.integers(0, 4)), int(rng.integers(0, 4)), float(rng.choice([1.0, 0.5, -2.0])),
+                    float(rng.choice([0.0, 1.0, 0.25]))))
+    return out
+
+
+@pytest.mark.parametrize("case", gemm_cases(48, 2004))
+def test_blas_gemm_random_shapes(gt, case):
+    ta, tb, m, n, k, pa, pb, pc, alpha, beta = case
+    rng = np.random.Generator(np.random.PCG64(hash(case[:8]) % (1 << 32)))
+    lda = (m if ta == "n" else k) + pa
+    ldb = (k if tb == "n" else n) + pb
+    ldc = m + pc
+    integer = (m + n + k) % 2 == 0                 # half of the cases on small integers: any summation order is exact
+    draw = (lambda size: rng.integers(-3, 4, size=size).astype(np.float32)) if integer else (lambda size: uniform(rng, size))
+    a = draw((lda * (k if ta == "n" else m),))
+    b = draw((ldb * (n if tb == "n" else k),))
+    c0 = draw((ldc * n,))
+    ref = c0.copy()
+    oracle.sgemm(ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, ref, ldc)
+    da, db, dc = dev(gt, a), dev(gt, b), dev(gt, c0)
+    gt.gputorch.gemm(ta, tb, m, n, k, alpha, da, lda, db, ldb, beta, dc, ldc)
+    got = dc.float().reshape(n, ldc)
+    ref = ref.reshape(n, ldc)
+    if integer:
+        assert np.array_equal(got, ref)
+    else:
+        assert rel_err(got[:, :m], ref[:, :m]) < gemm_tol(k)
+        assert np.array_equal(got[:, m:], c0.reshape(n, ldc)[:, m:])       # the padding of C is never written
