@@ -371,7 +371,7 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     // A store address is a wave-uniform row base plus a constant per-lane byte
     // offset (column, image and the lane half's four rows), as for the loads.
     // MODE 0: partial sums to the workspace; 1: alpha*acc (+bias); 2: also + beta*C.
-    const bool rows_shifted = i0 != own_i0;
+    const bool edge_tile = i0 != own_i0 || j0 != own_j0;  // an edge tile: some rows or columns belong to its neighbour
     auto write_out = [&](auto mode_tag, auto check_tag) {
         constexpr int MODE = decltype(mode_tag)::value;
         constexpr bool CHECK = decltype(check_tag)::value;
@@ -382,35 +382,45 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         const bool per_image = MODE != 0 && !RED && g.N != g.J;
         if (per_image) g.divN.divmod((unsigned)j0, img0, n0);
         char *const out = out0 + (per_image ? (long)img0 * g.bsC : (long)j0) * 4;
+        // Per 32-column block of the wavefront: the lane's byte offset and whether this tile owns the column.
+        unsigned voff[TN];
+        bool own[TN];
 #pragma unroll
         for (int b = 0; b < TN; ++b) {
             const int jg = j0 + wn * (TN * 32) + b * 32 + l32;
-            if (jg < own_j0) continue;  // owned by the neighbouring tile
+            own[b] = jg >= own_j0;  // else the neighbouring tile stores it
             long col = jg - j0;
             if (per_image) {
                 unsigned im, n;
                 g.divN.divmod((unsigned)jg, im, n);
                 col = (long)(im - img0) * g.bsC + n;
             }
-            const unsigned voff = (unsigned)(col * 4 + 4 * half * row_bytes);
+            voff[b] = (unsigned)(col * 4 + 4 * half * row_bytes);
+        }
+        // Rows outermost, the wavefront's column blocks innermost: the stores of one output row follow each other
+        // directly, so a cache line that two neighbouring 128-byte segments share (rows are rarely 128-byte aligned)
+        // is completed while it is still in L2 instead of going out to memory twice.
 #pragma unroll
-            for (int a = 0; a < TM; ++a) {
-                const int iu = i0 + wm * (TM * 32) + a * 32;  // uniform
-                float bias_v[16];
-                if (MODE != 0 && g.bias) {
+        for (int a = 0; a < TM; ++a) {
+            const int iu = i0 + wm * (TM * 32) + a * 32;  // uniform
+            float bias_v[16];
+            if (MODE != 0 && g.bias) {
 #pragma unroll
-                    for (int v = 0; v < 16; ++v)
-                        bias_v[v] = *reinterpret_cast<const float *>(
-                            reinterpret_cast<const char *>(g.bias + iu + 8 * (v / 4) + (v % 4)) + 16 * half);
-                } else {
+                for (int v = 0; v < 16; ++v)
+                    bias_v[v] = *reinterpret_cast<const float *>(
+                        reinterpret_cast<const char *>(g.bias + iu + 8 * (v / 4) + (v % 4)) + 16 * half);
+            } else {
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) bias_v[v] = 0.0f;
-                }
+                for (int v = 0; v < 16; ++v) bias_v[v] = 0.0f;
+            }
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int ir = iu + 8 * (v / 4) + (v % 4);  // uniform; the lane's row is ir + 4*half
-                    if (CHECK && ir + 4 * half < own_i0) continue;
-                    float *c = reinterpret_cast<float *>(out + (long)ir * row_bytes + voff);
+            for (int v = 0; v < 16; ++v) {
+                const int ir = iu + 8 * (v / 4) + (v % 4);  // uniform; the lane's row is ir + 4*half
+                if (CHECK && ir + 4 * half < own_i0) continue;
+#pragma unroll
+                for (int b = 0; b < TN; ++b) {
+                    if (CHECK && !own[b]) continue;
+                    float *c = reinterpret_cast<float *>(out + (long)ir * row_bytes + voff[b]);
                     float val = acc[a][b][v];
                     if ((DBG & 16) && (v != 0 || val != 12345.0f)) continue;
                     if (MODE != 0) val = val * g.alpha + bias_v[v];
@@ -428,10 +438,10 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     }
     using std::integral_constant;
     if (g.nsplit > 1) {
-        if (rows_shifted) write_out(integral_constant<int, 0>{}, integral_constant<bool, true>{});
+        if (edge_tile) write_out(integral_constant<int, 0>{}, integral_constant<bool, true>{});
         else write_out(integral_constant<int, 0>{}, integral_constant<bool, false>{});
     } else if (g.beta == 0.0f) {
-        if (rows_shifted) write_out(integral_constant<int, 1>{}, integral_constant<bool, true>{});
+        if (edge_tile) write_out(integral_constant<int, 1>{}, integral_constant<bool, true>{});
         else write_out(integral_constant<int, 1>{}, integral_constant<bool, false>{});
     } else {
         write_out(integral_constant<int, 2>{}, integral_constant<bool, true>{});
