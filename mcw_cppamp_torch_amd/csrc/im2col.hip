@@ -668,14 +668,18 @@ long im2col_plan_selftest() {
     long bad = 0;
     const int sizes[] = {1, 2, 5, 6, 7, 12, 13, 14, 24, 27, 28, 55, 56, 57, 112, 224, 231, 300, 1000, 5000};
     const int kernels[] = {1, 2, 3, 5, 7, 11};
+    const int strides[] = {1, 2, 4};
     for (int H : sizes)
         for (int W : sizes)
             for (int k : kernels)
-                for (int st = 1; st <= 4; st += (st == 1 ? 1 : 2))
-                    for (int pad = 0; pad <= k / 2; pad += (k / 2 > 0 ? k / 2 : 1)) {
+                for (int kw : {k, 3})  // square kernels, and every height against a width of 3
+                    for (int sH : strides)
+                        for (int sW : strides)
+                            for (int pad = 0; pad <= k / 2; pad += (k / 2 > 0 ? k / 2 : 1)) {
                         ConvGeom g;
-                        if (H + 2 * pad < k || W + 2 * pad < k) continue;
-                        if (make_geom(g, 4, 3, H, W, k, k, pad, pad, st, st)) continue;
+                        const int padw = pad < kw ? pad : kw - 1;
+                        if (H + 2 * pad < k || W + 2 * padw < kw) continue;
+                        if (make_geom(g, 4, 3, H, W, k, kw, pad, padw, sH, sW)) continue;
                         for (long planes : {1L, 7L, 4096L}) {
                             StripPlan p;
                             if (!plan_strips(g, planes, p)) continue;
