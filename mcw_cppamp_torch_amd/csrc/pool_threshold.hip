@@ -435,19 +435,22 @@ long pool_plan_selftest() {
     for (int H : sizes)
         for (int W : sizes)
             for (int k = 1; k <= 4; ++k)
-                for (int d = 1; d <= 4; ++d) {
-                    const int th = (k + d - 1) / d;
-                    if (H < k || W < k || !(th == 1 || th == 2)) continue;
+                for (int kw : {k, 2})  // square windows, and every height against a width of 2
+                    for (int d = 1; d <= 4; ++d)
+                        for (int dw : {d, 2}) {
+                    // the tile kernel takes th == tw in {1, 2}, as the launcher requires
+                    const int th = (k + d - 1) / d, tw = (kw + dw - 1) / dw;
+                    if (H < k || W < kw || th != tw || !(th == 1 || th == 2)) continue;
                     PoolGeom g;
-                    g.H = H; g.W = W; g.kH = k; g.kW = k; g.dH = d; g.dW = d;
+                    g.H = H; g.W = W; g.kH = k; g.kW = kw; g.dH = d; g.dW = dw;
                     g.Ho = (H - k) / d + 1;
-                    g.Wo = (W - k) / d + 1;
+                    g.Wo = (W - kw) / dw + 1;
                     for (long planes : {1L, 5L, 4096L}) {
                         PoolBwdPlan p;
-                        if (!plan_pool_bwd(g, planes, th, th, p)) continue;
+                        if (!plan_pool_bwd(g, planes, th, tw, p)) continue;
                         bool ok = p.G >= 1 && p.G <= planes && p.PR >= 1 && p.PR <= H && (p.G == 1 || p.PR == H) &&
                                   (long)p.G * p.RW * p.CW * 8 <= kPoolBwdLdsBytes && (long)p.tiles * p.PR >= H &&
-                                  (long)(p.tiles - 1) * p.PR < H && p.CW >= (W - 1) / d + th;
+                                  (long)(p.tiles - 1) * p.PR < H && p.CW >= (W - 1) / dw + tw;
                         for (int t = 0; t < p.tiles && ok; ++t) {
                             const int h0 = t * p.PR, h1 = (h0 + p.PR < H ? h0 + p.PR : H) - 1;
                             const int i_first = h0 / d - (th - 1);
