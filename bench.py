@@ -39,7 +39,7 @@ PEAK_HBM_GBS = 8000.0
 MEASURED_GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("alexnet", 128): 5.428e8}
 
 
-def cpu_baseline(workload, sample_batch, budget_s=20.0):
+def cpu_baseline(workload, sample_batch, budget_s=12.0):
     """Times the CPU oracle on `sample_batch` images of the workload."""
     import numpy as np
 
@@ -88,7 +88,7 @@ def cpu_baseline(workload, sample_batch, budget_s=20.0):
     step()  # first touch / thread start-up
     times = []
     t_begin = time.perf_counter()
-    while len(times) < 5 and (time.perf_counter() - t_begin < budget_s or not times):
+    while len(times) < 15 and (time.perf_counter() - t_begin < budget_s or not times):  # about 10 s of CPU work
         t0 = time.perf_counter()
         step()
         times.append(time.perf_counter() - t0)
