@@ -356,6 +356,16 @@ int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor
                                                  THGPUTensor *finput, THGPUTensor *fgradInput, int kW, int kH,
                                                  int dW, int dH, int padW, int padH, float scale);
 
+/* How the three entry points above compute (no counterpart in the reference, whose only route is
+ * im2col + sgemm + col2im, gpunn-impl/SpatialConvolutionMM.cpp:110-429).  Mode 0: that route, finput
+ * and fgradInput hold the K x N columns as in the reference.  Mode 1: wherever the shape allows, the
+ * GEMMs gather their second operand from a zero-padded copy of the image and no columns exist: finput
+ * then holds the padded input ([B,] C, H+2padH, W+2padW), fgradInput the padded gradOutput and the
+ * flipped kernels; same outputs to fp32 rounding.  The initial mode is 0, or 1 when the environment
+ * has THGPU_CONV=implicit.  set returns 0 or an error for any other mode. */
+int thgpu_conv_set_mode(int mode);
+int thgpu_conv_get_mode(void);
+
 /* nn.SpatialMaxPooling.  Replace gpunn_SpatialMaxPooling_updateOutput /
  * _updateGradInput (gpunn-impl/SpatialMaxPooling.cpp:205-281, 283-383).
  * indices is resized to [2,(B,)C,Ho,Wo] floats, plane 0 = ky+1, plane 1 = kx+1

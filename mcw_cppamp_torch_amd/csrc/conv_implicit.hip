@@ -1,0 +1,257 @@
+// nn.SpatialConvolutionMM without the column buffer: the GEMM's second operand is gathered straight
+// from a zero-padded copy of the image, element (r, x) at rowtab[r] + coltab[x] (gemm_mfma.h), so
+// im2col, col2im and the K x N column buffers (kH*kW times the image) drop out.
+//
+//   forward     output[b][m][n]   = bias[m] + sum_k weight[m][k] * P[b][tap(k) + pixel(n)]
+//   gradWeight  gradWeight[m][k] += scale * sum_b sum_n gradOutput[b][m][n] * P[b][pixel(n) + tap(k)]
+//   gradInput   gradInput[b][c][p] = sum_{m,kh,kw} Wt[c][(m,kh,kw)] * Q[b][tap'(m,kh,kw) + pixel'(p)]   (stride 1)
+//
+// P is the input padded by (padH, padW); tap(c,kh,kw) = c*Hp*Wp + kh*Wp + kw and pixel(ho,wo) =
+// ho*dH*Wp + wo*dW.  Q is gradOutput padded by (kH-1-padH, kW-1-padW) and Wt[c][(m,kh,kw)] =
+// weight[m][c][kH-1-kh][kW-1-kw]: a unit-stride convolution's gradInput is the correlation of the
+// padded gradOutput with the flipped kernels.  The sums run over the same products as
+// gpunn-impl/SpatialConvolutionMM.cpp:110-429 (im2col + sgemm + col2im), in a different order for
+// gradInput.
+#include "gemm_mfma.h"
+#include "kernels.h"
+
+#include <array>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+
+namespace thgpu {
+
+namespace {
+
+// out[plane][y][x] = in[plane][y - pH][x - pW], zero outside; one lane per output element.
+__global__ __launch_bounds__(256) void pad_planes_kernel(const float *__restrict__ in, float *__restrict__ out,
+                                                         unsigned total, int H, int W, int pH, int pW, FastDiv divWp,
+                                                         FastDiv divHp) {
+    const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= total) return;
+    unsigned rest, x, plane, y;
+    divWp.divmod(idx, rest, x);
+    divHp.divmod(rest, plane, y);
+    const int h = (int)y - pH, w = (int)x - pW;
+    float v = 0.0f;
+    if (h >= 0 && h < H && w >= 0 && w < W) v = in[((long)plane * H + h) * W + w];
+    out[idx] = v;
+}
+
+// wt[c][m][kh][kw] = w[m][c][kH-1-kh][kW-1-kw]
+__global__ __launch_bounds__(256) void flip_weight_kernel(const float *__restrict__ w, float *__restrict__ wt, int M,
+                                                          int C, int kH, int kW) {
+    const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+    const unsigned kk = (unsigned)(kH * kW);
+    if (idx >= (unsigned)M * C * kk) return;
+    const unsigned tap = idx % kk, cm = idx / kk;
+    const unsigned m = cm % M, c = cm / M;
+    const unsigned kh = tap / kW, kw = tap % kW;
+    wt[idx] = w[((long)m * C + c) * kk + (kH - 1 - kh) * kW + (kW - 1 - kw)];
+}
+
+// t[(c, kh, kw)] = c*plane + kh*pitch + kw
+__global__ __launch_bounds__(256) void tap_table_kernel(int *__restrict__ t, int planes, int kH, int kW, int plane,
+                                                        int pitch) {
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= planes * kH * kW) return;
+    const int kw = idx % kW, kh = (idx / kW) % kH, c = idx / (kW * kH);
+    t[idx] = c * plane + kh * pitch + kw;
+}
+
+// t[(y, x)] = y*row_step + x*col_step
+__global__ __launch_bounds__(256) void pixel_table_kernel(int *__restrict__ t, int Hn, int Wn, int row_step,
+                                                          int col_step) {
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= Hn * Wn) return;
+    t[idx] = (idx / Wn) * row_step + (idx % Wn) * col_step;
+}
+
+// Offset tables by geometry, built once on the device and kept for the life of the process (a few
+// KB each).  Everything runs on the one library stream, so a table is complete before its first use.
+using TableKey = std::array<int, 6>;
+std::map<TableKey, int *> g_tables;
+
+const int *table(int kind, int a, int b, int c, int d, int e, long count) {
+    const TableKey key{kind, a, b, c, d, e};
+    auto it = g_tables.find(key);
+    if (it != g_tables.end()) return it->second;
+    hipStream_t s = stream();
+    if (!s) return nullptr;
+    if (g_tables.size() >= 512) {  // a caller cycling through geometries: start over
+        if (hipStreamSynchronize(s) != hipSuccess) return nullptr;
+        for (auto &kv : g_tables) (void)hipFree(kv.second);
+        g_tables.clear();
+    }
+    int *t = nullptr;
+    if (hipMalloc(reinterpret_cast<void **>(&t), sizeof(int) * (size_t)count) != hipSuccess) {
+        (void)hipGetLastError();
+        fail("offset table allocation of %ld entries failed", count);
+        return nullptr;
+    }
+    const unsigned blocks = (unsigned)((count + 255) / 256);
+    if (kind == 0)
+        hipLaunchKernelGGL(tap_table_kernel, dim3(blocks), dim3(256), 0, s, t, a, b, c, d, e);
+    else
+        hipLaunchKernelGGL(pixel_table_kernel, dim3(blocks), dim3(256), 0, s, t, a, b, c, d);
+    if (check_launch("conv offset table")) {
+        (void)hipFree(t);
+        return nullptr;
+    }
+    g_tables[key] = t;
+    return t;
+}
+
+const int *tap_table(int planes, int kH, int kW, int plane, int pitch) {
+    return table(0, planes, kH, kW, plane, pitch, (long)planes * kH * kW);
+}
+const int *pixel_table(int Hn, int Wn, int row_step, int col_step) {
+    return table(1, Hn, Wn, row_step, col_step, 0, (long)Hn * Wn);
+}
+
+constexpr long kMaxExtent = 1L << 30;  // floats: the loaders address with 32-bit byte offsets
+
+int g_mode = -1;
+
+}  // namespace
+
+int conv_mode() {
+    if (g_mode < 0) {
+        const char *e = std::getenv("THGPU_CONV");
+        g_mode = (e && std::strcmp(e, "implicit") == 0) ? 1 : 0;
+    }
+    return g_mode;
+}
+
+void conv_set_mode(int mode) { g_mode = mode ? 1 : 0; }
+
+bool conv_implicit_fits(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
+    const long Hp = H + 2L * pH, Wp = W + 2L * pW;
+    const long Ho = (Hp - kH) / sH + 1, Wo = (Wp - kW) / sW + 1;
+    const long K = (long)C * kH * kW, N = Ho * Wo;
+    return M >= 64 && K >= 64 && N >= 16 && B * N >= 64 && B * C * Hp * Wp < kMaxExtent;
+}
+
+bool conv_implicit_gradinput_fits(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
+    if (sH != 1 || sW != 1 || kH - 1 - pH < 0 || kW - 1 - pW < 0) return false;
+    const long Hq = H + kH - 1, Wq = W + kW - 1;
+    return C >= 64 && B * H * W >= 64 && (long)M * kH * kW >= 16 && B * M * Hq * Wq < kMaxExtent &&
+           B * (long)H * W < (1L << 31);
+}
+
+long conv_implicit_gradinput_scratch(long B, int C, int H, int W, int M, int kH, int kW) {
+    return B * M * (H + kH - 1L) * (W + kW - 1L) + (long)C * M * kH * kW;
+}
+
+int pad_planes_launch(const float *in, long planes, int H, int W, int pH, int pW, float *out) {
+    hipStream_t s = stream();
+    if (!s) return 1;
+    const long Hp = H + 2L * pH, Wp = W + 2L * pW;
+    const long total = planes * Hp * Wp;
+    if (total <= 0) return 0;
+    if (total >= (1L << 31)) return fail("pad: %ld elements exceed 32-bit indexing", total);
+    {
+        LaunchScope scope("pad_planes", 0.0, 4.0 * (total + planes * H * W));
+        hipLaunchKernelGGL(pad_planes_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, in, out,
+                           (unsigned)total, H, W, pH, pW, FastDiv((uint32_t)Wp), FastDiv((uint32_t)Hp));
+    }
+    return check_launch("pad_planes");
+}
+
+int conv_implicit_forward(const float *padded, const float *weight, const float *bias, float *output, long B, int C,
+                          int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
+    const int Hp = H + 2 * pH, Wp = W + 2 * pW;
+    const int Ho = (Hp - kH) / sH + 1, Wo = (Wp - kW) / sW + 1;
+    const long N = (long)Ho * Wo;
+    GemmProblem p;
+    p.A = weight;
+    p.a_rc = true;
+    p.sA = (long)C * kH * kW;
+    p.B = padded;
+    p.rowtab = tap_table(C, kH, kW, Hp * Wp, Wp);
+    p.coltab = pixel_table(Ho, Wo, sH * Wp, sW);
+    if (!p.rowtab || !p.coltab) return 1;
+    p.bsB = (long)C * Hp * Wp;
+    p.b_extent = B * p.bsB;
+    p.C = output;
+    p.sC = N;
+    p.bsC = (long)M * N;
+    p.bias = bias;
+    p.M = M;
+    p.J = (int)(B * N);
+    p.N = (int)N;
+    p.R = C * kH * kW;
+    p.tag = "gemm_conv_fwd";
+    return gemm_launch(p);
+}
+
+int conv_implicit_gradweight(const float *padded, const float *gradOutput, float *gradWeight, long B, int C, int H,
+                             int W, int M, int kH, int kW, int pH, int pW, int sH, int sW, float scale) {
+    const int Hp = H + 2 * pH, Wp = W + 2 * pW;
+    const int Ho = (Hp - kH) / sH + 1, Wo = (Wp - kW) / sW + 1;
+    const long N = (long)Ho * Wo;
+    const int K = C * kH * kW;
+    GemmProblem p;
+    p.A = gradOutput;
+    p.a_rc = true;
+    p.sA = N;
+    p.rbA = (long)M * N;
+    p.B = padded;
+    p.rowtab = pixel_table(Ho, Wo, sH * Wp, sW);
+    p.coltab = tap_table(C, kH, kW, Hp * Wp, Wp);
+    if (!p.rowtab || !p.coltab) return 1;
+    p.rbB = (long)C * Hp * Wp;
+    p.b_extent = B * p.rbB;
+    p.C = gradWeight;
+    p.sC = K;
+    p.M = M;
+    p.J = K;
+    p.N = K;
+    p.R = (int)N;
+    p.nb = (int)B;
+    p.alpha = scale;
+    p.beta = 1.0f;
+    p.tag = "gemm_conv_gradweight";
+    return gemm_launch(p);
+}
+
+int conv_implicit_gradinput(const float *gradOutput, const float *weight, float *scratch, float *gradInput, long B,
+                            int C, int H, int W, int M, int kH, int kW, int pH, int pW) {
+    hipStream_t s = stream();
+    if (!s) return 1;
+    const int Ho = H + 2 * pH - kH + 1, Wo = W + 2 * pW - kW + 1;
+    const int qH = kH - 1 - pH, qW = kW - 1 - pW;
+    const int Hq = Ho + 2 * qH, Wq = Wo + 2 * qW;  // = H + kH - 1, W + kW - 1
+    float *Q = scratch;
+    float *Wt = scratch + B * M * (long)Hq * Wq;
+    if (pad_planes_launch(gradOutput, B * M, Ho, Wo, qH, qW, Q)) return 1;
+    const long nw = (long)M * C * kH * kW;
+    {
+        LaunchScope scope("flip_weight", 0.0, 8.0 * nw);
+        hipLaunchKernelGGL(flip_weight_kernel, dim3((unsigned)((nw + 255) / 256)), dim3(256), 0, s, weight, Wt, M, C, kH,
+                           kW);
+    }
+    if (check_launch("flip_weight")) return 1;
+    GemmProblem p;
+    p.A = Wt;
+    p.a_rc = true;
+    p.sA = (long)M * kH * kW;
+    p.B = Q;
+    p.rowtab = tap_table(M, kH, kW, Hq * Wq, Wq);
+    p.coltab = pixel_table(H, W, Wq, 1);
+    if (!p.rowtab || !p.coltab) return 1;
+    p.bsB = (long)M * Hq * Wq;
+    p.b_extent = B * p.bsB;
+    p.C = gradInput;
+    p.sC = (long)H * W;
+    p.bsC = (long)C * H * W;
+    p.M = C;
+    p.J = (int)(B * H * W);
+    p.N = H * W;
+    p.R = M * kH * kW;
+    p.tag = "gemm_conv_gradinput";
+    return gemm_launch(p);
+}
+
+}  // namespace thgpu

@@ -106,7 +106,9 @@ int gemm_launch(const GemmProblem &p) {
     if ((long)p.M * p.J >= (1L << 31)) return fail("gemm: output of %d x %d exceeds 32-bit tile indexing", p.M, p.J);
 
     const bool red = p.nb > 1;
-    if (red && !(p.a_rc && p.b_rc)) return fail("gemm: reduction batching needs r-contiguous operands");
+    const bool gather = p.rowtab != nullptr;
+    if (gather && (!p.coltab || p.b_rc || !p.a_rc)) return fail("gemm: a gathered B needs both tables and an r-contiguous A");
+    if (red && !(p.a_rc && (p.b_rc || gather))) return fail("gemm: reduction batching needs r-contiguous operands");
 
     GemmArgs g;
     std::memset(&g, 0, sizeof(g));
@@ -114,6 +116,8 @@ int gemm_launch(const GemmProblem &p) {
     g.B = p.B;
     g.C = p.C;
     g.bias = p.bias;
+    g.rowtab = p.rowtab;
+    g.coltab = p.coltab;
     g.M = p.M;
     g.J = p.J;
     g.R = p.R;
@@ -150,7 +154,9 @@ int gemm_launch(const GemmProblem &p) {
     auto offsets_fit = [&](int bm, int bn) {
         const long offA = p.a_rc ? (long)(bm - 1) * p.sA + GEMM_BK : (long)(GEMM_BK - 1) * p.sA + bm;
         const long span = (bn - 1) / n_img + 2;  // images a tile's columns can touch
-        const long offB = p.b_rc ? (long)(bn - 1) * p.sB + GEMM_BK : (long)(GEMM_BK - 1) * p.sB + span * p.bsB + n_img;
+        const long offB = gather ? p.b_extent
+                          : p.b_rc ? (long)(bn - 1) * p.sB + GEMM_BK
+                                   : (long)(GEMM_BK - 1) * p.sB + span * p.bsB + n_img;
         const long offC = 4 * (p.sC > p.J ? p.sC : (long)p.J) + span * p.bsC + n_img;
         return offA < (1L << 30) && offB < (1L << 30) && offC < (1L << 30);
     };
@@ -202,7 +208,8 @@ int gemm_launch(const GemmProblem &p) {
 
     // ---- loaders: r-contiguous operands use 128-bit loads (4-byte alignment suffices) --------
     const int la = p.a_rc ? LD_RC_VEC : LD_XC_SCALAR;
-    const int lb = p.b_rc ? LD_RC_VEC : LD_XC_SCALAR;
+    const int lb = p.b_rc ? LD_RC_VEC : gather ? LD_XC_GATHER : LD_XC_SCALAR;
+    if (gather && !best) return fail("gemm: a gathered B needs a shape the tiled kernel takes (M, J >= 64, R >= 16)");
 
     int rc;
     {

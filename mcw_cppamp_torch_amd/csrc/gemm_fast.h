@@ -81,8 +81,12 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     // The kind the A loader really uses: x-contiguous with 192 rows goes block-wise.
     constexpr int KA = (LA == LD_XC_SCALAR && NT % BM != 0) ? LD_XC_BLOCK : LA;
     static_assert(KA != LD_XC_BLOCK || (NT == 256 && BM % 64 == 0 && NA == BM / 16), "block loader shape");
-    static_assert(LB != LD_XC_SCALAR || NT % BN == 0, "x-contiguous loaders give every thread one row/column");
-    static_assert(!RED || (LA != LD_XC_SCALAR && LB != LD_XC_SCALAR), "reduction batching needs r-contiguous operands");
+    static_assert((LB != LD_XC_SCALAR && LB != LD_XC_GATHER) || NT % BN == 0,
+                  "x-contiguous loaders give every thread one row/column");
+    static_assert(LB != LD_XC_GATHER || BN % 64 == 0, "a wavefront of the gathering loader shares its reduction indices");
+    static_assert(LA != LD_XC_GATHER, "only the second operand is gathered");
+    static_assert(!RED || (LA != LD_XC_SCALAR && LB != LD_XC_SCALAR),
+                  "reduction batching needs r-contiguous or gathered operands");
 
     using RowA = LdsRow<KA>;
     using RowB = LdsRow<LB>;
@@ -148,7 +152,15 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         voffA = (unsigned)(((long)a_x * g.sA + a_r) * 4);
         tileA = reinterpret_cast<const char *>(g.A + (long)i0 * g.sA);
     }
-    if (LB == LD_XC_SCALAR) {
+    if (LB == LD_XC_GATHER) {
+        b_x = tid % BN;
+        b_r = (wave * 64 / BN) * NB;  // = (tid / BN) * NB, kept uniform: the row offsets are scalar loads
+        unsigned img0, n0, img, n;
+        g.divN.divmod((unsigned)j0, img0, n0);
+        g.divN.divmod((unsigned)(j0 + b_x), img, n);
+        voffB = (unsigned)(((long)(img - img0) * g.bsB + g.coltab[n]) * 4);
+        tileB = reinterpret_cast<const char *>(g.B + (long)img0 * g.bsB);
+    } else if (LB == LD_XC_SCALAR) {
         b_x = tid % BN;
         b_r = (tid / BN) * NB;
         unsigned img0, n0, img, n;
@@ -174,6 +186,7 @@ __global__ __launch_bounds__(WGM *WGN * 64)
             for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
 
     float ra[NA], rb[NB];
+    int roff[LB == LD_XC_GATHER ? NB : 1];  // gathered B: float offsets of the step's rows (uniform)
 
     // Load number u of an operand for the step whose uniform base is `base`.
     auto load_unit = [&](auto kind_tag, const char *base, long stride, unsigned voff, float *dst, int u) {
@@ -188,6 +201,8 @@ __global__ __launch_bounds__(WGM *WGN * 64)
             dst[u] = *reinterpret_cast<const float *>(base + (long)(u * (NT / 16)) * stride * 4 + voff);
         } else if (KIND == LD_XC_BLOCK) {
             dst[u] = *reinterpret_cast<const float *>(base + (long)(u & 3) * stride * 4 + (u >> 2) * 256 + voff);
+        } else if (KIND == LD_XC_GATHER) {
+            dst[u] = *reinterpret_cast<const float *>(base + (long)roff[u] * 4 + voff);
         } else {
             dst[u] = *reinterpret_cast<const float *>(base + (long)u * stride * 4 + voff);
         }
@@ -201,7 +216,14 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         const int r0 = ld_r0 + BK <= g.R ? ld_r0 : g.R - BK;
         shift = ld_r0 - r0;
         ga = tileA + ((RED ? (long)ld_img * g.rbA : 0L) + (LA == LD_XC_SCALAR ? (long)r0 * g.sA : (long)r0)) * 4;
-        gb = tileB + ((RED ? (long)ld_img * g.rbB : 0L) + (LB == LD_XC_SCALAR ? (long)r0 * g.sB : (long)r0)) * 4;
+        if (LB == LD_XC_GATHER) {
+            gb = tileB + (RED ? (long)ld_img * g.rbB : 0L) * 4;
+            const int *rt = g.rowtab + r0 + b_r;
+#pragma unroll
+            for (int u = 0; u < NB; ++u) roff[u] = rt[u];
+        } else {
+            gb = tileB + ((RED ? (long)ld_img * g.rbB : 0L) + (LB == LD_XC_SCALAR ? (long)r0 * g.sB : (long)r0)) * 4;
+        }
     };
     auto advance = [&]() {
         ld_r0 += BK;
@@ -461,7 +483,7 @@ int gemm_fast_dispatch(const GemmArgs &g, int la, int lb, bool red, hipStream_t 
     if (la == LA_ && lb == LB_) {                                                      \
         if constexpr ((LA_ == LD_XC_SCALAR && (WGM * WGN * 64) % BM != 0 &&            \
                        !((WGM * WGN * 64) == 256 && BM % 64 == 0)) ||                  \
-                      (LB_ == LD_XC_SCALAR && (WGM * WGN * 64) % BN != 0)) {           \
+                      ((LB_ == LD_XC_SCALAR || LB_ == LD_XC_GATHER) && (WGM * WGN * 64) % BN != 0)) { \
             return fail("gemm: this tile has no x-contiguous loader for that side");   \
         } else {                                                                       \
             if (red) {                                                                 \
@@ -476,6 +498,7 @@ int gemm_fast_dispatch(const GemmArgs &g, int la, int lb, bool red, hipStream_t 
     THGPU_CASE(LD_RC_VEC, LD_RC_VEC)
     THGPU_CASE(LD_RC_VEC, LD_RC_SCALAR)
     THGPU_CASE(LD_RC_VEC, LD_XC_SCALAR)
+    THGPU_CASE(LD_RC_VEC, LD_XC_GATHER)
     THGPU_CASE(LD_RC_SCALAR, LD_RC_VEC)
     THGPU_CASE(LD_RC_SCALAR, LD_RC_SCALAR)
     THGPU_CASE(LD_RC_SCALAR, LD_XC_SCALAR)

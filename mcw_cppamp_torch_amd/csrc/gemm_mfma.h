@@ -28,6 +28,11 @@ struct GemmProblem {
     int R = 0;                    // reduction length (per image in reduction batching)
     bool a_rc = true;             // A contiguous along r (else along i)
     bool b_rc = false;            // B contiguous along r (else along j)
+    // Gathered B (implicit im2col): B(r, j) = B[image(j)*bsB + rowtab[r] + coltab[n(j)]] (with reduction batching:
+    // B[image*rbB + rowtab[r] + coltab[j]]).  Needs !b_rc, a_rc and a shape the tiled kernel takes; sB is unused.
+    const int *rowtab = nullptr;  // R entries (floats)
+    const int *coltab = nullptr;  // N entries (floats)
+    long b_extent = 0;            // floats addressable from B (gathered B only; checked against 32-bit offsets)
     long sA = 0;                  // the non-unit stride of A
     long sB = 0;                  // the non-unit stride of B
     long sC = 0;                  // row stride of C
@@ -54,6 +59,7 @@ struct GemmArgs {
     float *C;
     const float *bias;
     float *ws;  // partial sums [nsplit][M][J] when nsplit > 1
+    const int *rowtab, *coltab;  // gathered B
     int M, J, R, N;
     long sA, sB, sC, bsB, bsC, rbA, rbB;
     int nb;
@@ -84,6 +90,8 @@ enum Loader {
     LD_RC_VEC = 0,     // contiguous along r: 128-bit loads along r (rows need 4-byte alignment only)
     LD_RC_SCALAR = 1,  // contiguous along r: 16 lanes read 16 consecutive r, one float each
     LD_XC_SCALAR = 2,  // contiguous along the free index: lanes read consecutive rows/columns
+    // 3 is used inside the kernel (block-wise x-contiguous loads of a 192-row first operand)
+    LD_XC_GATHER = 4,  // second operand only: element (r, x) at rowtab[r] + coltab[x]; lanes run along x
 };
 
 // Launch one tile configuration of the fast kernel (gemm_fast.h).  la/lb are

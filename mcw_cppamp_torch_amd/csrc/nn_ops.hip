@@ -63,6 +63,22 @@ int check_grad_output(const ConvShape &s, const THGPUTensor *gradOutput) {
 // Device pointer of element 0; tensors that reach a kernel are contiguous.
 inline float *dptr(const THGPUTensor *t) { return THGPUTensor_data(t); }
 
+// The padded input a module keeps in finput when it runs without the column buffer:
+// [B,] C, H + 2 padH, W + 2 padW.
+bool is_padded(const THGPUTensor *t, const ConvShape &s, int padH, int padW) {
+    const int o = s.batched ? 1 : 0;
+    return t->nDimension == 3 + o && (!s.batched || t->size[0] == s.B) && t->size[o] == s.C &&
+           t->size[o + 1] == s.H + 2 * padH && t->size[o + 2] == s.W + 2 * padW && THGPUTensor_isContiguous(t);
+}
+int size_padded(THGPUTensor *t, const ConvShape &s, int padH, int padW) {
+    if (s.batched)
+        THGPUTensor_resize4d(t, s.B, s.C, s.H + 2 * padH, s.W + 2 * padW);
+    else
+        THGPUTensor_resize3d(t, s.C, s.H + 2 * padH, s.W + 2 * padW);
+    if (!is_padded(t, s, padH, padW)) return fail("SpatialConvolutionMM: could not size finput");
+    return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -79,18 +95,36 @@ int thgpu_SpatialConvolutionMM_updateOutput(THGPUTensor *input, THGPUTensor *wei
     THGPUTensor *in = THGPUTensor_newContiguous(input);
     if (!in) return 1;
 
-    if (s.batched) {
+    const bool implicit = conv_mode() == 1 && conv_implicit_fits(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW);
+    if (implicit) {
+        // finput holds the padded input instead of the columns
+        if (size_padded(finput, s, padH, padW)) {
+            THGPUTensor_free(in);
+            return 1;
+        }
+    } else if (s.batched) {
         THGPUTensor_resize3d(finput, s.B, s.K, s.N);
-        THGPUTensor_resize4d(output, s.B, s.M, s.Ho, s.Wo);
     } else {
         THGPUTensor_resize2d(finput, s.K, s.N);
-        THGPUTensor_resize3d(output, s.M, s.Ho, s.Wo);
     }
+    if (s.batched)
+        THGPUTensor_resize4d(output, s.B, s.M, s.Ho, s.Wo);
+    else
+        THGPUTensor_resize3d(output, s.M, s.Ho, s.Wo);
     int rc = 0;
     if (!THGPUTensor_isContiguous(finput) || !THGPUTensor_isContiguous(output) ||
-        THGPUTensor_nElement(finput) != s.B * s.K * s.N || THGPUTensor_nElement(output) != s.B * s.M * s.N)
+        (!implicit && THGPUTensor_nElement(finput) != s.B * s.K * s.N) ||
+        THGPUTensor_nElement(output) != s.B * s.M * s.N)
         rc = fail("SpatialConvolutionMM: could not size finput/output");
 
+    if (implicit) {
+        if (!rc) rc = pad_planes_launch(dptr(in), s.B * s.C, s.H, s.W, padH, padW, dptr(finput));
+        if (!rc)
+            rc = conv_implicit_forward(dptr(finput), dptr(weight), dptr(bias), dptr(output), s.B, s.C, s.H, s.W, s.M, kH,
+                                       kW, padH, padW, dH, dW);
+        THGPUTensor_free(in);
+        return rc;
+    }
     if (!rc) rc = im2col_launch(dptr(in), s.B, s.C, s.H, s.W, kH, kW, padH, padW, dH, dW, dptr(finput));
     if (!rc) {
         // output[b][m][n] = bias[m] + sum_k weight[m][k] * finput[b][k][n]
@@ -130,6 +164,24 @@ int thgpu_SpatialConvolutionMM_updateGradInput(THGPUTensor *input, THGPUTensor *
     THGPUTensor *go = THGPUTensor_newContiguous(gradOutput);
     if (!go) return 1;
 
+    if (conv_mode() == 1 && conv_implicit_gradinput_fits(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW)) {
+        // fgradInput holds the padded gradOutput and the flipped kernels instead of the gradient columns
+        const long need = conv_implicit_gradinput_scratch(s.B, s.C, s.H, s.W, s.M, kH, kW);
+        if (s.batched)
+            THGPUTensor_resize4d(gradInput, s.B, s.C, s.H, s.W);
+        else
+            THGPUTensor_resize3d(gradInput, s.C, s.H, s.W);
+        THGPUTensor_resize1d(fgradInput, need);
+        int rc = 0;
+        if (!THGPUTensor_isContiguous(gradInput) || !THGPUTensor_isContiguous(fgradInput) ||
+            THGPUTensor_nElement(fgradInput) != need || THGPUTensor_nElement(gradInput) != s.B * (long)s.C * s.H * s.W)
+            rc = fail("SpatialConvolutionMM: could not size gradInput/fgradInput");
+        if (!rc)
+            rc = conv_implicit_gradinput(dptr(go), dptr(weight), dptr(fgradInput), dptr(gradInput), s.B, s.C, s.H, s.W,
+                                         s.M, kH, kW, padH, padW);
+        THGPUTensor_free(go);
+        return rc;
+    }
     if (s.batched) {
         THGPUTensor_resize4d(gradInput, s.B, s.C, s.H, s.W);
         THGPUTensor_resize3d(fgradInput, s.B, s.K, s.N);
@@ -182,6 +234,22 @@ int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor
     THGPUTensor *go = THGPUTensor_newContiguous(gradOutput);
     if (!go) return 1;
     int rc = 0;
+    if (conv_mode() == 1 && conv_implicit_fits(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW)) {
+        // finput holds the forward's padded input; rebuilt when it does not have that shape
+        if (!is_padded(finput, s, padH, padW)) {
+            THGPUTensor *in = THGPUTensor_newContiguous(input);
+            if (!in) rc = 1;
+            if (!rc) rc = size_padded(finput, s, padH, padW);
+            if (!rc) rc = pad_planes_launch(dptr(in), s.B * s.C, s.H, s.W, padH, padW, dptr(finput));
+            if (in) THGPUTensor_free(in);
+        }
+        if (!rc)
+            rc = conv_implicit_gradweight(dptr(finput), dptr(go), dptr(gradWeight), s.B, s.C, s.H, s.W, s.M, kH, kW,
+                                          padH, padW, dH, dW, scale);
+        if (!rc) rc = gradbias_launch(dptr(go), dptr(gradBias), s.B, s.M, s.N, scale);
+        THGPUTensor_free(go);
+        return rc;
+    }
     // The CPU module reuses the forward's columns (mcw_nn/generic/
     // SpatialConvolutionMM.c:318,336).  If finput does not have the forward's
     // shape (the module was never run forward on this input size) the columns
@@ -317,5 +385,13 @@ int thgpu_Threshold_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput,
     THGPUTensor_free(go);
     return rc;
 }
+
+int thgpu_conv_set_mode(int mode) {
+    if (mode != 0 && mode != 1) return fail("conv mode must be 0 (im2col/GEMM/col2im) or 1 (gathered GEMMs)");
+    conv_set_mode(mode);
+    return 0;
+}
+
+int thgpu_conv_get_mode(void) { return conv_mode(); }
 
 }  // extern "C"
