@@ -1,0 +1,198 @@
+"""GPU parity tests of nn.SpatialConvolutionMM in mode 1 (no column buffer: the GEMMs gather their second
+operand from a zero-padded copy of the image), through the C ABI, against the CPU oracle's
+im2col + sgemm + col2im on identical seeded inputs.
+
+Bars: fp32 outputs and gradients within a norm-wise relative error of 1e-4*sqrt(reduction length); the
+padded input kept in finput bit-exact; repeated runs bit-identical.
+"""
+import numpy as np
+import pytest
+
+from helpers import gemm_tol, oracle_stack, rel_err, rng_for, uniform
+
+pytestmark = pytest.mark.gpu
+
+import oracle  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def gt():
+    import mcw_cppamp_torch_amd as pkg
+    assert pkg._lib.lib.thgpu_init() == 0, pkg._lib.lib.thgpu_last_error()
+    return pkg
+
+
+@pytest.fixture
+def gathered(gt):
+    lib = gt._lib.lib
+    before = lib.thgpu_conv_get_mode()
+    assert lib.thgpu_conv_set_mode(1) == 0
+    yield
+    assert lib.thgpu_conv_set_mode(before) == 0
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+def dev(gt, a):
+    return gt.GPUTensor.from_numpy(np.ascontiguousarray(a, np.float32))
+
+
+def run_conv(gt, x, w, b, go, geo, scale=1.0, gw0=None, gb0=None, forward_first=True):
+    kH, kW, pH, pW, sH, sW = geo
+    M = w.shape[0]
+    C = x.shape[-3]
+    m = gt.nn.SpatialConvolutionMM(C, M, kW, kH, sW, sH, 0, padW=pW, padH=pH)
+    m._assign("weight", w)
+    m._assign("bias", b)
+    m.gradWeight[...] = 0 if gw0 is None else gw0
+    m.gradBias[...] = 0 if gb0 is None else gb0
+    m.gpu()
+    dx, dgo = dev(gt, x), dev(gt, go)
+    out = m.forward(dx).float() if forward_first else None
+    finput = m.finput.float()
+    gi = m.updateGradInput(dx, dgo).float()
+    m.accGradParameters(dx, dgo, scale)
+    return dict(output=out, finput=finput, finput_after=m.finput.float(), gradInput=gi,
+                gradWeight=m.gradWeight.float(), gradBias=m.gradBias.float())
+
+
+def padded(x, pH, pW):
+    return np.pad(x, [(0, 0)] * (x.ndim - 2) + [(pH, pH), (pW, pW)])
+
+
+def reference(x, w, b, go_shape_rng, geo, scale, gw0, gb0):
+    out_ref, finput_ref = oracle.conv_updateOutput(x, w, b, *geo)
+    go = uniform(go_shape_rng, out_ref.shape)
+    gi_ref, _ = oracle.conv_updateGradInput(go, w, x.shape, *geo)
+    gw_ref, gb_ref = gw0.copy(), gb0.copy()
+    oracle.conv_accGradParameters(go, finput_ref, gw_ref, gb_ref, scale)
+    return out_ref, go, gi_ref, gw_ref, gb_ref
+
+
+GATHERED = [
+    # B, C, H, W, M, kH, kW, pH, pW, sH, sW            forward/gradWeight gathered, gradInput gathered
+    (2, 64, 9, 9, 64, 3, 3, 1, 1, 1, 1),               # yes, yes
+    (3, 70, 12, 10, 80, 3, 3, 1, 1, 2, 2),             # yes, no (stride 2)
+    (2, 64, 8, 8, 64, 5, 5, 2, 2, 1, 1),               # yes, yes
+    (1, 64, 16, 16, 96, 3, 3, 0, 0, 1, 1),             # no padding
+    (4, 64, 27, 27, 192, 5, 5, 2, 2, 1, 1),            # AlexNet conv2 shape
+    (1, 384, 13, 13, 256, 3, 3, 1, 1, 1, 1),           # batch 1
+    (2, 64, 20, 17, 128, 7, 3, 3, 1, 1, 1),            # anisotropic kernel and padding
+    (3, 66, 11, 13, 72, 3, 5, 2, 0, 1, 1),             # padding kH-1 in one direction, none in the other
+    (2, 64, 10, 10, 64, 3, 3, 3, 3, 1, 1),             # padding above kH-1: gradInput takes the column route
+    (2, 130, 9, 9, 70, 3, 3, 1, 1, 1, 1),              # nothing a multiple of the tile
+    (5, 67, 23, 19, 65, 4, 2, 1, 0, 3, 2),             # even kernels, strides 3 x 2
+    (16, 3, 224, 224, 64, 11, 11, 2, 2, 4, 4),         # first benchmark configuration, full size
+    (2, 48, 12, 12, 64, 3, 3, 1, 1, 1, 1),             # C < 64: forward gathered, gradInput by columns
+    (2, 64, 12, 12, 48, 3, 3, 1, 1, 1, 1),             # M < 64: forward by columns, gradInput gathered
+]
+
+
+@pytest.mark.parametrize("cfg", GATHERED)
+def test_gathered_conv_fwd_bwd_parity(gt, gathered, cfg):
+    B, C, H, W, M, kH, kW, pH, pW, sH, sW = cfg
+    geo = (kH, kW, pH, pW, sH, sW)
+    K = C * kH * kW
+    rng = rng_for(41)
+    s = 1.0 / np.sqrt(K)
+    x = uniform(rng, (B, C, H, W))
+    w, b = uniform(rng, (M, K), -s, s), uniform(rng, (M,), -s, s)
+    gw0, gb0 = uniform(rng, (M, K)), uniform(rng, (M,))
+    scale = 0.5
+    out_ref, go, gi_ref, gw_ref, gb_ref = reference(x, w, b, rng, geo, scale, gw0, gb0)
+    got = run_conv(gt, x, w, b, go, geo, scale, gw0, gb0)
+    N = out_ref.shape[2] * out_ref.shape[3]
+    if M >= 64 and K >= 64:
+        assert np.array_equal(bits(got["finput"]), bits(padded(x, pH, pW)))   # the padded input, not columns
+    else:
+        assert got["finput"].shape == (B, K, N)
+    assert rel_err(got["output"], out_ref) < gemm_tol(K)
+    assert rel_err(got["gradInput"], gi_ref) < gemm_tol(M * kH * kW)
+    assert rel_err(got["gradWeight"], gw_ref) < gemm_tol(B * N)
+    assert rel_err(got["gradBias"], gb_ref) < gemm_tol(B * N)
+
+
+def test_gathered_matches_column_route_and_reruns_identically(gt, gathered):
+    B, C, H, W, M, kH, kW = 3, 64, 14, 15, 96, 3, 5
+    geo = (kH, kW, 1, 2, 1, 1)
+    rng = rng_for(42)
+    x, w, b = uniform(rng, (B, C, H, W)), uniform(rng, (M, C * kH * kW), -0.05, 0.05), uniform(rng, (M,))
+    ref, _ = oracle.conv_updateOutput(x, w, b, *geo)
+    go = uniform(rng, ref.shape)
+    a = run_conv(gt, x, w, b, go, geo)
+    a2 = run_conv(gt, x, w, b, go, geo)
+    for k in a:
+        assert np.array_equal(bits(a[k]), bits(a2[k])), k   # deterministic: no atomics anywhere
+    lib = gt._lib.lib
+    assert lib.thgpu_conv_set_mode(0) == 0
+    try:
+        c = run_conv(gt, x, w, b, go, geo)
+    finally:
+        assert lib.thgpu_conv_set_mode(1) == 0
+    assert c["finput"].shape == (B, C * kH * kW, ref.shape[2] * ref.shape[3])
+    for k in ("output", "gradInput", "gradWeight", "gradBias"):
+        assert rel_err(a[k], c[k]) < 1e-5, k
+
+
+def test_gathered_non_batch_input(gt, gathered):
+    C, H, W, M, kH, kW = 64, 12, 11, 64, 3, 3
+    geo = (kH, kW, 1, 1, 1, 1)
+    rng = rng_for(43)
+    x, w, b = uniform(rng, (C, H, W)), uniform(rng, (M, C * kH * kW), -0.05, 0.05), uniform(rng, (M,))
+    gw0, gb0 = np.zeros((M, C * kH * kW), np.float32), np.zeros((M,), np.float32)
+    out_ref, go, gi_ref, gw_ref, gb_ref = reference(x[None], w, b, rng, geo, 1.0, gw0, gb0)
+    got = run_conv(gt, x, w, b, go[0], geo)
+    assert got["output"].shape == out_ref.shape[1:] and got["gradInput"].shape == x.shape
+    assert got["finput"].shape == (C, H + 2, W + 2)
+    assert rel_err(got["output"], out_ref[0]) < gemm_tol(C * kH * kW)
+    assert rel_err(got["gradInput"], gi_ref[0]) < gemm_tol(M * kH * kW)
+    assert rel_err(got["gradWeight"], gw_ref) < gemm_tol(H * W)
+
+
+def test_gathered_gradweight_without_forward_rebuilds_the_padded_input(gt, gathered):
+    B, C, H, W, M, kH, kW = 2, 64, 10, 9, 64, 3, 3
+    geo = (kH, kW, 1, 1, 1, 1)
+    rng = rng_for(44)
+    x, w, b = uniform(rng, (B, C, H, W)), uniform(rng, (M, C * kH * kW), -0.05, 0.05), uniform(rng, (M,))
+    gw0, gb0 = uniform(rng, (M, C * kH * kW)), uniform(rng, (M,))
+    out_ref, go, gi_ref, gw_ref, gb_ref = reference(x, w, b, rng, geo, 2.0, gw0, gb0)
+    got = run_conv(gt, x, w, b, go, geo, 2.0, gw0, gb0, forward_first=False)
+    assert got["finput"].shape != (B, C, H + 2, W + 2)   # no forward pass has filled it
+    assert np.array_equal(bits(got["finput_after"]), bits(padded(x, 1, 1)))
+    assert rel_err(got["gradWeight"], gw_ref) < gemm_tol(B * H * W)
+    assert rel_err(got["gradBias"], gb_ref) < gemm_tol(B * H * W)
+    assert rel_err(got["gradInput"], gi_ref) < gemm_tol(M * kH * kW)
+
+
+def test_conv_mode_api(gt):
+    lib = gt._lib.lib
+    before = lib.thgpu_conv_get_mode()
+    assert before in (0, 1)
+    assert lib.thgpu_conv_set_mode(2) != 0 and b"mode" in lib.thgpu_last_error()
+    assert lib.thgpu_conv_get_mode() == before
+    assert lib.thgpu_conv_set_mode(1) == 0 and lib.thgpu_conv_get_mode() == 1
+    assert lib.thgpu_conv_set_mode(0) == 0 and lib.thgpu_conv_get_mode() == 0
+    assert lib.thgpu_conv_set_mode(before) == 0
+
+
+def test_gathered_alexnet_stack_matches_oracle(gt, gathered):
+    stacks = gt.stacks
+    name, B = "alexnet", 2
+    layers = stacks.STACKS[name]["layers"]
+    net = stacks.build(name, seed_base=2100)
+    params = [(np.array(m.weight), np.array(m.bias)) if hasattr(m, "weight") else None for m in net.modules]
+    x = stacks.make_input(name, B, seed=2100)
+    go = uniform(rng_for(2103), stacks.output_shape(name, B))
+    outs, gins, grads = oracle_stack(layers, params, x, go)
+    net.gpu()
+    dx = dev(gt, x)
+    out = net.forward(dx).float()
+    gi = net.backward(dx, dev(gt, go)).float()
+    assert rel_err(out, outs[-1]) < 1e-3
+    assert rel_err(gi, gins[0]) < 5e-3
+    for m, g in zip(net.modules, grads):
+        if g is not None:
+            assert rel_err(m.gradWeight.float(), g[0]) < 5e-3
+            assert rel_err(m.gradBias.float(), g[1]) < 5e-3
