@@ -357,12 +357,16 @@ int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor
                                                  int dW, int dH, int padW, int padH, float scale);
 
 /* How the three entry points above compute (no counterpart in the reference, whose only route is
- * im2col + sgemm + col2im, gpunn-impl/SpatialConvolutionMM.cpp:110-429).  Mode 0: that route, finput
- * and fgradInput hold the K x N columns as in the reference.  Mode 1: wherever the shape allows, the
- * GEMMs gather their second operand from a zero-padded copy of the image and no columns exist: finput
- * then holds the padded input ([B,] C, H+2padH, W+2padW), fgradInput the padded gradOutput and the
- * flipped kernels; same outputs to fp32 rounding.  The initial mode is 0, or 1 when the environment
- * has THGPU_CONV=implicit.  set returns 0 or an error for any other mode. */
+ * im2col + sgemm + col2im, gpunn-impl/SpatialConvolutionMM.cpp:110-429).
+ *   mode 0: that route; finput and fgradInput hold the K x N columns as in the reference.
+ *   mode 1 (initial): per layer and pass, the GEMM gathers its second operand from a zero-padded copy
+ *           of the image and no columns exist, where the shape allows it and it is the faster route
+ *           (layers with fewer than 512 output planes); the column route otherwise.
+ *   mode 2: gathered wherever the shape allows it.
+ * On the gathered route finput holds the padded input ([B,] C, H+2padH, W+2padW) and fgradInput the
+ * padded gradOutput followed by the flipped kernels; outputs and gradients are the same sums of the
+ * same products, equal to the column route's to fp32 rounding.  The environment variable THGPU_CONV
+ * (columns | auto | gathered) sets the initial mode.  set returns 0, or an error for any other mode. */
 int thgpu_conv_set_mode(int mode);
 int thgpu_conv_get_mode(void);
 

@@ -24,19 +24,35 @@ namespace thgpu {
 
 namespace {
 
-// out[plane][y][x] = in[plane][y - pH][x - pW], zero outside; one lane per output element.
+// out[plane][y][x] = in[plane][y - pH][x - pW], zero outside.  A lane produces four consecutive
+// output elements (one 128-bit store; single stores at the end of an odd-sized buffer or into an unaligned one).
 __global__ __launch_bounds__(256) void pad_planes_kernel(const float *__restrict__ in, float *__restrict__ out,
-                                                         unsigned total, int H, int W, int pH, int pW, FastDiv divWp,
-                                                         FastDiv divHp) {
-    const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+                                                         unsigned total, int H, int W, int pH, int pW, int Hp, int Wp,
+                                                         FastDiv divWp, FastDiv divHp, bool aligned) {
+    const unsigned idx = (blockIdx.x * 256u + threadIdx.x) * 4u;
     if (idx >= total) return;
     unsigned rest, x, plane, y;
     divWp.divmod(idx, rest, x);
     divHp.divmod(rest, plane, y);
-    const int h = (int)y - pH, w = (int)x - pW;
-    float v = 0.0f;
-    if (h >= 0 && h < H && w >= 0 && w < W) v = in[((long)plane * H + h) * W + w];
-    out[idx] = v;
+    float v[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int h = (int)y - pH, w = (int)x - pW;
+        v[q] = 0.0f;
+        if (h >= 0 && h < H && w >= 0 && w < W && idx + q < total) v[q] = in[((long)plane * H + h) * W + w];
+        if (++x == (unsigned)Wp) {
+            x = 0;
+            if (++y == (unsigned)Hp) {
+                y = 0;
+                ++plane;
+            }
+        }
+    }
+    if (aligned && idx + 4 <= total) {
+        *reinterpret_cast<float4 *>(out + idx) = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+        for (unsigned q = 0; idx + q < total; ++q) out[idx + q] = v[q];
+    }
 }
 
 // wt[c][m][kh][kw] = w[m][c][kH-1-kh][kW-1-kw]
@@ -119,25 +135,46 @@ int g_mode = -1;
 int conv_mode() {
     if (g_mode < 0) {
         const char *e = std::getenv("THGPU_CONV");
-        g_mode = (e && std::strcmp(e, "implicit") == 0) ? 1 : 0;
+        g_mode = !e ? 1 : std::strcmp(e, "columns") == 0 ? 0 : std::strcmp(e, "gathered") == 0 ? 2 : 1;
     }
     return g_mode;
 }
 
-void conv_set_mode(int mode) { g_mode = mode ? 1 : 0; }
+void conv_set_mode(int mode) { g_mode = mode; }
 
-bool conv_implicit_fits(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
+// Shapes the gathered GEMMs take: a tile of the fast kernel must fit (M, J >= 64, R >= 16) and the padded
+// batch must stay within 32-bit byte offsets.
+static bool forward_fits(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
     const long Hp = H + 2L * pH, Wp = W + 2L * pW;
     const long Ho = (Hp - kH) / sH + 1, Wo = (Wp - kW) / sW + 1;
     const long K = (long)C * kH * kW, N = Ho * Wo;
     return M >= 64 && K >= 64 && N >= 16 && B * N >= 64 && B * C * Hp * Wp < kMaxExtent;
 }
 
-bool conv_implicit_gradinput_fits(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
+static bool gradinput_fits(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
     if (sH != 1 || sW != 1 || kH - 1 - pH < 0 || kW - 1 - pW < 0) return false;
     const long Hq = H + kH - 1, Wq = W + kW - 1;
     return C >= 64 && B * H * W >= 64 && (long)M * kH * kW >= 16 && B * M * Hq * Wq < kMaxExtent &&
            B * (long)H * W < (1L << 31);
+}
+
+// Where the gathered route pays (measured on the AlexNet-, OverFeat- and VGG-style layers): the column
+// traffic it saves is proportional to K*N, the GEMM time it costs (the gathered gradWeight product runs
+// about 8 % under the one on r-contiguous columns; a gradInput product with few output planes leaves the
+// column route's GEMM a short reduction) to M*K*N, so it wins for layers with fewer than about 512
+// output planes and is a wash or a loss above.  The gathered gradInput product has one row per input
+// plane, so it also wants C to fill its 64-row tiles.
+bool conv_use_gathered(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
+    const int mode = conv_mode();
+    if (mode == 0 || !forward_fits(B, C, H, W, M, kH, kW, pH, pW, sH, sW)) return false;
+    return mode == 2 || M < 512;
+}
+
+bool conv_use_gathered_gradinput(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
+    const int mode = conv_mode();
+    if (mode == 0 || !gradinput_fits(B, C, H, W, M, kH, kW, pH, pW, sH, sW)) return false;
+    const long rows = (C + 63L) / 64 * 64;
+    return mode == 2 || (M < 512 && rows * 8 <= C * 9L);
 }
 
 long conv_implicit_gradinput_scratch(long B, int C, int H, int W, int M, int kH, int kW) {
@@ -153,8 +190,9 @@ int pad_planes_launch(const float *in, long planes, int H, int W, int pH, int pW
     if (total >= (1L << 31)) return fail("pad: %ld elements exceed 32-bit indexing", total);
     {
         LaunchScope scope("pad_planes", 0.0, 4.0 * (total + planes * H * W));
-        hipLaunchKernelGGL(pad_planes_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, in, out,
-                           (unsigned)total, H, W, pH, pW, FastDiv((uint32_t)Wp), FastDiv((uint32_t)Hp));
+        hipLaunchKernelGGL(pad_planes_kernel, dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0, s, in, out,
+                           (unsigned)total, H, W, pH, pW, (int)Hp, (int)Wp, FastDiv((uint32_t)Wp),
+                           FastDiv((uint32_t)Hp), (reinterpret_cast<uintptr_t>(out) & 15) == 0);
     }
     return check_launch("pad_planes");
 }

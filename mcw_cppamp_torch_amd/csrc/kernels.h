@@ -19,12 +19,14 @@ int threshold_bwd_launch(const float *in, const float *gout, float *gin, long n,
 int gradbias_launch(const float *gout, float *gbias, long B, int M, long N, float scale);
 
 // Convolution without the column buffer (conv_implicit.hip).  conv_mode: 0 = im2col / GEMM / col2im,
-// 1 = gathered GEMMs wherever the shape fits.  `padded` is the input padded by (pH, pW), B*C planes of
-// (H+2pH) x (W+2pW); `scratch` takes conv_implicit_gradinput_scratch floats.
+// 1 = gathered GEMMs where the shape fits and the route pays, 2 = wherever the shape fits.  The two
+// predicates answer for the current mode: forward and gradWeight go together (they share finput),
+// gradInput on its own.  `padded` is the input padded by (pH, pW), B*C planes of (H+2pH) x (W+2pW);
+// `scratch` takes conv_implicit_gradinput_scratch floats.
 int conv_mode();
 void conv_set_mode(int mode);
-bool conv_implicit_fits(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW);
-bool conv_implicit_gradinput_fits(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW);
+bool conv_use_gathered(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW);
+bool conv_use_gathered_gradinput(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW);
 long conv_implicit_gradinput_scratch(long B, int C, int H, int W, int M, int kH, int kW);
 int pad_planes_launch(const float *in, long planes, int H, int W, int pH, int pW, float *out);
 int conv_implicit_forward(const float *padded, const float *weight, const float *bias, float *output, long B, int C,

@@ -95,7 +95,7 @@ int thgpu_SpatialConvolutionMM_updateOutput(THGPUTensor *input, THGPUTensor *wei
     THGPUTensor *in = THGPUTensor_newContiguous(input);
     if (!in) return 1;
 
-    const bool implicit = conv_mode() == 1 && conv_implicit_fits(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW);
+    const bool implicit = conv_use_gathered(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW);
     if (implicit) {
         // finput holds the padded input instead of the columns
         if (size_padded(finput, s, padH, padW)) {
@@ -164,7 +164,7 @@ int thgpu_SpatialConvolutionMM_updateGradInput(THGPUTensor *input, THGPUTensor *
     THGPUTensor *go = THGPUTensor_newContiguous(gradOutput);
     if (!go) return 1;
 
-    if (conv_mode() == 1 && conv_implicit_gradinput_fits(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW)) {
+    if (conv_use_gathered_gradinput(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW)) {
         // fgradInput holds the padded gradOutput and the flipped kernels instead of the gradient columns
         const long need = conv_implicit_gradinput_scratch(s.B, s.C, s.H, s.W, s.M, kH, kW);
         if (s.batched)
@@ -234,7 +234,7 @@ int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor
     THGPUTensor *go = THGPUTensor_newContiguous(gradOutput);
     if (!go) return 1;
     int rc = 0;
-    if (conv_mode() == 1 && conv_implicit_fits(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW)) {
+    if (conv_use_gathered(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW)) {
         // finput holds the forward's padded input; rebuilt when it does not have that shape
         if (!is_padded(finput, s, padH, padW)) {
             THGPUTensor *in = THGPUTensor_newContiguous(input);
@@ -387,7 +387,8 @@ int thgpu_Threshold_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput,
 }
 
 int thgpu_conv_set_mode(int mode) {
-    if (mode != 0 && mode != 1) return fail("conv mode must be 0 (im2col/GEMM/col2im) or 1 (gathered GEMMs)");
+    if (mode < 0 || mode > 2)
+        return fail("conv mode must be 0 (columns), 1 (gathered where it pays) or 2 (gathered where it fits)");
     conv_set_mode(mode);
     return 0;
 }

@@ -10,3 +10,20 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+def _conv_mode_fixture(mode):
+    @pytest.fixture
+    def fixture():
+        """Runs the test with nn.SpatialConvolutionMM on one route, then restores the library's mode."""
+        import mcw_cppamp_torch_amd as pkg
+        lib = pkg._lib.lib
+        before = lib.thgpu_conv_get_mode()
+        assert lib.thgpu_conv_set_mode(mode) == 0
+        yield
+        assert lib.thgpu_conv_set_mode(before) == 0
+    return fixture
+
+
+columns_route = _conv_mode_fixture(0)    # im2col / GEMM / col2im: finput and fgradInput hold columns
+gathered_route = _conv_mode_fixture(2)   # gathered GEMMs wherever the shape fits

@@ -22,15 +22,6 @@ def gt():
     return pkg
 
 
-@pytest.fixture
-def gathered(gt):
-    lib = gt._lib.lib
-    before = lib.thgpu_conv_get_mode()
-    assert lib.thgpu_conv_set_mode(1) == 0
-    yield
-    assert lib.thgpu_conv_set_mode(before) == 0
-
-
 def bits(a):
     return np.ascontiguousarray(a, np.float32).view(np.uint32)
 
@@ -91,7 +82,7 @@ GATHERED = [
 
 
 @pytest.mark.parametrize("cfg", GATHERED)
-def test_gathered_conv_fwd_bwd_parity(gt, gathered, cfg):
+def test_gathered_conv_fwd_bwd_parity(gt, gathered_route, cfg):
     B, C, H, W, M, kH, kW, pH, pW, sH, sW = cfg
     geo = (kH, kW, pH, pW, sH, sW)
     K = C * kH * kW
@@ -114,7 +105,7 @@ def test_gathered_conv_fwd_bwd_parity(gt, gathered, cfg):
     assert rel_err(got["gradBias"], gb_ref) < gemm_tol(B * N)
 
 
-def test_gathered_matches_column_route_and_reruns_identically(gt, gathered):
+def test_gathered_matches_column_route_and_reruns_identically(gt, gathered_route):
     B, C, H, W, M, kH, kW = 3, 64, 14, 15, 96, 3, 5
     geo = (kH, kW, 1, 2, 1, 1)
     rng = rng_for(42)
@@ -130,13 +121,13 @@ def test_gathered_matches_column_route_and_reruns_identically(gt, gathered):
     try:
         c = run_conv(gt, x, w, b, go, geo)
     finally:
-        assert lib.thgpu_conv_set_mode(1) == 0
+        assert lib.thgpu_conv_set_mode(2) == 0
     assert c["finput"].shape == (B, C * kH * kW, ref.shape[2] * ref.shape[3])
     for k in ("output", "gradInput", "gradWeight", "gradBias"):
         assert rel_err(a[k], c[k]) < 1e-5, k
 
 
-def test_gathered_non_batch_input(gt, gathered):
+def test_gathered_non_batch_input(gt, gathered_route):
     C, H, W, M, kH, kW = 64, 12, 11, 64, 3, 3
     geo = (kH, kW, 1, 1, 1, 1)
     rng = rng_for(43)
@@ -151,7 +142,7 @@ def test_gathered_non_batch_input(gt, gathered):
     assert rel_err(got["gradWeight"], gw_ref) < gemm_tol(H * W)
 
 
-def test_gathered_gradweight_without_forward_rebuilds_the_padded_input(gt, gathered):
+def test_gathered_gradweight_without_forward_rebuilds_the_padded_input(gt, gathered_route):
     B, C, H, W, M, kH, kW = 2, 64, 10, 9, 64, 3, 3
     geo = (kH, kW, 1, 1, 1, 1)
     rng = rng_for(44)
@@ -166,18 +157,79 @@ def test_gathered_gradweight_without_forward_rebuilds_the_padded_input(gt, gathe
     assert rel_err(got["gradInput"], gi_ref) < gemm_tol(M * kH * kW)
 
 
+def random_gathered_geometries(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < n:
+        kH, kW = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        sH, sW = (1, 1) if rng.random() < 0.6 else (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        pH, pW = int(rng.integers(0, kH + 1)), int(rng.integers(0, kW + 1))
+        C, M = int(rng.integers(64, 150)), int(rng.integers(64, 150))
+        H, W = int(rng.integers(6, 20)), int(rng.integers(6, 20))
+        B = int(rng.integers(1, 4))
+        if H + 2 * pH < kH or W + 2 * pW < kW:
+            continue
+        Ho, Wo = (H + 2 * pH - kH) // sH + 1, (W + 2 * pW - kW) // sW + 1
+        if Ho * Wo < 16 or B * Ho * Wo < 64:
+            continue
+        out.append((B, C, H, W, M, kH, kW, pH, pW, sH, sW))
+    return out
+
+
+@pytest.mark.parametrize("cfg", random_gathered_geometries(24, 2101))
+def test_gathered_conv_random_geometry(gt, gathered_route, cfg):
+    B, C, H, W, M, kH, kW, pH, pW, sH, sW = cfg
+    geo = (kH, kW, pH, pW, sH, sW)
+    K = C * kH * kW
+    rng = rng_for(45)
+    s = 1.0 / np.sqrt(K)
+    x = uniform(rng, (B, C, H, W))
+    w, b = uniform(rng, (M, K), -s, s), uniform(rng, (M,), -s, s)
+    gw0, gb0 = uniform(rng, (M, K)), uniform(rng, (M,))
+    out_ref, go, gi_ref, gw_ref, gb_ref = reference(x, w, b, rng, geo, 1.5, gw0, gb0)
+    got = run_conv(gt, x, w, b, go, geo, 1.5, gw0, gb0)
+    N = out_ref.shape[2] * out_ref.shape[3]
+    assert np.array_equal(bits(got["finput"]), bits(padded(x, pH, pW)))
+    assert rel_err(got["output"], out_ref) < gemm_tol(K)
+    assert rel_err(got["gradInput"], gi_ref) < gemm_tol(M * kH * kW)
+    assert rel_err(got["gradWeight"], gw_ref) < gemm_tol(B * N)
+    assert rel_err(got["gradBias"], gb_ref) < gemm_tol(B * N)
+
+
+def test_mode_1_gathers_narrow_layers_only(gt):
+    lib = gt._lib.lib
+    before = lib.thgpu_conv_get_mode()
+    assert lib.thgpu_conv_set_mode(1) == 0
+    try:
+        rng = rng_for(46)
+        for M, gathers in ((128, True), (512, False)):
+            B, C, H, W, kH, kW = 2, 64, 8, 8, 3, 3
+            geo = (kH, kW, 1, 1, 1, 1)
+            x, w, b = uniform(rng, (B, C, H, W)), uniform(rng, (M, C * kH * kW), -0.05, 0.05), uniform(rng, (M,))
+            gw0, gb0 = np.zeros((M, C * kH * kW), np.float32), np.zeros((M,), np.float32)
+            out_ref, go, gi_ref, gw_ref, gb_ref = reference(x, w, b, rng, geo, 1.0, gw0, gb0)
+            got = run_conv(gt, x, w, b, go, geo)
+            assert got["finput"].shape == ((B, C, H + 2, W + 2) if gathers else (B, C * kH * kW, H * W))
+            assert rel_err(got["output"], out_ref) < gemm_tol(C * kH * kW)
+            assert rel_err(got["gradInput"], gi_ref) < gemm_tol(M * kH * kW)
+            assert rel_err(got["gradWeight"], gw_ref) < gemm_tol(B * H * W)
+    finally:
+        assert lib.thgpu_conv_set_mode(before) == 0
+
+
 def test_conv_mode_api(gt):
     lib = gt._lib.lib
     before = lib.thgpu_conv_get_mode()
-    assert before in (0, 1)
-    assert lib.thgpu_conv_set_mode(2) != 0 and b"mode" in lib.thgpu_last_error()
-    assert lib.thgpu_conv_get_mode() == before
-    assert lib.thgpu_conv_set_mode(1) == 0 and lib.thgpu_conv_get_mode() == 1
-    assert lib.thgpu_conv_set_mode(0) == 0 and lib.thgpu_conv_get_mode() == 0
+    assert before in (0, 1, 2)
+    for bad in (-1, 3):
+        assert lib.thgpu_conv_set_mode(bad) != 0 and b"mode" in lib.thgpu_last_error()
+        assert lib.thgpu_conv_get_mode() == before
+    for mode in (2, 1, 0):
+        assert lib.thgpu_conv_set_mode(mode) == 0 and lib.thgpu_conv_get_mode() == mode
     assert lib.thgpu_conv_set_mode(before) == 0
 
 
-def test_gathered_alexnet_stack_matches_oracle(gt, gathered):
+def test_gathered_alexnet_stack_matches_oracle(gt, gathered_route):
     stacks = gt.stacks
     name, B = "alexnet", 2
     layers = stacks.STACKS[name]["layers"]

@@ -14,7 +14,8 @@ import pytest
 from helpers import (check_digest, gemm_tol, kat_conv_inputs, kat_pool_inputs, load_kat, oracle_stack, rel_err,
                      rng_for, uniform)
 
-pytestmark = pytest.mark.gpu
+# These tests check the column buffers too, so they pin the column route.
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("columns_route")]
 
 import oracle  # noqa: E402
 

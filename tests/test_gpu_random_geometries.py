@@ -13,7 +13,8 @@ import pytest
 import oracle
 from helpers import gemm_tol, rel_err, uniform
 
-pytestmark = pytest.mark.gpu
+# These tests check the column buffers too, so they pin the column route.
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("columns_route")]
 
 
 @pytest.fixture(scope="module")

@@ -6,8 +6,10 @@ gradOutput of its layer, so a layer's result is compared at the strict bar and
 does not inherit the rounding of the layers before it:
   * conv output / gradInput / gradWeight / gradBias within 1e-4*sqrt(reduction
     length) (max error relative to the largest reference magnitude);
-  * the im2col buffer, max-pool output, argmax-driven gradient and ReLU
-    bit-exact.
+  * the im2col buffer (on the gathered route: the zero-padded input), max-pool
+    output, argmax-driven gradient and ReLU bit-exact.
+Every stack runs on the column route (mode 0) and with the library choosing the
+route per layer (mode 1, its initial mode).
 The oracle's sgemm runs on the host BLAS here (tests/test_oracle_math.py pins
 that path against the reference's plain loops).
 """
@@ -36,20 +38,45 @@ def dev(gt, a):
     return gt.GPUTensor.from_numpy(np.ascontiguousarray(a, np.float32))
 
 
+_oracle_runs = {}
+
+
+def oracle_run(stacks, name):
+    """Forward + backward of a stack through the oracle, once per stack for the module."""
+    if name not in _oracle_runs:
+        cfg = stacks.STACKS[name]
+        B, layers = cfg["batch"], cfg["layers"]
+        net = stacks.build(name, seed_base=4000)
+        params = [(np.array(m.weight), np.array(m.bias)) if hasattr(m, "weight") else None for m in net.modules]
+        x = stacks.make_input(name, B, seed=4000)
+        go = uniform(rng_for(4003), stacks.output_shape(name, B))
+        oracle.use_blas(True)
+        try:
+            outs, gins, grads = oracle_stack(layers, params, x, go)
+        finally:
+            oracle.use_blas(False)
+        _oracle_runs[name] = (x, go, outs, gins, grads)
+    return _oracle_runs[name]
+
+
+@pytest.mark.parametrize("mode", [0, 1], ids=["columns", "auto"])
 @pytest.mark.parametrize("name", ["alexnet", "overfeat", "vgg_a"])
-def test_full_size_stack_layerwise(gt, name):
+def test_full_size_stack_layerwise(gt, name, mode):
     stacks = gt.stacks
     cfg = stacks.STACKS[name]
     B, layers = cfg["batch"], cfg["layers"]
+    x, go, outs, gins, grads = oracle_run(stacks, name)
     net = stacks.build(name, seed_base=4000)
-    params = [(np.array(m.weight), np.array(m.bias)) if hasattr(m, "weight") else None for m in net.modules]
-    x = stacks.make_input(name, B, seed=4000)
-    go = uniform(rng_for(4003), stacks.output_shape(name, B))
-    oracle.use_blas(True)
+    lib = gt._lib.lib
+    before = lib.thgpu_conv_get_mode()
+    assert lib.thgpu_conv_set_mode(mode) == 0
     try:
-        outs, gins, grads = oracle_stack(layers, params, x, go)
+        check_layers(gt, name, net, layers, B, x, go, outs, gins, grads, mode)
     finally:
-        oracle.use_blas(False)
+        assert lib.thgpu_conv_set_mode(before) == 0
+
+
+def check_layers(gt, name, net, layers, B, x, go, outs, gins, grads, mode):
     net.gpu()
     ins = [x] + outs[:-1]
     gouts = gins[1:] + [go]
@@ -64,10 +91,15 @@ def test_full_size_stack_layerwise(gt, name):
             K = cin * kH * kW
             N = outs[i].shape[2] * outs[i].shape[3]
             assert rel_err(out, outs[i]) < gemm_tol(K), (name, i)
-            assert rel_err(gi, gins[i]) < gemm_tol(cout), (name, i)
+            gathered = m.finput.dim() == 4   # [B, C, H+2pH, W+2pW] instead of [B, K, N]
+            # the gathered gradInput product sums over (plane, tap) at once, the column route over planes
+            assert rel_err(gi, gins[i]) < gemm_tol(cout if mode == 0 else cout * kH * kW), (name, i)
             assert rel_err(m.gradWeight.float(), grads[i][0]) < gemm_tol(B * N), (name, i)
             assert rel_err(m.gradBias.float(), grads[i][1]) < gemm_tol(B * N), (name, i)
-            if B * K * N * 4 <= (1 << 30):  # the column buffer, where the copy back stays modest
+            if gathered:
+                ref_pad = np.pad(ins[i], [(0, 0), (0, 0), (pH, pH), (pW, pW)])
+                assert np.array_equal(bits(m.finput.float()), bits(ref_pad)), (name, i)
+            elif B * K * N * 4 <= (1 << 30):  # the column buffer, where the copy back stays modest
                 ref_cols = oracle.im2col(ins[i], kH, kW, pH, pW, dH, dW)
                 assert np.array_equal(bits(m.finput.float()), bits(ref_cols)), (name, i)
         else:
