@@ -16,6 +16,11 @@ Beside the throughput the line carries
   gemm_shapes   every GEMM of the stack on its own (shape, chosen tile and split,
                 TFLOP/s): the small-K GEMMs of first layers are HBM-bound themselves;
   hbm_shapes    every im2col / col2im / pooling launch geometry on its own (GB/s);
+  column_route  the same steps once more with every convolution on the reference's
+                route (im2col, GEMM, col2im): throughput, GEMM roofline, and the
+                im2col / col2im figures at the workload's full geometries.  The
+                headline run lets the library pick the route per layer (--conv-route
+                auto, its default: narrow layers gather straight from a padded image);
   cpu_baseline  the CPU oracle (a port of the reference CPU nn path, OpenMP over
                 the batch + an optimised BLAS sgemm where one is found) timed
                 on this host on a reduced batch of the same stack.
@@ -36,7 +41,8 @@ PEAK_HBM_GBS = 8000.0
 # script (FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0, the factors a plain copy kernel of known size gives);
 # the summary with the commands is profiles/hbm_traffic_alexnet_b128_pmc.txt.  Counters cannot be read
 # from inside the timed process, so the figure is carried here for the configuration it was measured on.
-MEASURED_GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("alexnet", 128): 5.343e8}
+MEASURED_GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("alexnet", 128, "columns"): 5.343e8}
+ROUTES = {"columns": 0, "auto": 1, "gathered": 2}   # thgpu_conv_set_mode values
 
 
 def cpu_baseline(workload, sample_batch, budget_s=12.0):
@@ -112,6 +118,10 @@ def main():
     ap.add_argument("--cpu-sample-batch", type=int, default=128)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
+    ap.add_argument("--conv-route", default="auto", choices=sorted(ROUTES),
+                    help="how nn.SpatialConvolutionMM computes: im2col/GEMM/col2im columns, GEMMs that gather from "
+                         "the padded image, or the library's choice per layer (its default)")
+    ap.add_argument("--no-column-route", action="store_true", help="skip the second measurement on the column route")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the path is built and measured on a single MI355X "
@@ -123,8 +133,9 @@ def main():
     import mcw_cppamp_torch_amd as pkg
     from mcw_cppamp_torch_amd import gputorch, stacks
 
-    if pkg._lib.lib.thgpu_init() != 0:
-        sys.exit("no GPU: " + pkg._lib.lib.thgpu_last_error().decode())
+    lib = pkg._lib.lib
+    if lib.thgpu_init() != 0:
+        sys.exit("no GPU: " + lib.thgpu_last_error().decode())
 
     name = args.workload
     B = args.batch or stacks.STACKS[name]["batch"]
@@ -138,37 +149,30 @@ def main():
         net.forward(x)
         net.backward(x, go)
 
-    for _ in range(args.warmup):
-        step()
-    gputorch.synchronize()
-
-    ev0, ev1 = gputorch.Event(), gputorch.Event()
-    t0 = time.perf_counter()
-    ev0.record()
-    for _ in range(args.steps):
-        step()
-    ev1.record()
-    gputorch.synchronize()
-    wall = time.perf_counter() - t0
-    dev_ms = ev0.elapsed_ms(ev1)
-    ms_per_step = wall * 1e3 / args.steps
-
-    # Host<->device copies of one batch (blocking, pageable host memory), outside the timed region.
-    host_x = stacks.make_input(name, B, seed=1000)
-    t1 = time.perf_counter()
-    x.copy(host_x)
-    gputorch.synchronize()
-    h2d_ms = (time.perf_counter() - t1) * 1e3
-    t1 = time.perf_counter()
-    net.gradInput.float()
-    d2h_ms = (time.perf_counter() - t1) * 1e3
-
-    w = stacks.work(name, B)
-    kernels, roofline, gemm_shapes, hbm_shapes = {}, None, [], []
-    if not args.no_kernel_timing:
+    def measure(route, steps, warmup, kernel_timing):
+        """Times `steps` steps with the convolutions on `route`, then (kernel_timing) the same steps again with
+        every launch bracketed by HIP events on the library's stream."""
+        if lib.thgpu_conv_set_mode(ROUTES[route]) != 0:
+            sys.exit(lib.thgpu_last_error().decode())
+        for _ in range(warmup):
+            step()
+        gputorch.synchronize()
+        ev0, ev1 = gputorch.Event(), gputorch.Event()
+        t0 = time.perf_counter()
+        ev0.record()
+        for _ in range(steps):
+            step()
+        ev1.record()
+        gputorch.synchronize()
+        wall = time.perf_counter() - t0
+        res = {"ms_per_step": wall * 1e3 / steps, "device_ms_per_step": ev0.elapsed_ms(ev1) / steps,
+               "kernels": {}, "roofline": None, "gemm_shapes": [], "hbm_shapes": []}
+        if not kernel_timing:
+            return res
+        kernels, gemm_shapes, hbm_shapes = res["kernels"], res["gemm_shapes"], res["hbm_shapes"]
         gputorch.prof_reset()
         gputorch.prof_enable(True)
-        for _ in range(args.steps):
+        for _ in range(steps):
             step()
         gputorch.synchronize()
         rep = gputorch.prof_report()
@@ -176,18 +180,17 @@ def main():
         gputorch.prof_reset()
         g_ms = g_fl = 0.0
         g_calls = 0
-        gemm_shapes = []
         for kname, r in sorted(rep.items()):
-            ms = r["ms"] / args.steps
+            ms = r["ms"] / steps
             family = kname.split(" ")[0]          # GEMM records are labelled "<family> M=.. J=.. R=.. tile=.. split=.."
             if family.startswith("gemm_conv") or family == "gemm_blas":
-                fl = r["flops"] / args.steps
+                fl = r["flops"] / steps
                 ent = kernels.setdefault(family, {"launches_per_step": 0.0, "ms_per_step": 0.0, "bound": "mfma",
                                                   "flops_per_step": 0.0})
-                ent["launches_per_step"] += r["calls"] / args.steps
+                ent["launches_per_step"] += r["calls"] / steps
                 ent["ms_per_step"] += ms
                 ent["flops_per_step"] += fl
-                gemm_shapes.append({"gemm": kname, "launches_per_step": r["calls"] / args.steps,
+                gemm_shapes.append({"gemm": kname, "launches_per_step": r["calls"] / steps,
                                     "ms_per_step": round(ms, 4), "tflops": round(fl / ms / 1e9, 2),
                                     "frac": round(fl / ms / 1e9 / PEAK_MFMA_F32_TFLOPS, 4)})
                 g_ms += ms
@@ -196,12 +199,12 @@ def main():
                 continue
             # HBM-bound kernels: im2col / col2im / pooling records carry their geometry after the family name
             ent = kernels.setdefault(family, {"launches_per_step": 0.0, "ms_per_step": 0.0, "bytes_per_step": 0.0})
-            ent["launches_per_step"] += r["calls"] / args.steps
+            ent["launches_per_step"] += r["calls"] / steps
             ent["ms_per_step"] += ms
-            ent["bytes_per_step"] += r["bytes"] / args.steps
+            ent["bytes_per_step"] += r["bytes"] / steps
             if family != kname and r["bytes"] > 0:
-                by = r["bytes"] / args.steps
-                hbm_shapes.append({"kernel": kname, "launches_per_step": r["calls"] / args.steps,
+                by = r["bytes"] / steps
+                hbm_shapes.append({"kernel": kname, "launches_per_step": r["calls"] / steps,
                                    "ms_per_step": round(ms, 4), "gbs": round(by / ms / 1e6, 1),
                                    "frac": round(by / ms / 1e6 / PEAK_HBM_GBS, 4)})
         for ent in kernels.values():
@@ -215,14 +218,46 @@ def main():
                 if by > 0:
                     ent.update(bound="hbm", gbs=round(by / ms / 1e6, 1), frac=round(by / ms / 1e6 / PEAK_HBM_GBS, 4))
         if g_ms > 0:
-            roofline = {
+            res["roofline"] = {
                 "bound": "mfma", "kernel": "gemm_fast_kernel<...> (all conv GEMM launches of a step)",
                 "achieved": round(g_fl / g_ms / 1e9, 2), "peak": PEAK_MFMA_F32_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(g_fl / g_ms / 1e9 / PEAK_MFMA_F32_TFLOPS, 4),
-                "traffic": MEASURED_GEMM_TRAFFIC_BYTES_PER_LAUNCH.get((name, B)),
-                "launches_per_step": g_calls / args.steps, "ms_per_step": round(g_ms, 4),
+                "traffic": MEASURED_GEMM_TRAFFIC_BYTES_PER_LAUNCH.get((name, B, route)),
+                "launches_per_step": g_calls / steps, "ms_per_step": round(g_ms, 4),
                 "flops_per_step": g_fl,
             }
+        return res
+
+    main_run = measure(args.conv_route, args.steps, args.warmup, not args.no_kernel_timing)
+    ms_per_step = main_run["ms_per_step"]
+    kernels, roofline = main_run["kernels"], main_run["roofline"]
+    gemm_shapes, hbm_shapes = main_run["gemm_shapes"], main_run["hbm_shapes"]
+
+    # The same steps with every convolution on the column route (im2col, GEMM, col2im), for the figures of
+    # those kernels at this workload's full geometries.
+    column_route = None
+    if args.conv_route != "columns" and not args.no_column_route:
+        col = measure("columns", args.steps, 2, not args.no_kernel_timing)
+        column_route = {
+            "value": round(B / (col["ms_per_step"] / 1e3), 2), "unit": "images/s",
+            "ms_per_step": round(col["ms_per_step"], 4), "roofline": col["roofline"],
+            "kernels": {k: v for k, v in col["kernels"].items() if k in ("im2col", "col2im") or k.startswith("gemm_conv")},
+            "hbm_shapes": [h for h in col["hbm_shapes"] if h["kernel"].startswith(("im2col", "col2im"))],
+        }
+        if lib.thgpu_conv_set_mode(ROUTES[args.conv_route]) != 0:
+            sys.exit(lib.thgpu_last_error().decode())
+
+    # Host<->device copies of one batch (blocking, pageable host memory), outside the timed region.
+    host_x = stacks.make_input(name, B, seed=1000)
+    t1 = time.perf_counter()
+    x.copy(host_x)
+    gputorch.synchronize()
+    h2d_ms = (time.perf_counter() - t1) * 1e3
+    t1 = time.perf_counter()
+    net.gradInput.float()
+    d2h_ms = (time.perf_counter() - t1) * 1e3
+
+    w = stacks.work(name, B)
 
     cpu = None
     if not args.no_cpu_baseline:
@@ -234,13 +269,13 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s conv stack, batch %d, input %s, fwd+bwd (zeroGradParameters, forward, "
                                "updateGradInput, accGradParameters)" % (name, B, "x".join(map(str, stacks.STACKS[name]["input"]))),
-                   "batch": B, "device": gputorch.getDeviceProperties()["name"]},
-        "device_ms_per_step": round(dev_ms / args.steps, 4),
+                   "batch": B, "conv_route": args.conv_route, "device": gputorch.getDeviceProperties()["name"]},
+        "device_ms_per_step": round(main_run["device_ms_per_step"], 4),
         "transfers": {"h2d_input_ms": round(h2d_ms, 3), "d2h_gradinput_ms": round(d2h_ms, 3),
                       "images_per_s_including_transfers": round(B / ((ms_per_step + h2d_ms + d2h_ms) / 1e3), 1)},
         "gemm_tflops_over_whole_step": round(w["gemm_flops"] / (ms_per_step / 1e3) / 1e12, 2),
         "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels, "gemm_shapes": gemm_shapes,
-        "hbm_shapes": hbm_shapes,
+        "hbm_shapes": hbm_shapes, "column_route": column_route,
     }
     print(json.dumps(line))
 
