@@ -70,6 +70,12 @@ bool is_padded(const THGPUTensor *t, const ConvShape &s, int padH, int padW) {
     return t->nDimension == 3 + o && (!s.batched || t->size[0] == s.B) && t->size[o] == s.C &&
            t->size[o + 1] == s.H + 2 * padH && t->size[o + 2] == s.W + 2 * padW && THGPUTensor_isContiguous(t);
 }
+// The forward's columns: [B,] K, N.
+bool is_columns(const THGPUTensor *t, const ConvShape &s) {
+    const int o = s.batched ? 1 : 0;
+    return t->nDimension == 2 + o && (!s.batched || t->size[0] == s.B) && t->size[o] == s.K && t->size[o + 1] == s.N &&
+           THGPUTensor_isContiguous(t);
+}
 int size_padded(THGPUTensor *t, const ConvShape &s, int padH, int padW) {
     if (s.batched)
         THGPUTensor_resize4d(t, s.B, s.C, s.H + 2 * padH, s.W + 2 * padW);
@@ -255,7 +261,7 @@ int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor
     // shape (the module was never run forward on this input size) the columns
     // are rebuilt from the input, as the reference GPU code always did
     // (gpunn-impl/SpatialConvolutionMM.cpp:394-396).
-    if (THGPUTensor_nElement(finput) != s.B * s.K * s.N || !THGPUTensor_isContiguous(finput)) {
+    if (!is_columns(finput, s)) {
         THGPUTensor *in = THGPUTensor_newContiguous(input);
         if (s.batched)
             THGPUTensor_resize3d(finput, s.B, s.K, s.N);

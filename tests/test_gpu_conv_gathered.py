@@ -217,6 +217,37 @@ def test_mode_1_gathers_narrow_layers_only(gt):
         assert lib.thgpu_conv_set_mode(before) == 0
 
 
+def test_route_switched_between_forward_and_accgradparameters(gt):
+    """2x2 kernels at stride 2 on an even image: the columns have as many elements as the (unpadded) image, so only
+    the buffer's shape tells accGradParameters which of the two finput holds."""
+    B, C, H, W, M, k = 2, 64, 12, 12, 64, 2
+    geo = (k, k, 0, 0, 2, 2)
+    rng = rng_for(47)
+    x, w, b = uniform(rng, (B, C, H, W)), uniform(rng, (M, C * k * k), -0.05, 0.05), uniform(rng, (M,))
+    gw0, gb0 = np.zeros((M, C * k * k), np.float32), np.zeros((M,), np.float32)
+    out_ref, go, gi_ref, gw_ref, gb_ref = reference(x, w, b, rng, geo, 1.0, gw0, gb0)
+    lib = gt._lib.lib
+    before = lib.thgpu_conv_get_mode()
+    try:
+        for fwd_mode, acc_mode in ((2, 0), (0, 2)):
+            m = gt.nn.SpatialConvolutionMM(C, M, k, k, 2, 2, 0)
+            m._assign("weight", w)
+            m._assign("bias", b)
+            m.gradWeight[...] = 0
+            m.gradBias[...] = 0
+            m.gpu()
+            dx, dgo = dev(gt, x), dev(gt, go)
+            assert lib.thgpu_conv_set_mode(fwd_mode) == 0
+            out = m.forward(dx).float()
+            assert m.finput.float().size == B * C * H * W
+            assert lib.thgpu_conv_set_mode(acc_mode) == 0
+            m.accGradParameters(dx, dgo, 1.0)
+            assert rel_err(out, out_ref) < gemm_tol(C * k * k)
+            assert rel_err(m.gradWeight.float(), gw_ref) < gemm_tol(B * out_ref.shape[2] * out_ref.shape[3])
+    finally:
+        assert lib.thgpu_conv_set_mode(before) == 0
+
+
 def test_conv_mode_api(gt):
     lib = gt._lib.lib
     before = lib.thgpu_conv_get_mode()
