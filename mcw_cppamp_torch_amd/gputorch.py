@@ -68,6 +68,30 @@ def _host_tensor_struct(arr):
     return kind, tensor, (arr, sizes, strides, storage)
 
 
+def _ascii_tokens(f, n):
+    """Reads n whitespace-separated tokens from a byte stream, then the newline that follows a non-empty array
+    (the auto-spacing of THDiskFile's ASCII mode, mcw_torch7_core/lib/TH/THDiskFile.c:55-68)."""
+    out = []
+    while len(out) < n:
+        tok = b""
+        while True:
+            c = f.read(1)
+            if not c:
+                break
+            if c.isspace():
+                if tok:
+                    break
+                continue
+            tok += c
+        if not tok:
+            raise _lib.THGPUError("read error: read %d blocks instead of %d" % (len(out), n))
+        out.append(tok)
+        last = c
+    if n > 0 and last not in (b"\n", b""):
+        f.seek(-1, 1)   # only a newline right after the last element belongs to the array
+    return out
+
+
 class GPUStorage(object):
     """torch.GPUStorage (gputorch/Storage.cpp, gputorch/lib/THC/THCStorage.cpp)."""
 
@@ -125,6 +149,42 @@ class GPUStorage(object):
             st.size = host.size
             getattr(lib, "THGPUStorage_copy%s" % kind)(self._p, ctypes.byref(st))
         _lib.check()
+        return self
+
+    def write(self, f, binary=True):
+        """storage:write(file): the element count as a long, then the floats staged through host memory
+        (gputorch/torch/generic/Storage.c:180-189 with the THFile_writeRealRaw of gputorch/Storage.cpp:23-31), in
+        the disk file's native binary encoding or its ASCII mode ("%ld", "%.9g", elements separated by one space, a
+        newline after each non-empty array: mcw_torch7_core/lib/TH/THDiskFile.c:88-130,304-310).  `f` is a file
+        object opened for writing bytes."""
+        host = self.float()
+        if binary:
+            f.write(np.int64(host.size).tobytes())
+            f.write(host.tobytes())
+        else:
+            f.write(b"%d\n" % host.size)
+            if host.size:
+                f.write(" ".join("%.9g" % float(v) for v in host).encode("ascii") + b"\n")
+        return self
+
+    def read(self, f, binary=True):
+        """storage:read(file): the inverse of write (gputorch/torch/generic/Storage.c:191-201,
+        gputorch/Storage.cpp:14-21); resizes the storage to the stored element count."""
+        if binary:
+            head = f.read(8)
+            if len(head) != 8:
+                raise _lib.THGPUError("read error: read 0 blocks instead of 1")
+            n = int(np.frombuffer(head, np.int64)[0])
+            raw = f.read(4 * n)
+            if n < 0 or len(raw) != 4 * n:
+                raise _lib.THGPUError("read error: read %d blocks instead of %d" % (len(raw) // 4, n))
+            host = np.frombuffer(raw, np.float32)
+        else:
+            n = int(_ascii_tokens(f, 1)[0])
+            host = np.array([float(t) for t in _ascii_tokens(f, n)], np.float32)
+        self.resize(n)
+        if n:
+            self.copy(host)
         return self
 
     def float(self):

@@ -264,3 +264,34 @@ def test_allocation_failure_is_reported_and_leaves_the_library_usable(gt):
     assert np.array_equal(t.float(), np.full((3, 3), 2.0, np.float32))
     with pytest.raises(gt.THGPUError):
         gt.GPUTensor(1 << 23, 1 << 23)
+
+
+def test_storage_write_read_binary_and_ascii_known_answers(gt):
+    """storage:write / :read (gputorch/torch/generic/Storage.c:180-201 over gputorch/Storage.cpp:14-31) against
+    byte strings written out by hand from THDiskFile's formats: a native long and raw floats, or "%ld" / "%.9g"
+    text with single spaces and a newline after each non-empty array."""
+    import io
+    import struct
+    vals = [1.0, 2.5, -1.0 / 3.0, 1e-7, 16777216.0]
+    st = gt.gputorch.GPUStorage(vals)
+    f = io.BytesIO()
+    st.write(f)
+    assert f.getvalue() == struct.pack("<q", 5) + struct.pack("<5f", *vals)
+    f = io.BytesIO()
+    st.write(f, binary=False)
+    assert f.getvalue() == b"5\n1 2.5 -0.333333343 1.00000001e-07 16777216\n"
+    for binary in (True, False):
+        f = io.BytesIO()
+        st.write(f, binary=binary)
+        gt.gputorch.GPUStorage().write(f, binary=binary)          # an empty storage after it
+        gt.gputorch.GPUStorage([7.0]).write(f, binary=binary)
+        f.seek(0)
+        back = gt.gputorch.GPUStorage(3).read(f, binary=binary)
+        assert back.size() == 5 and np.array_equal(back.float(), np.array(vals, np.float32))
+        assert gt.gputorch.GPUStorage(2).read(f, binary=binary).size() == 0
+        assert gt.gputorch.GPUStorage().read(f, binary=binary).float().tolist() == [7.0]
+        assert f.read() == b""
+    with pytest.raises(gt._lib.THGPUError):
+        gt.gputorch.GPUStorage().read(io.BytesIO(struct.pack("<q", 4) + b"\0" * 8))
+    with pytest.raises(gt._lib.THGPUError):
+        gt.gputorch.GPUStorage().read(io.BytesIO(b"3\n1 2\n"), binary=False)
