@@ -196,6 +196,29 @@ def test_gathered_conv_random_geometry(gt, gathered_route, cfg):
     assert rel_err(got["gradBias"], gb_ref) < gemm_tol(B * N)
 
 
+@pytest.mark.parametrize("split", [1, 3])
+@pytest.mark.parametrize("tile", ["128x128", "192x128", "64x256", "128x256", "256x128", "64x64"])
+def test_gathered_conv_every_tile_configuration(gt, gathered_route, tile, split, monkeypatch):
+    """Every tile of the GEMM has its own gathering kernels (plain and reduction-batched); the library's choice
+    would leave most of them to the large benchmark shapes, so each is forced here on a shape all of them fit."""
+    monkeypatch.setenv("THGPU_GEMM_TILE", tile)
+    monkeypatch.setenv("THGPU_GEMM_SPLIT", str(split))
+    B, C, H, W, M, kH, kW = 2, 256, 12, 12, 256, 3, 3
+    geo = (kH, kW, 1, 1, 1, 1)
+    K = C * kH * kW
+    rng = rng_for(48)
+    s = 1.0 / np.sqrt(K)
+    x = uniform(rng, (B, C, H, W))
+    w, b = uniform(rng, (M, K), -s, s), uniform(rng, (M,), -s, s)
+    gw0, gb0 = uniform(rng, (M, K)), uniform(rng, (M,))
+    out_ref, go, gi_ref, gw_ref, gb_ref = reference(x, w, b, rng, geo, 1.0, gw0, gb0)
+    got = run_conv(gt, x, w, b, go, geo, 1.0, gw0, gb0)
+    assert got["finput"].shape == (B, C, H + 2, W + 2)
+    assert rel_err(got["output"], out_ref) < gemm_tol(K)
+    assert rel_err(got["gradInput"], gi_ref) < gemm_tol(M * kH * kW)
+    assert rel_err(got["gradWeight"], gw_ref) < gemm_tol(B * H * W)
+
+
 def test_mode_1_gathers_narrow_layers_only(gt):
     lib = gt._lib.lib
     before = lib.thgpu_conv_get_mode()
