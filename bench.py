@@ -41,7 +41,7 @@ PEAK_HBM_GBS = 8000.0
 # script (FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0, the factors a plain copy kernel of known size gives);
 # the summary with the commands is profiles/hbm_traffic_alexnet_b128_pmc.txt.  Counters cannot be read
 # from inside the timed process, so the figure is carried here for the configuration it was measured on.
-MEASURED_GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("alexnet", 128, "auto"): 1.725e8, ("alexnet", 128, "columns"): 5.342e8}
+MEASURED_GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("alexnet", 128, "auto"): 1.750e8, ("alexnet", 128, "columns"): 5.339e8}
 ROUTES = {"columns": 0, "auto": 1, "gathered": 2}   # thgpu_conv_set_mode values
 
 
