@@ -95,11 +95,6 @@ const int *table(int kind, int a, int b, int c, int d, int e, long count) {
     if (it != g_tables.end()) return it->second;
     hipStream_t s = stream();
     if (!s) return nullptr;
-    if (g_tables.size() >= 512) {  // a caller cycling through geometries: start over
-        if (hipStreamSynchronize(s) != hipSuccess) return nullptr;
-        for (auto &kv : g_tables) (void)hipFree(kv.second);
-        g_tables.clear();
-    }
     int *t = nullptr;
     if (hipMalloc(reinterpret_cast<void **>(&t), sizeof(int) * (size_t)count) != hipSuccess) {
         (void)hipGetLastError();
@@ -117,6 +112,19 @@ const int *table(int kind, int a, int b, int c, int d, int e, long count) {
     }
     g_tables[key] = t;
     return t;
+}
+
+// Called once at the start of a convolution pass, before it takes its two tables: a caller cycling
+// through many geometries starts the cache over (never between the two look-ups of one pass, which
+// would free the first table under the pass that is about to use it).
+int trim_tables() {
+    if (g_tables.size() < 512) return 0;
+    hipStream_t s = stream();
+    if (!s) return 1;
+    THGPU_HIP_TRY(hipStreamSynchronize(s));
+    for (auto &kv : g_tables) (void)hipFree(kv.second);
+    g_tables.clear();
+    return 0;
 }
 
 const int *tap_table(int planes, int kH, int kW, int plane, int pitch) {
@@ -202,6 +210,7 @@ int conv_implicit_forward(const float *padded, const float *weight, const float 
     const int Hp = H + 2 * pH, Wp = W + 2 * pW;
     const int Ho = (Hp - kH) / sH + 1, Wo = (Wp - kW) / sW + 1;
     const long N = (long)Ho * Wo;
+    if (trim_tables()) return 1;
     GemmProblem p;
     p.A = weight;
     p.a_rc = true;
@@ -230,6 +239,7 @@ int conv_implicit_gradweight(const float *padded, const float *gradOutput, float
     const int Ho = (Hp - kH) / sH + 1, Wo = (Wp - kW) / sW + 1;
     const long N = (long)Ho * Wo;
     const int K = C * kH * kW;
+    if (trim_tables()) return 1;
     GemmProblem p;
     p.A = gradOutput;
     p.a_rc = true;
@@ -271,6 +281,7 @@ int conv_implicit_gradinput(const float *gradOutput, const float *weight, float 
                            kW);
     }
     if (check_launch("flip_weight")) return 1;
+    if (trim_tables()) return 1;
     GemmProblem p;
     p.A = Wt;
     p.a_rc = true;

@@ -271,6 +271,30 @@ def test_route_switched_between_forward_and_accgradparameters(gt):
         assert lib.thgpu_conv_set_mode(before) == 0
 
 
+def test_offset_table_cache_starts_over_after_many_geometries(gt, gathered_route):
+    """The per-geometry offset tables are cached (two per pass); past 512 entries the cache is emptied.  Results
+    before, across and after that point must agree with the column route."""
+    lib = gt._lib.lib
+    B, C, H, M, k = 1, 64, 8, 64, 3
+    rng = rng_for(49)
+    w, b = uniform(rng, (M, C * k * k), -0.05, 0.05), uniform(rng, (M,))
+    m = gt.nn.SpatialConvolutionMM(C, M, k, k, 1, 1, 1)
+    m._assign("weight", w)
+    m._assign("bias", b)
+    m.gpu()
+    for W in range(8, 8 + 280):                     # 280 geometries x 2 tables
+        x = uniform(rng, (B, C, H, W))
+        dx = dev(gt, x)
+        out = m.forward(dx).float()
+        if W % 40 == 0 or W >= 8 + 254:            # the cache is emptied near the 256th geometry
+            assert lib.thgpu_conv_set_mode(0) == 0
+            try:
+                ref = m.forward(dx).float()
+            finally:
+                assert lib.thgpu_conv_set_mode(2) == 0
+            assert rel_err(out, ref) < 1e-5, W
+
+
 def test_conv_mode_api(gt):
     lib = gt._lib.lib
     before = lib.thgpu_conv_get_mode()
