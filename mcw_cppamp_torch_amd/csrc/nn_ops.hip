@@ -101,8 +101,8 @@ int thgpu_SpatialConvolutionMM_updateOutput(THGPUTensor *input, THGPUTensor *wei
     THGPUTensor *in = THGPUTensor_newContiguous(input);
     if (!in) return 1;
 
-    const bool implicit = conv_use_gathered(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW);
-    if (implicit) {
+    const bool gathered = conv_use_gathered(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW);
+    if (gathered) {
         // finput holds the padded input instead of the columns
         if (size_padded(finput, s, padH, padW)) {
             THGPUTensor_free(in);
@@ -119,11 +119,11 @@ int thgpu_SpatialConvolutionMM_updateOutput(THGPUTensor *input, THGPUTensor *wei
         THGPUTensor_resize3d(output, s.M, s.Ho, s.Wo);
     int rc = 0;
     if (!THGPUTensor_isContiguous(finput) || !THGPUTensor_isContiguous(output) ||
-        (!implicit && THGPUTensor_nElement(finput) != s.B * s.K * s.N) ||
+        (!gathered && THGPUTensor_nElement(finput) != s.B * s.K * s.N) ||
         THGPUTensor_nElement(output) != s.B * s.M * s.N)
         rc = fail("SpatialConvolutionMM: could not size finput/output");
 
-    if (implicit) {
+    if (gathered) {
         if (!rc) rc = pad_planes_launch(dptr(in), s.B * s.C, s.H, s.W, padH, padW, dptr(finput));
         if (!rc)
             rc = conv_implicit_forward(dptr(finput), dptr(weight), dptr(bias), dptr(output), s.B, s.C, s.H, s.W, s.M, kH,
