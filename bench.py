@@ -15,7 +15,7 @@ Beside the throughput the line carries
   kernels       the same for every kernel family (HBM-bound ones in GB/s);
   gemm_shapes   every GEMM of the stack on its own (shape, chosen tile and split,
                 TFLOP/s): the small-K GEMMs of first layers are HBM-bound themselves;
-  hbm_shapes    every im2col / col2im / pooling launch geometry on its own (GB/s);
+  hbm_shapes    every im2col / col2im / pad / pooling launch geometry on its own (GB/s);
   column_route  the same steps once more with every convolution on the reference's
                 route (im2col, GEMM, col2im): throughput, GEMM roofline, and the
                 im2col / col2im figures at the workload's full geometries.  The

@@ -197,7 +197,9 @@ int pad_planes_launch(const float *in, long planes, int H, int W, int pH, int pW
     if (total <= 0) return 0;
     if (total >= (1L << 31)) return fail("pad: %ld elements exceed 32-bit indexing", total);
     {
-        LaunchScope scope("pad_planes", 0.0, 4.0 * (total + planes * H * W));
+        const char *label = prof_enabled() ? prof_label("pad_planes planes=%ld %dx%d p=%dx%d", planes, H, W, pH, pW)
+                                           : "pad_planes";
+        LaunchScope scope(label, 0.0, 4.0 * (total + planes * H * W));
         hipLaunchKernelGGL(pad_planes_kernel, dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0, s, in, out,
                            (unsigned)total, H, W, pH, pW, (int)Hp, (int)Wp, FastDiv((uint32_t)Wp),
                            FastDiv((uint32_t)Hp), (reinterpret_cast<uintptr_t>(out) & 15) == 0);
