@@ -106,6 +106,14 @@ const char *thgpu_last_error(void);
  * else; explicit call returns non-zero if no usable GPU is present. */
 int thgpu_init(void);
 
+/* Testing and tuning switches (no counterpart in the reference).  name: gemm_tile (a tile configuration such
+ * as "128x128"), gemm_split (a reduction split count), im2col_kernel (unit | strip | direct), im2col_plan
+ * ("v,PL,TG"), col2im_generic ("1"), pool_bwd_direct ("1"); value NULL or "" restores the library's own
+ * choice.  The environment variables THGPU_GEMM_TILE, THGPU_GEMM_SPLIT, THGPU_IM2COL_KERNEL, THGPU_IM2COL_PLAN,
+ * THGPU_COL2IM_GENERIC and THGPU_POOL_BWD_DIRECT give the initial values and are read once, when the library
+ * initialises; no operator call reads the environment. */
+int thgpu_debug_set(const char *name, const char *value);
+
 /* Real stream synchronisation, replacing the no-op gputorch.synchronize
  * (gputorch/init.cpp:10-14). */
 int thgpu_synchronize(void);
@@ -339,11 +347,14 @@ int thgpu_col2im(const float *col, long B, int C, int H, int W, int kH, int kW, 
  * 110-225, 227-311, 313-429); arguments are the module fields those read by
  * name (:116-128) with the single `padding` split into padW/padH.  input is
  * [C,H,W] or [B,C,H,W] contiguous and is never modified; weight is
- * [M, C*kH*kW].  Buffer semantics follow the CPU module, the parity target
- * (mcw_nn/generic/SpatialConvolutionMM.c:179,243,318): finput is resized to
+ * [M, C*kH*kW].  Buffer shapes follow the CPU module, the parity target
+ * (mcw_nn/generic/SpatialConvolutionMM.c:179,243): finput is resized to
  * [B,K,N] and keeps the whole batch of columns, fgradInput likewise holds the
- * column gradients, and accGradParameters reuses finput from the preceding
- * updateOutput without recomputing it. */
+ * column gradients.  accGradParameters rebuilds finput from its `input`
+ * argument on every call, as the reference GPU code does (:388-396), so its
+ * result depends on its arguments alone: finput and fgradInput may be shared
+ * between modules, and `input` need not be the last forward pass's (see
+ * thgpu_conv_set_finput_reuse for the CPU module's behaviour). */
 int thgpu_SpatialConvolutionMM_updateOutput(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias,
                                             THGPUTensor *finput, THGPUTensor *fgradInput, THGPUTensor *output,
                                             int kW, int kH, int dW, int dH, int padW, int padH);
@@ -369,6 +380,14 @@ int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor
  * (columns | auto | gathered) sets the initial mode.  set returns 0, or an error for any other mode. */
 int thgpu_conv_set_mode(int mode);
 int thgpu_conv_get_mode(void);
+
+/* on != 0: accGradParameters takes a finput that has the shape the forward pass gives it to BE the forward
+ * pass's and does not rebuild it -- the CPU module's behaviour (mcw_nn/generic/SpatialConvolutionMM.c:318,
+ * 336), which saves one pass over the input per call and is wrong when `input` is not what the last
+ * updateOutput of this module saw or when another module wrote the shared buffer in between (no
+ * counterpart in the reference GPU code, which always rebuilds).  Initially off.  Returns 0. */
+int thgpu_conv_set_finput_reuse(int on);
+int thgpu_conv_get_finput_reuse(void);
 
 /* nn.SpatialMaxPooling.  Replace gpunn_SpatialMaxPooling_updateOutput /
  * _updateGradInput (gpunn-impl/SpatialMaxPooling.cpp:205-281, 283-383).

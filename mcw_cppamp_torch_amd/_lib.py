@@ -63,8 +63,11 @@ _SIGNATURES = {
     "thgpu_last_error": (c_char_p, []),
     "thgpu_init": (c_int, []),
     "thgpu_synchronize": (c_int, []),
+    "thgpu_debug_set": (c_int, [c_char_p, c_char_p]),
     "thgpu_conv_set_mode": (c_int, [c_int]),
     "thgpu_conv_get_mode": (c_int, []),
+    "thgpu_conv_set_finput_reuse": (c_int, [c_int]),
+    "thgpu_conv_get_finput_reuse": (c_int, []),
     "thgpu_device_info": (c_int, [c_char_p, c_long, ctypes.POINTER(c_int), longp]),
     "thgpu_event_create": (c_int, []),
     "thgpu_event_record": (c_int, [c_int]),

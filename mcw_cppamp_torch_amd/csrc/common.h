@@ -55,6 +55,20 @@ hipStream_t stream();
 float *workspace(size_t bytes);
 int num_cus();
 
+// Testing and tuning switches.  Filled from the environment once, when the library initialises
+// (THGPU_GEMM_TILE, THGPU_GEMM_SPLIT, THGPU_IM2COL_KERNEL, THGPU_IM2COL_PLAN, THGPU_COL2IM_GENERIC,
+// THGPU_POOL_BWD_DIRECT), and changed afterwards only through thgpu_debug_set: no launch reads the
+// environment.
+struct Tuning {
+    char gemm_tile[16] = "";      // a tile configuration by name; "" leaves the choice to the cost model
+    int gemm_split = 0;           // reduction split count; 0 leaves it to the cost model
+    char im2col_kernel[16] = "";  // unit | strip | direct
+    int im2col_plan[3] = {0, 0, 0};  // strip shape "v,PL,TG"
+    bool col2im_generic = false;
+    bool pool_bwd_direct = false;
+};
+const Tuning &tuning();
+
 // Brackets one kernel launch with events when per-kernel timing is enabled.
 struct LaunchScope {
     LaunchScope(const char *name, double flops, double bytes);
@@ -75,6 +89,26 @@ int fill_device(float *p, long n, float v);           // async on the library st
 int copy_h2d(float *dst, const float *src, long n);   // blocking
 int copy_d2h(float *dst, const float *src, long n);   // blocking
 int copy_d2d(float *dst, const float *src, long n);   // async on the library stream
+
+// ---- tensors as kernel operands -------------------------------------------------
+// Whether every element the tensor's shape addresses lies inside its storage: the check an operator
+// makes on each tensor it has resized, and on the caller's, before any kernel is given its pointer.
+inline bool tensor_backed(const THGPUTensor *t) {
+    if (!t) return false;
+    long extent = t->nDimension > 0 ? 1 : 0;
+    for (int d = 0; d < t->nDimension; ++d) {
+        if (t->size[d] <= 0) return true;  // no elements: nothing to back
+        if (t->stride[d] < 0) return false;
+        extent += (t->size[d] - 1) * t->stride[d];
+    }
+    if (extent == 0) return true;
+    return t->storage && t->storage->data && t->storageOffset >= 0 &&
+           t->storageOffset + extent <= t->storage->size;
+}
+// A dense tensor of exactly n elements with memory behind all of them.
+inline bool tensor_ready(const THGPUTensor *t, long n) {
+    return t && THGPUTensor_isContiguous(t) && THGPUTensor_nElement(t) == n && tensor_backed(t);
+}
 
 // ---- unsigned division by a run-time constant ---------------------------------
 // q = n / d for 0 <= n < 2^31, 1 <= d < 2^31 via one mul-hi and a shift.

@@ -138,6 +138,76 @@ constexpr long kMaxExtent = 1L << 30;  // floats: the loaders address with 32-bi
 
 int g_mode = -1;
 
+// The three products as GEMM problems, without pointers and tables (those are filled in by the launchers; a
+// problem with `gathered` set is enough for the planner to say whether a tiled kernel takes it).
+const int kNoTable = 0;  // stands in for a table where only the planner looks at the problem
+
+GemmProblem forward_problem(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
+    const int Hp = H + 2 * pH, Wp = W + 2 * pW;
+    const int Ho = (Hp - kH) / sH + 1, Wo = (Wp - kW) / sW + 1;
+    const long N = (long)Ho * Wo;
+    GemmProblem p;
+    p.a_rc = true;
+    p.sA = (long)C * kH * kW;
+    p.rowtab = p.coltab = &kNoTable;
+    p.bsB = (long)C * Hp * Wp;
+    p.b_extent = B * p.bsB;
+    p.sC = N;
+    p.bsC = (long)M * N;
+    p.M = M;
+    p.J = (int)(B * N);
+    p.N = (int)N;
+    p.R = C * kH * kW;
+    p.flops = 2.0 * M * (double)N * p.R * B;
+    p.tag = "gemm_conv_fwd";
+    return p;
+}
+
+GemmProblem gradweight_problem(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
+    const int Hp = H + 2 * pH, Wp = W + 2 * pW;
+    const int Ho = (Hp - kH) / sH + 1, Wo = (Wp - kW) / sW + 1;
+    const long N = (long)Ho * Wo;
+    const int K = C * kH * kW;
+    GemmProblem p;
+    p.a_rc = true;
+    p.sA = N;
+    p.rbA = (long)M * N;
+    p.rowtab = p.coltab = &kNoTable;
+    p.rbB = (long)C * Hp * Wp;
+    p.b_extent = B * p.rbB;
+    p.sC = K;
+    p.M = M;
+    p.J = K;
+    p.N = K;
+    p.R = (int)N;
+    p.nb = (int)B;
+    p.beta = 1.0f;
+    p.flops = 2.0 * M * (double)N * K * B;
+    p.tag = "gemm_conv_gradweight";
+    return p;
+}
+
+// Unit stride only: one column per input pixel, one reduction index per (output plane, tap).
+GemmProblem gradinput_problem(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW) {
+    const int Ho = H + 2 * pH - kH + 1, Wo = W + 2 * pW - kW + 1;
+    const int Hq = H + kH - 1, Wq = W + kW - 1;
+    GemmProblem p;
+    p.a_rc = true;
+    p.sA = (long)M * kH * kW;
+    p.rowtab = p.coltab = &kNoTable;
+    p.bsB = (long)M * Hq * Wq;
+    p.b_extent = B * p.bsB;
+    p.sC = (long)H * W;
+    p.bsC = (long)C * H * W;
+    p.M = C;
+    p.J = (int)(B * H * W);
+    p.N = H * W;
+    p.R = M * kH * kW;
+    p.flops = 2.0 * M * (double)Ho * Wo * C * kH * kW * B;  // the convolution's own count: Ho*Wo <= H*W columns
+    p.tag = "gemm_conv_gradinput";
+    return p;
+}
+
 }  // namespace
 
 int conv_mode() {
@@ -150,20 +220,25 @@ int conv_mode() {
 
 void conv_set_mode(int mode) { g_mode = mode; }
 
-// Shapes the gathered GEMMs take: a tile of the fast kernel must fit (M, J >= 64, R >= 16) and the padded
-// batch must stay within 32-bit byte offsets.
+// Shapes the gathered GEMMs take: the padded batch must stay within 32-bit byte offsets and a tile of the fast
+// kernel must take both products that share finput (the GEMM's own planner answers that: M, J >= 64, R >= 16,
+// offsets of operands and output below 2^30 floats, a tile the tuning switches allow).
 static bool forward_fits(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
     const long Hp = H + 2L * pH, Wp = W + 2L * pW;
     const long Ho = (Hp - kH) / sH + 1, Wo = (Wp - kW) / sW + 1;
     const long K = (long)C * kH * kW, N = Ho * Wo;
-    return M >= 64 && K >= 64 && N >= 16 && B * N >= 64 && B * C * Hp * Wp < kMaxExtent;
+    if (!(M >= 64 && K >= 64 && N >= 16 && B * N >= 64 && B * N < (1L << 31) && B * C * Hp * Wp < kMaxExtent)) return false;
+    return gemm_tiled_fits(forward_problem(B, C, H, W, M, kH, kW, pH, pW, sH, sW)) &&
+           gemm_tiled_fits(gradweight_problem(B, C, H, W, M, kH, kW, pH, pW, sH, sW));
 }
 
 static bool gradinput_fits(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
     if (sH != 1 || sW != 1 || kH - 1 - pH < 0 || kW - 1 - pW < 0) return false;
     const long Hq = H + kH - 1, Wq = W + kW - 1;
-    return C >= 64 && B * H * W >= 64 && (long)M * kH * kW >= 16 && B * M * Hq * Wq < kMaxExtent &&
-           B * (long)H * W < (1L << 31);
+    if (!(C >= 64 && B * H * W >= 64 && (long)M * kH * kW >= 16 && B * M * Hq * Wq < kMaxExtent &&
+          B * (long)H * W < (1L << 31)))
+        return false;
+    return gemm_tiled_fits(gradinput_problem(B, C, H, W, M, kH, kW, pH, pW));
 }
 
 // Where the gathered route pays (measured on the AlexNet-, OverFeat- and VGG-style layers): the column
@@ -211,27 +286,15 @@ int conv_implicit_forward(const float *padded, const float *weight, const float 
                           int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
     const int Hp = H + 2 * pH, Wp = W + 2 * pW;
     const int Ho = (Hp - kH) / sH + 1, Wo = (Wp - kW) / sW + 1;
-    const long N = (long)Ho * Wo;
     if (trim_tables()) return 1;
-    GemmProblem p;
+    GemmProblem p = forward_problem(B, C, H, W, M, kH, kW, pH, pW, sH, sW);
     p.A = weight;
-    p.a_rc = true;
-    p.sA = (long)C * kH * kW;
     p.B = padded;
     p.rowtab = tap_table(C, kH, kW, Hp * Wp, Wp);
     p.coltab = pixel_table(Ho, Wo, sH * Wp, sW);
     if (!p.rowtab || !p.coltab) return 1;
-    p.bsB = (long)C * Hp * Wp;
-    p.b_extent = B * p.bsB;
     p.C = output;
-    p.sC = N;
-    p.bsC = (long)M * N;
     p.bias = bias;
-    p.M = M;
-    p.J = (int)(B * N);
-    p.N = (int)N;
-    p.R = C * kH * kW;
-    p.tag = "gemm_conv_fwd";
     return gemm_launch(p);
 }
 
@@ -239,30 +302,15 @@ int conv_implicit_gradweight(const float *padded, const float *gradOutput, float
                              int W, int M, int kH, int kW, int pH, int pW, int sH, int sW, float scale) {
     const int Hp = H + 2 * pH, Wp = W + 2 * pW;
     const int Ho = (Hp - kH) / sH + 1, Wo = (Wp - kW) / sW + 1;
-    const long N = (long)Ho * Wo;
-    const int K = C * kH * kW;
     if (trim_tables()) return 1;
-    GemmProblem p;
+    GemmProblem p = gradweight_problem(B, C, H, W, M, kH, kW, pH, pW, sH, sW);
     p.A = gradOutput;
-    p.a_rc = true;
-    p.sA = N;
-    p.rbA = (long)M * N;
     p.B = padded;
     p.rowtab = pixel_table(Ho, Wo, sH * Wp, sW);
     p.coltab = tap_table(C, kH, kW, Hp * Wp, Wp);
     if (!p.rowtab || !p.coltab) return 1;
-    p.rbB = (long)C * Hp * Wp;
-    p.b_extent = B * p.rbB;
     p.C = gradWeight;
-    p.sC = K;
-    p.M = M;
-    p.J = K;
-    p.N = K;
-    p.R = (int)N;
-    p.nb = (int)B;
     p.alpha = scale;
-    p.beta = 1.0f;
-    p.tag = "gemm_conv_gradweight";
     return gemm_launch(p);
 }
 
@@ -284,24 +332,13 @@ int conv_implicit_gradinput(const float *gradOutput, const float *weight, float 
     }
     if (check_launch("flip_weight")) return 1;
     if (trim_tables()) return 1;
-    GemmProblem p;
+    GemmProblem p = gradinput_problem(B, C, H, W, M, kH, kW, pH, pW);
     p.A = Wt;
-    p.a_rc = true;
-    p.sA = (long)M * kH * kW;
     p.B = Q;
     p.rowtab = tap_table(M, kH, kW, Hq * Wq, Wq);
     p.coltab = pixel_table(H, W, Wq, 1);
     if (!p.rowtab || !p.coltab) return 1;
-    p.bsB = (long)M * Hq * Wq;
-    p.b_extent = B * p.bsB;
     p.C = gradInput;
-    p.sC = (long)H * W;
-    p.bsC = (long)C * H * W;
-    p.M = C;
-    p.J = (int)(B * H * W);
-    p.N = H * W;
-    p.R = M * kH * kW;
-    p.tag = "gemm_conv_gradinput";
     return gemm_launch(p);
 }
 

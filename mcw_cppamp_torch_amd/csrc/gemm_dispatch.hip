@@ -4,7 +4,6 @@
 // Also the THGPUBlas_gemm entry point.
 #include "gemm_mfma.h"
 
-#include <cstdlib>
 #include <cstring>
 
 namespace thgpu {
@@ -98,7 +97,68 @@ double model_cycles(const TileCfg &c, int layout, long M, long J, long steps_tot
     return t;
 }
 
+// The tile configuration and reduction split for a problem; cfg == nullptr when no tiled kernel takes it.
+struct GemmPlan {
+    const TileCfg *cfg = nullptr;
+    int nsplit = 1;
+};
+
+GemmPlan plan_gemm(const GemmProblem &p, int steps_total) {
+    GemmPlan plan;
+    const bool gather = p.rowtab != nullptr;
+    const int cus = num_cus();
+    double best_t = 0;
+    // Tuning aids: the gemm_tile switch forces a configuration by name, gemm_split a split count.
+    const Tuning &tune = tuning();
+    const char *force = tune.gemm_tile[0] ? tune.gemm_tile : nullptr;
+    const int fsplit = tune.gemm_split;
+    // The fast kernel addresses each operand as a uniform base plus a 32-bit
+    // per-thread byte offset and moves a partial last step back by up to 15
+    // reduction indices: it needs R >= 16 and tile-local offsets below 2^30 floats.
+    // The output is addressed the same way (four rows and a tile's columns per lane).
+    const long n_img = p.N > 0 ? p.N : p.J;
+    auto offsets_fit = [&](int bm, int bn) {
+        const long offA = p.a_rc ? (long)(bm - 1) * p.sA + GEMM_BK : (long)(GEMM_BK - 1) * p.sA + bm;
+        const long span = (bn - 1) / n_img + 2;  // images a tile's columns can touch
+        const long offB = gather ? p.b_extent
+                          : p.b_rc ? (long)(bn - 1) * p.sB + GEMM_BK
+                                   : (long)(GEMM_BK - 1) * p.sB + span * p.bsB + n_img;
+        const long offC = 4 * (p.sC > p.J ? p.sC : (long)p.J) + span * p.bsC + n_img;
+        return offA < (1L << 30) && offB < (1L << 30) && offC < (1L << 30);
+    };
+    const bool fast_ok = p.R == 0 || p.R >= GEMM_BK;
+    const int layout = gather ? 4 : p.a_rc ? (p.b_rc ? 2 : 0) : (p.b_rc ? 3 : 1);
+    for (const TileCfg &c : kCfgs) {
+        if (!fast_ok || p.M < c.bm || p.J < c.bn || !offsets_fit(c.bm, c.bn)) continue;
+        if (force && std::strcmp(force, c.name) != 0) continue;
+        const long tiles = cdiv(p.M, c.bm) * cdiv(p.J, c.bn);
+        const int max_split = (int)(steps_total / 8 > 0 ? (steps_total / 8 < 256 ? steps_total / 8 : 256) : 1);
+        for (int ns = 1; ns <= max_split; ++ns) {
+            if (fsplit > 0 && ns != (fsplit < max_split ? fsplit : max_split)) continue;
+            if (tiles * ns > 8L * cus * c.resident && ns > 1 && fsplit <= 0) break;
+            const int sps = (int)cdiv(steps_total, ns);
+            if ((int)cdiv(steps_total, sps) != ns) continue;  // would leave an empty split
+            const double t = model_cycles(c, layout, p.M, p.J, steps_total, ns, cus);
+            if (!plan.cfg || t < best_t) {
+                plan.cfg = &c;
+                plan.nsplit = ns;
+                best_t = t;
+            }
+        }
+    }
+    return plan;
+}
+
+inline int steps_of(const GemmProblem &p) {
+    return (p.R + GEMM_BK - 1) / GEMM_BK * (p.nb > 1 ? p.nb : 1);
+}
+
 }  // namespace
+
+bool gemm_tiled_fits(const GemmProblem &p) {
+    if (p.M <= 0 || p.J <= 0 || (long)p.M * p.J >= (1L << 31)) return false;
+    return plan_gemm(p, steps_of(p)).cfg != nullptr;
+}
 
 int gemm_launch(const GemmProblem &p) {
     hipStream_t s = stream();
@@ -138,49 +198,10 @@ int gemm_launch(const GemmProblem &p) {
     g.steps_total = g.steps_per_img * (red ? p.nb : 1);
     g.divSpi = FastDiv((uint32_t)(g.steps_per_img > 0 ? g.steps_per_img : 1));
 
-    // ---- tile configuration and reduction split --------------------------------------
     const int cus = num_cus();
-    const TileCfg *best = nullptr;
-    int best_split = 1;
-    double best_t = 0;
-    // Tuning aids: THGPU_GEMM_TILE forces a configuration by name, THGPU_GEMM_SPLIT a split count.
-    const char *force = std::getenv("THGPU_GEMM_TILE");
-    const char *force_split = std::getenv("THGPU_GEMM_SPLIT");
-    const int fsplit = force_split ? std::atoi(force_split) : 0;
-    // The fast kernel addresses each operand as a uniform base plus a 32-bit
-    // per-thread byte offset and moves a partial last step back by up to 15
-    // reduction indices: it needs R >= 16 and tile-local offsets below 2^30 floats.
-    // The output is addressed the same way (four rows and a tile's columns per lane).
-    const long n_img = g.N;
-    auto offsets_fit = [&](int bm, int bn) {
-        const long offA = p.a_rc ? (long)(bm - 1) * p.sA + GEMM_BK : (long)(GEMM_BK - 1) * p.sA + bm;
-        const long span = (bn - 1) / n_img + 2;  // images a tile's columns can touch
-        const long offB = gather ? p.b_extent
-                          : p.b_rc ? (long)(bn - 1) * p.sB + GEMM_BK
-                                   : (long)(GEMM_BK - 1) * p.sB + span * p.bsB + n_img;
-        const long offC = 4 * (p.sC > p.J ? p.sC : (long)p.J) + span * p.bsC + n_img;
-        return offA < (1L << 30) && offB < (1L << 30) && offC < (1L << 30);
-    };
-    const bool fast_ok = p.R == 0 || p.R >= GEMM_BK;
-    const int layout = gather ? 4 : p.a_rc ? (p.b_rc ? 2 : 0) : (p.b_rc ? 3 : 1);
-    for (const TileCfg &c : kCfgs) {
-        if (!fast_ok || p.M < c.bm || p.J < c.bn || !offsets_fit(c.bm, c.bn)) continue;
-        if (force && std::strcmp(force, c.name) != 0) continue;
-        const long tiles = cdiv(p.M, c.bm) * cdiv(p.J, c.bn);
-        const int max_split = (int)(g.steps_total / 8 > 0 ? (g.steps_total / 8 < 256 ? g.steps_total / 8 : 256) : 1);
-        for (int ns = 1; ns <= max_split; ++ns) {
-            if (fsplit > 0 && ns != (fsplit < max_split ? fsplit : max_split)) continue;
-            if (tiles * ns > 8L * cus * c.resident && ns > 1 && fsplit <= 0) break;
-            const int sps = (int)cdiv(g.steps_total, ns);
-            if ((int)cdiv(g.steps_total, sps) != ns) continue;  // would leave an empty split
-            const double t = model_cycles(c, layout, p.M, p.J, g.steps_total, ns, cus);
-            if (!best || t < best_t) {
-                best = &c;
-                best_split = ns;
-                best_t = t;
-            }
-        }
-    }
+    const GemmPlan plan = plan_gemm(p, g.steps_total);
+    const TileCfg *best = plan.cfg;
+    const int best_split = plan.nsplit;
 
     g.nsplit = best ? best_split : 1;
     const int bm = best ? best->bm : 64, bn = best ? best->bn : 64;
@@ -218,7 +239,7 @@ int gemm_launch(const GemmProblem &p) {
         if (prof_enabled())
             label = prof_label("%s M=%d J=%d R=%ld tile=%s split=%d", p.tag, p.M, p.J, (long)p.R * (red ? p.nb : 1),
                                best ? best->name : "generic", g.nsplit);
-        LaunchScope scope(label, 2.0 * p.M * p.J * (double)p.R * (red ? p.nb : 1), 0.0);
+        LaunchScope scope(label, p.flops > 0 ? p.flops : 2.0 * p.M * p.J * (double)p.R * (red ? p.nb : 1), 0.0);
         rc = best ? best->launch(g, la, lb, red, s) : gemm_generic_64x64(g, p.a_rc, p.b_rc, red, s);
     }
     if (rc) return rc;
@@ -240,12 +261,16 @@ int gemm_launch(const GemmProblem &p) {
 
 using namespace thgpu;
 
-extern "C" void THGPUBlas_gemm(char transa, char transb, long m, long n, long k, float alpha, float *a, long lda,
-                               float *b, long ldb, float beta, float *c, long ldc) {
+namespace {
+
+// Column-major BLAS arguments as a GemmProblem.  Returns 1 for the quick returns of the reference
+// dispatcher (nothing to do), -1 for a dimension the kernels cannot index, 0 otherwise.
+int blas_problem(GemmProblem &p, char transa, char transb, long m, long n, long k, float alpha, const float *a,
+                 long lda, const float *b, long ldb, float beta, float *c, long ldc) {
     const bool ta = (transa == 't' || transa == 'T');
     const bool tb = (transb == 't' || transb == 'T');
     // Quick returns of the reference dispatcher (gputorch/lib/THC/THCBlas.cpp:257).
-    if (!m || !n || ((alpha == 0 || !k) && beta == 1)) return;
+    if (!m || !n || ((alpha == 0 || !k) && beta == 1)) return 1;
     // Degenerate leading dimensions as TH fixes them up (TH/generic/THBlas.c:275-298).
     if (n == 1) ldc = m;
     if (ta) {
@@ -258,14 +283,10 @@ extern "C" void THGPUBlas_gemm(char transa, char transb, long m, long n, long k,
     } else {
         if (n == 1) ldb = k;
     }
-    if (m >= (1L << 31) || n >= (1L << 31) || k >= (1L << 31)) {
-        raise("THGPUBlas_gemm: dimension exceeds 2^31");
-        return;
-    }
+    if (m < 0 || n < 0 || k < 0 || m >= (1L << 31) || n >= (1L << 31) || k >= (1L << 31)) return -1;
     // Column-major C(m x n) is the row-major n x m matrix C'(i', j') =
     // c[j' + i'*ldc]; C' = op(B)' * op(A)' with
     //   A'(i', r) = op(B)(r, i'),  B'(r, j') = op(A)(j', r).
-    GemmProblem p;
     p.A = b;
     p.B = a;
     p.C = c;
@@ -281,6 +302,20 @@ extern "C" void THGPUBlas_gemm(char transa, char transb, long m, long n, long k,
     p.alpha = alpha;
     p.beta = beta;
     p.tag = "gemm_blas";
+    return 0;
+}
+
+}  // namespace
+
+extern "C" void THGPUBlas_gemm(char transa, char transb, long m, long n, long k, float alpha, float *a, long lda,
+                               float *b, long ldb, float beta, float *c, long ldc) {
+    GemmProblem p;
+    const int rc = blas_problem(p, transa, transb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+    if (rc > 0) return;
+    if (rc < 0) {
+        raise("THGPUBlas_gemm: dimension exceeds 2^31");
+        return;
+    }
     if (gemm_launch(p)) raise("%s", thgpu_last_error());
 }
 

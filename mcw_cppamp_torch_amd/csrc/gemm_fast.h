@@ -62,14 +62,7 @@ constexpr int gemm_min_waves() {
     return (BM / WGM) * (BN / WGN) / 64 >= 96 ? 2 : 3;
 }
 
-// DBG is 0 in the library; experiments switch phases off with it (1: no global
-// fetch in the loop, 2: no LDS operand reads, 4: no LDS stores, 8: no barrier,
-// 16: epilogue stores only one value per lane) or instrument the kernel (128:
-// each workgroup writes its shader-clock and wall-clock duration to g.ws; 256:
-// each wavefront accumulates the cycles it spends per step waiting for its LDS
-// operands / issuing MFMAs and loads / waiting for the loads / storing to LDS /
-// at the barrier, and writes the five sums to g.ws past the first 8 MiB).
-template <int BM, int BN, int WGM, int WGN, int LA, int LB, bool RED, int DBG = 0>
+template <int BM, int BN, int WGM, int WGN, int LA, int LB, bool RED>
 __global__ __launch_bounds__(WGM *WGN * 64)
     __attribute__((amdgpu_waves_per_eu(gemm_min_waves<BM, BN, WGM, WGN>()))) void gemm_fast_kernel(const GemmArgs g) {
     constexpr int NT = WGM * WGN * 64;
@@ -93,11 +86,6 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     __shared__ __attribute__((aligned(16))) float As[2][BM][RowA::kPitch];
     __shared__ __attribute__((aligned(16))) float Bs[2][BN][RowB::kPitch];
 
-    long dbg_c0 = 0, dbg_w0 = 0;
-    if (DBG & 128) {
-        dbg_c0 = (long)clock64();
-        dbg_w0 = (long)wall_clock64();
-    }
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: row bases stay uniform
     const int wm = wave / WGN, wn = wave % WGN;
@@ -297,31 +285,17 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     // in slices between its MFMAs (a steady trickle of requests; a burst at the
     // head of the step would hold the wavefront, and with it its MFMAs, in the
     // memory pipeline's queue) and written to the other buffer afterwards.
-    long ph[5] = {0, 0, 0, 0, 0};
-    long tprev = (DBG & 256) ? (long)__builtin_readcyclecounter() : 0;
-#define THGPU_PHASE(k)                                        \
-    if (DBG & 256) {                                          \
-        const long tn = (long)__builtin_readcyclecounter();   \
-        ph[k] += tn - tprev;                                  \
-        tprev = tn;                                           \
-    }
     for (int s = 0; s < nsteps; ++s) {
         const int buf = s & 1;
-        const bool more = !(DBG & 1) && s + 1 < nsteps;
+        const bool more = s + 1 < nsteps;
         // The last step has nothing to fetch; it re-reads the previous addresses
         // (valid, cached) rather than branching around the loads.
         if (more) step_bases(ga, gb, shift);
 
         // MFMA operands: 8 reduction indices per lane and block, two 128-bit reads.
         float4 av[TM][2], bv[TN][2];
-        if (DBG & 2) {
-            for (int h2 = 0; h2 < 2; ++h2) {
-                for (int a = 0; a < TM; ++a) av[a][h2] = make_float4(1.f + lane, 2.f, 3.f, 4.f);
-                for (int b = 0; b < TN; ++b) bv[b][h2] = make_float4(1.f, 2.f + lane, 3.f, 4.f);
-            }
-        }
 #pragma unroll
-        for (int h2 = 0; h2 < 2 && !(DBG & 2); ++h2) {
+        for (int h2 = 0; h2 < 2; ++h2) {
 #pragma unroll
             for (int a = 0; a < TM; ++a)
                 av[a][h2] = *reinterpret_cast<const float4 *>(
@@ -330,10 +304,6 @@ __global__ __launch_bounds__(WGM *WGN * 64)
             for (int b = 0; b < TN; ++b)
                 bv[b][h2] = *reinterpret_cast<const float4 *>(
                     &Bs[buf][wn * (TN * 32) + b * 32 + l32][RowB::col(l32, 8 * half + 4 * h2)]);
-        }
-        if (DBG & 256) {
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            THGPU_PHASE(0)  // LDS operand reads
         }
 #pragma unroll
         for (int h2 = 0; h2 < 2; ++h2) {
@@ -351,41 +321,20 @@ __global__ __launch_bounds__(WGM *WGN * 64)
                         acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, acc[a][b], 0, 0, 0);
                     }
                 }
-                if (!(DBG & 1)) {
 #pragma unroll
-                    for (int u = 0; u < UA; ++u)
-                        if (u * SLICES / UA == slice)
-                            load_unit(std::integral_constant<int, KA>{}, ga, g.sA, voffA, ra, u);
+                for (int u = 0; u < UA; ++u)
+                    if (u * SLICES / UA == slice) load_unit(std::integral_constant<int, KA>{}, ga, g.sA, voffA, ra, u);
 #pragma unroll
-                    for (int u = 0; u < UB; ++u)
-                        if (u * SLICES / UB == slice)
-                            load_unit(std::integral_constant<int, LB>{}, gb, g.sB, voffB, rb, u);
-                }
+                for (int u = 0; u < UB; ++u)
+                    if (u * SLICES / UB == slice) load_unit(std::integral_constant<int, LB>{}, gb, g.sB, voffB, rb, u);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        THGPU_PHASE(1)  // MFMA and load issue
-        if (DBG & 256) {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            THGPU_PHASE(2)  // waiting for the loads
-        }
         if (more) {
-            if (!(DBG & 4)) stash(buf ^ 1, shift);
+            stash(buf ^ 1, shift);
             advance();
         }
-        if (DBG & 256) {
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            THGPU_PHASE(3)  // stash
-        }
-        if (!(DBG & 8)) __syncthreads();
-        THGPU_PHASE(4)  // barrier
-    }
-#undef THGPU_PHASE
-    if (DBG & 256) {
-        if (lane == 0) {
-            long *o = reinterpret_cast<long *>(g.ws) + (1L << 20) + ((long)blockIdx.x * 4 + wave) * 5;
-            for (int k = 0; k < 5; ++k) o[k] = ph[k];
-        }
+        __syncthreads();
     }
 
     // ---- epilogue ----------------------------------------------------------------------
@@ -444,7 +393,6 @@ __global__ __launch_bounds__(WGM *WGN * 64)
                     if (CHECK && !own[b]) continue;
                     float *c = reinterpret_cast<float *>(out + (long)ir * row_bytes + voff[b]);
                     float val = acc[a][b][v];
-                    if ((DBG & 16) && (v != 0 || val != 12345.0f)) continue;
                     if (MODE != 0) val = val * g.alpha + bias_v[v];
                     if (MODE == 2) val += g.beta * *c;
                     *c = val;
@@ -452,12 +400,6 @@ __global__ __launch_bounds__(WGM *WGN * 64)
             }
         }
     };
-    if (DBG & 128) {
-        if (tid == 0) {
-            reinterpret_cast<long *>(g.ws)[2 * blockIdx.x] = (long)clock64() - dbg_c0;
-            reinterpret_cast<long *>(g.ws)[2 * blockIdx.x + 1] = (long)wall_clock64() - dbg_w0;
-        }
-    }
     using std::integral_constant;
     if (g.nsplit > 1) {
         if (edge_tile) write_out(integral_constant<int, 0>{}, integral_constant<bool, true>{});

@@ -44,10 +44,18 @@ struct GemmProblem {
     long rbA = 0, rbB = 0;
     float alpha = 1.0f, beta = 0.0f;
     const char *tag = "gemm";     // name used by per-kernel timing
+    // Flops the per-kernel timing credits the launch with; 0 means the product's own 2*M*J*R*nb.  A
+    // convolution pass sets its algorithmic 2*M*N*K*B here, which a gathered gradInput product (one
+    // column per input pixel) can exceed.
+    double flops = 0.0;
 };
 
 // Enqueues the GEMM on the library stream.  Returns 0 or a recorded error.
 int gemm_launch(const GemmProblem &p);
+// Whether one of the tiled kernels takes the problem (shape at least a tile, operand and output offsets
+// within the kernels' 32-bit addressing, a tile the tuning switches allow): the test a gathered second
+// operand, which has no generic kernel, must pass before it is launched.
+bool gemm_tiled_fits(const GemmProblem &p);
 
 // ---- shared between the kernel translation units ------------------------------
 

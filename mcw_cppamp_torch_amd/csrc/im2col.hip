@@ -219,9 +219,8 @@ bool plan_strips(const ConvGeom &g, long planes, StripPlan &p) {
     const bool grouped = g.N <= 256;                 // several whole planes per workgroup
     const bool whole = !grouped && g.N <= 1024 && bytes(1, g.Ho) <= kLdsBytes;  // one whole plane
     if (grouped && bytes(1, g.Ho) > kLdsBytes) return false;
-    // THGPU_IM2COL_PLAN="v,PL,TG" pins the shape (a tuning aid): v = planes per group or rows per strip.
-    int fv = 0, fPL = 0, fTG = 0;
-    if (const char *e = std::getenv("THGPU_IM2COL_PLAN")) std::sscanf(e, "%d,%d,%d", &fv, &fPL, &fTG);
+    // The im2col_plan switch "v,PL,TG" pins the shape (a tuning aid): v = planes per group or rows per strip.
+    const int fv = tuning().im2col_plan[0], fPL = tuning().im2col_plan[1], fTG = tuning().im2col_plan[2];
     long vmax = grouped ? 1024 / g.N : whole ? g.Ho : 1024 / g.Wo;
     if (grouped && vmax > planes) vmax = planes;
     if (!grouped && vmax > g.Ho) vmax = g.Ho;
@@ -578,11 +577,11 @@ int im2col_launch(const float *im, long B, int C, int H, int W, int kH, int kW, 
     // Kernel choice.  Measured on gfx950: 3x3 unit-stride layers run fastest on the
     // per-position kernel, other unit-stride layers on the LDS-staged strips
     // (many column rows per workgroup favour its few, long stores), strided
-    // first layers on the direct kernel.  THGPU_IM2COL_KERNEL=unit|strip|direct
+    // first layers on the direct kernel.  The im2col_kernel switch (unit | strip | direct)
     // forces one where it applies (a testing and tuning aid).
-    const char *force = std::getenv("THGPU_IM2COL_KERNEL");
-    const bool f_unit = force && !std::strcmp(force, "unit"), f_strip = force && !std::strcmp(force, "strip"),
-               f_direct = force && !std::strcmp(force, "direct");
+    const char *force = tuning().im2col_kernel;
+    const bool f_unit = !std::strcmp(force, "unit"), f_strip = !std::strcmp(force, "strip"),
+               f_direct = !std::strcmp(force, "direct");
     const long span_out = 256 / (long)g.N + 2;  // planes one workgroup of the per-position kernel can touch
     const bool unit_ok = sH == 1 && sW == 1 && kH == kW && (kH == 3 || kH == 5) && planes * g.N < (1L << 32) &&
                          span_out * kH * kW * g.N * 4 < (1L << 32) && span_out * H * W * 4 < (1L << 31);
@@ -716,9 +715,8 @@ int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW,
     const double bytes = 4.0 * ((double)total + (double)B * C * kH * kW * g.Ho * g.Wo);
     // Lane offsets of the unit-stride kernel are 32-bit: the planes one workgroup can touch must span < 4 GiB.
     const long span_planes = 256 / ((long)H * W) + 2;
-    // THGPU_COL2IM_GENERIC=1 forces the general kernel (a testing and tuning aid).
-    const char *generic = std::getenv("THGPU_COL2IM_GENERIC");
-    if (!(generic && generic[0] == '1') && sH == 1 && sW == 1 && kH == kW && (kH == 3 || kH == 5) &&
+    // The col2im_generic switch forces the general kernel (a testing and tuning aid).
+    if (!tuning().col2im_generic && sH == 1 && sW == 1 && kH == kW && (kH == 3 || kH == 5) &&
         span_planes * kH * kW * g.N * 4 < (1L << 32) && total < (1L << 32)) {
         {
             LaunchScope scope(geom_label("col2im", g, B), 0.0, bytes);
@@ -733,7 +731,7 @@ int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW,
     }
     const int th = (kH + sH - 1) / sH, tw = (kW + sW - 1) / sW;
     const int Qh = (H - 1 + pH) / sH + 1, Qw = (W - 1 + pW) / sW + 1;  // quotient ranges of (h+pH)/sH, (w+pW)/sW
-    if (!(generic && generic[0] == '1') && (sW > 1 || sH > 1) && W >= 64 && th <= 3 && tw <= 3) {
+    if (!tuning().col2im_generic && (sW > 1 || sH > 1) && W >= 64 && th <= 3 && tw <= 3) {
         // R quotient rows per workgroup: about 256 (qh, qw) pairs, image rows within the LDS budget
         int R = 256 / Qw;
         if (R < 1) R = 1;

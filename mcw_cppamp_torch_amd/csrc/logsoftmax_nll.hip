@@ -134,7 +134,7 @@ int thgpu_LogSoftMax_updateOutput(THGPUTensor *input, THGPUTensor *output) {
     if (!in) return 1;
     THGPUTensor_resizeAs(output, in);
     int rc = 0;
-    if (!THGPUTensor_isContiguous(output) || THGPUTensor_nElement(output) != nframe * dim)
+    if (!tensor_ready(output, nframe * dim))
         rc = fail("LogSoftMax: could not size output");
     if (!rc && nframe * dim > 0) {
         {
@@ -165,7 +165,7 @@ int thgpu_LogSoftMax_updateGradInput(THGPUTensor *gradOutput, THGPUTensor *outpu
     }
     THGPUTensor_resizeAs(gradInput, out);
     int rc = 0;
-    if (!THGPUTensor_isContiguous(gradInput) || THGPUTensor_nElement(gradInput) != nframe * dim)
+    if (!tensor_ready(gradInput, nframe * dim))
         rc = fail("LogSoftMax: could not size gradInput");
     if (!rc && nframe * dim > 0) {
         {
@@ -218,7 +218,7 @@ int thgpu_ClassNLLCriterion_updateGradInput(THGPUTensor *input, THGPUTensor *tar
     const long ntarget = target->nDimension > 1 ? target->size[1] : 1;
     if (input->nDimension == 1 && ntarget > 1) return fail("multi-target not implemented");
     if (THGPUTensor_nElement(target) != nframe * ntarget) return fail("ClassNLLCriterion: one target per frame expected");
-    if (THGPUTensor_nElement(gradInput) != nframe * ndim || !THGPUTensor_isContiguous(gradInput))
+    if (!tensor_ready(gradInput, nframe * ndim))
         return fail("ClassNLLCriterion: gradInput must be contiguous and sized like the input");
     hipStream_t st = stream();
     if (!st) return 1;

@@ -76,12 +76,14 @@ bool is_columns(const THGPUTensor *t, const ConvShape &s) {
     return t->nDimension == 2 + o && (!s.batched || t->size[0] == s.B) && t->size[o] == s.K && t->size[o + 1] == s.N &&
            THGPUTensor_isContiguous(t);
 }
+bool g_finput_reuse = false;
+
 int size_padded(THGPUTensor *t, const ConvShape &s, int padH, int padW) {
     if (s.batched)
         THGPUTensor_resize4d(t, s.B, s.C, s.H + 2 * padH, s.W + 2 * padW);
     else
         THGPUTensor_resize3d(t, s.C, s.H + 2 * padH, s.W + 2 * padW);
-    if (!is_padded(t, s, padH, padW)) return fail("SpatialConvolutionMM: could not size finput");
+    if (!is_padded(t, s, padH, padW) || !tensor_backed(t)) return fail("SpatialConvolutionMM: could not size finput");
     return 0;
 }
 
@@ -118,10 +120,11 @@ int thgpu_SpatialConvolutionMM_updateOutput(THGPUTensor *input, THGPUTensor *wei
     else
         THGPUTensor_resize3d(output, s.M, s.Ho, s.Wo);
     int rc = 0;
-    if (!THGPUTensor_isContiguous(finput) || !THGPUTensor_isContiguous(output) ||
-        (!gathered && THGPUTensor_nElement(finput) != s.B * s.K * s.N) ||
-        THGPUTensor_nElement(output) != s.B * s.M * s.N)
+    if (!tensor_ready(finput, gathered ? s.B * s.C * (s.H + 2L * padH) * (s.W + 2L * padW) : s.B * s.K * s.N) ||
+        !tensor_ready(output, s.B * s.M * s.N))
         rc = fail("SpatialConvolutionMM: could not size finput/output");
+    if (!rc && !(tensor_backed(in) && tensor_backed(weight) && tensor_backed(bias)))
+        rc = fail("SpatialConvolutionMM: a tensor's shape exceeds its storage");
 
     if (gathered) {
         if (!rc) rc = pad_planes_launch(dptr(in), s.B * s.C, s.H, s.W, padH, padW, dptr(finput));
@@ -151,6 +154,7 @@ int thgpu_SpatialConvolutionMM_updateOutput(THGPUTensor *input, THGPUTensor *wei
         p.N = (int)s.N;
         p.R = s.K;
         p.tag = "gemm_conv_fwd";
+        p.flops = 2.0 * s.M * (double)s.N * s.K * s.B;
         rc = gemm_launch(p);
     }
     THGPUTensor_free(in);
@@ -179,9 +183,10 @@ int thgpu_SpatialConvolutionMM_updateGradInput(THGPUTensor *input, THGPUTensor *
             THGPUTensor_resize3d(gradInput, s.C, s.H, s.W);
         THGPUTensor_resize1d(fgradInput, need);
         int rc = 0;
-        if (!THGPUTensor_isContiguous(gradInput) || !THGPUTensor_isContiguous(fgradInput) ||
-            THGPUTensor_nElement(fgradInput) != need || THGPUTensor_nElement(gradInput) != s.B * (long)s.C * s.H * s.W)
+        if (!tensor_ready(fgradInput, need) || !tensor_ready(gradInput, s.B * (long)s.C * s.H * s.W))
             rc = fail("SpatialConvolutionMM: could not size gradInput/fgradInput");
+        if (!rc && !(tensor_backed(go) && tensor_backed(weight)))
+            rc = fail("SpatialConvolutionMM: a tensor's shape exceeds its storage");
         if (!rc)
             rc = conv_implicit_gradinput(dptr(go), dptr(weight), dptr(fgradInput), dptr(gradInput), s.B, s.C, s.H, s.W,
                                          s.M, kH, kW, padH, padW);
@@ -196,10 +201,10 @@ int thgpu_SpatialConvolutionMM_updateGradInput(THGPUTensor *input, THGPUTensor *
         THGPUTensor_resize2d(fgradInput, s.K, s.N);
     }
     int rc = 0;
-    if (!THGPUTensor_isContiguous(gradInput) || !THGPUTensor_isContiguous(fgradInput) ||
-        THGPUTensor_nElement(fgradInput) != s.B * s.K * s.N ||
-        THGPUTensor_nElement(gradInput) != s.B * (long)s.C * s.H * s.W)
+    if (!tensor_ready(fgradInput, s.B * s.K * s.N) || !tensor_ready(gradInput, s.B * (long)s.C * s.H * s.W))
         rc = fail("SpatialConvolutionMM: could not size gradInput/fgradInput");
+    if (!rc && !(tensor_backed(go) && tensor_backed(weight)))
+        rc = fail("SpatialConvolutionMM: a tensor's shape exceeds its storage");
 
     if (!rc) {
         // fgradInput[b][k][n] = sum_m weight[m][k] * gradOutput[b][m][n]
@@ -219,6 +224,7 @@ int thgpu_SpatialConvolutionMM_updateGradInput(THGPUTensor *input, THGPUTensor *
         p.N = (int)s.N;
         p.R = s.M;
         p.tag = "gemm_conv_gradinput";
+        p.flops = 2.0 * s.M * (double)s.N * s.K * s.B;
         rc = gemm_launch(p);
     }
     if (!rc) rc = col2im_launch(dptr(fgradInput), s.B, s.C, s.H, s.W, kH, kW, padH, padW, dH, dW, dptr(gradInput));
@@ -240,38 +246,42 @@ int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor
     THGPUTensor *go = THGPUTensor_newContiguous(gradOutput);
     if (!go) return 1;
     int rc = 0;
-    if (conv_use_gathered(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW)) {
-        // finput holds the forward's padded input; rebuilt when it does not have that shape
-        if (!is_padded(finput, s, padH, padW)) {
-            THGPUTensor *in = THGPUTensor_newContiguous(input);
-            if (!in) rc = 1;
-            if (!rc) rc = size_padded(finput, s, padH, padW);
+    THGPUTensor *in = THGPUTensor_newContiguous(input);
+    if (!in) {
+        THGPUTensor_free(go);
+        return 1;
+    }
+    if (!(tensor_backed(in) && tensor_backed(go) && tensor_backed(gradWeight) && tensor_backed(gradBias)))
+        rc = fail("SpatialConvolutionMM: a tensor's shape exceeds its storage");
+    // finput is rebuilt from `input` on every call, as the reference GPU code does
+    // (gpunn-impl/SpatialConvolutionMM.cpp:388-396): the result then depends on the arguments alone,
+    // whatever input the last forward pass saw and whoever else shares the buffer.  With
+    // thgpu_conv_set_finput_reuse(1) a finput of the right shape is taken to be the forward's, as the CPU
+    // module takes it (mcw_nn/generic/SpatialConvolutionMM.c:318,336).
+    const bool reuse = g_finput_reuse;
+    if (!rc && conv_use_gathered(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW)) {
+        // finput holds the padded input
+        if (!(reuse && is_padded(finput, s, padH, padW) && tensor_backed(finput))) {
+            rc = size_padded(finput, s, padH, padW);
             if (!rc) rc = pad_planes_launch(dptr(in), s.B * s.C, s.H, s.W, padH, padW, dptr(finput));
-            if (in) THGPUTensor_free(in);
         }
         if (!rc)
             rc = conv_implicit_gradweight(dptr(finput), dptr(go), dptr(gradWeight), s.B, s.C, s.H, s.W, s.M, kH, kW,
                                           padH, padW, dH, dW, scale);
         if (!rc) rc = gradbias_launch(dptr(go), dptr(gradBias), s.B, s.M, s.N, scale);
+        THGPUTensor_free(in);
         THGPUTensor_free(go);
         return rc;
     }
-    // The CPU module reuses the forward's columns (mcw_nn/generic/
-    // SpatialConvolutionMM.c:318,336).  If finput does not have the forward's
-    // shape (the module was never run forward on this input size) the columns
-    // are rebuilt from the input, as the reference GPU code always did
-    // (gpunn-impl/SpatialConvolutionMM.cpp:394-396).
-    if (!is_columns(finput, s)) {
-        THGPUTensor *in = THGPUTensor_newContiguous(input);
+    if (!rc && !(reuse && is_columns(finput, s) && tensor_backed(finput))) {
         if (s.batched)
             THGPUTensor_resize3d(finput, s.B, s.K, s.N);
         else
             THGPUTensor_resize2d(finput, s.K, s.N);
-        if (THGPUTensor_nElement(finput) != s.B * s.K * s.N)
-            rc = fail("SpatialConvolutionMM: could not size finput");
+        if (!tensor_ready(finput, s.B * s.K * s.N)) rc = fail("SpatialConvolutionMM: could not size finput");
         if (!rc) rc = im2col_launch(dptr(in), s.B, s.C, s.H, s.W, kH, kW, padH, padW, dH, dW, dptr(finput));
-        THGPUTensor_free(in);
     }
+    THGPUTensor_free(in);
     if (!rc) {
         // gradWeight[m][k] += scale * sum_b sum_n gradOutput[b][m][n] * finput[b][k][n]
         GemmProblem p;
@@ -293,6 +303,7 @@ int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor
         p.alpha = scale;
         p.beta = 1.0f;
         p.tag = "gemm_conv_gradweight";
+        p.flops = 2.0 * s.M * (double)s.N * s.K * s.B;
         rc = gemm_launch(p);
     }
     if (!rc) rc = gradbias_launch(dptr(go), dptr(gradBias), s.B, s.M, s.N, scale);
@@ -322,8 +333,7 @@ int thgpu_SpatialMaxPooling_updateOutput(THGPUTensor *input, THGPUTensor *output
         THGPUTensor_resize4d(indices, 2, C, Ho, Wo);
     }
     int rc = 0;
-    if (!THGPUTensor_isContiguous(output) || !THGPUTensor_isContiguous(indices) ||
-        THGPUTensor_nElement(output) != B * C * Ho * Wo || THGPUTensor_nElement(indices) != 2 * B * C * Ho * Wo)
+    if (!tensor_ready(output, B * C * Ho * Wo) || !tensor_ready(indices, 2 * B * C * Ho * Wo) || !tensor_backed(in))
         rc = fail("SpatialMaxPooling: could not size output/indices");
     if (!rc) rc = maxpool_fwd_launch(dptr(in), B * C, H, W, kH, kW, dH, dW, dptr(output), dptr(indices));
     THGPUTensor_free(in);
@@ -345,13 +355,13 @@ int thgpu_SpatialMaxPooling_updateGradInput(THGPUTensor *input, THGPUTensor *gra
     if (gradOutput->nDimension != input->nDimension || gradOutput->size[o] != C || gradOutput->size[o + 1] != Ho ||
         gradOutput->size[o + 2] != Wo || (batched && gradOutput->size[0] != B))
         return fail("SpatialMaxPooling: gradOutput size does not match the output size");
-    if (THGPUTensor_nElement(indices) != 2 * B * C * Ho * Wo || !THGPUTensor_isContiguous(indices))
+    if (!tensor_ready(indices, 2 * B * C * Ho * Wo))
         return fail("SpatialMaxPooling: indices do not match (run updateOutput first)");
     THGPUTensor *go = THGPUTensor_newContiguous(gradOutput);
     if (!go) return 1;
     THGPUTensor_resizeAs(gradInput, input);
     int rc = 0;
-    if (!THGPUTensor_isContiguous(gradInput) || THGPUTensor_nElement(gradInput) != B * C * H * W)
+    if (!tensor_ready(gradInput, B * C * H * W) || !tensor_backed(go))
         rc = fail("SpatialMaxPooling: could not size gradInput");
     if (!rc)
         rc = maxpool_bwd_launch(dptr(go), dptr(indices), B * C, H, W, Ho, Wo, kH, kW, dH, dW, dptr(gradInput));
@@ -366,8 +376,7 @@ int thgpu_Threshold_updateOutput(THGPUTensor *input, THGPUTensor *output, float 
     THGPUTensor_resizeAs(output, in);
     long n = THGPUTensor_nElement(in);
     int rc = 0;
-    if (THGPUTensor_nElement(output) != n || !THGPUTensor_isContiguous(output))
-        rc = fail("Threshold: could not size output");
+    if (!tensor_ready(output, n) || !tensor_backed(in)) rc = fail("Threshold: could not size output");
     if (!rc) rc = threshold_fwd_launch(dptr(in), dptr(output), n, threshold, val);
     THGPUTensor_free(in);
     return rc;
@@ -379,12 +388,15 @@ int thgpu_Threshold_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput,
     if (THGPUTensor_nElement(input) != THGPUTensor_nElement(gradOutput))
         return fail("Threshold: input and gradOutput sizes do not match");
     THGPUTensor *in = THGPUTensor_newContiguous(input);
-    THGPUTensor *go = THGPUTensor_newContiguous(gradOutput);
-    if (!in || !go) return 1;
+    THGPUTensor *go = in ? THGPUTensor_newContiguous(gradOutput) : nullptr;
+    if (!in || !go) {
+        if (in) THGPUTensor_free(in);
+        return 1;
+    }
     THGPUTensor_resizeAs(gradInput, in);
     long n = THGPUTensor_nElement(in);
     int rc = 0;
-    if (THGPUTensor_nElement(gradInput) != n || !THGPUTensor_isContiguous(gradInput))
+    if (!tensor_ready(gradInput, n) || !tensor_backed(in) || !tensor_backed(go))
         rc = fail("Threshold: could not size gradInput");
     if (!rc) rc = threshold_bwd_launch(dptr(in), dptr(go), dptr(gradInput), n, threshold);
     THGPUTensor_free(in);
@@ -400,5 +412,12 @@ int thgpu_conv_set_mode(int mode) {
 }
 
 int thgpu_conv_get_mode(void) { return conv_mode(); }
+
+int thgpu_conv_set_finput_reuse(int on) {
+    g_finput_reuse = on != 0;
+    return 0;
+}
+
+int thgpu_conv_get_finput_reuse(void) { return g_finput_reuse ? 1 : 0; }
 
 }  // extern "C"

@@ -480,9 +480,8 @@ int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int
     const int th = (kH + dH - 1) / dH, tw = (kW + dW - 1) / dW;
     const double bytes = 4.0 * ((double)total + 3.0 * ototal);
     PoolBwdPlan plan;
-    // THGPU_POOL_BWD_DIRECT=1 forces the direct kernel (a testing and tuning aid).
-    const char *direct = std::getenv("THGPU_POOL_BWD_DIRECT");
-    if (!(direct && direct[0] == '1') && ((th == 2 && tw == 2) || (th == 1 && tw == 1)) &&
+    // The pool_bwd_direct switch forces the direct kernel (a testing and tuning aid).
+    if (!tuning().pool_bwd_direct && ((th == 2 && tw == 2) || (th == 1 && tw == 1)) &&
         plan_pool_bwd(g, planes, th, tw, plan)) {
         const long blocks = ((planes + plan.G - 1) / plan.G) * plan.tiles;
         if (blocks < (1L << 31)) {

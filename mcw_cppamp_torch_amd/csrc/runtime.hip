@@ -38,6 +38,44 @@ void raise(const char *fmt, ...) {
     g_handler(g_last_error, g_handler_data);
 }
 
+// ---- tuning switches -----------------------------------------------------------
+static Tuning g_tuning;
+static bool g_tuning_read = false;
+
+static int tuning_set(const char *name, const char *value) {
+    const char *v = value ? value : "";
+    if (!std::strcmp(name, "gemm_tile")) {
+        std::snprintf(g_tuning.gemm_tile, sizeof(g_tuning.gemm_tile), "%s", v);
+    } else if (!std::strcmp(name, "gemm_split")) {
+        g_tuning.gemm_split = std::atoi(v);
+    } else if (!std::strcmp(name, "im2col_kernel")) {
+        std::snprintf(g_tuning.im2col_kernel, sizeof(g_tuning.im2col_kernel), "%s", v);
+    } else if (!std::strcmp(name, "im2col_plan")) {
+        g_tuning.im2col_plan[0] = g_tuning.im2col_plan[1] = g_tuning.im2col_plan[2] = 0;
+        std::sscanf(v, "%d,%d,%d", &g_tuning.im2col_plan[0], &g_tuning.im2col_plan[1], &g_tuning.im2col_plan[2]);
+    } else if (!std::strcmp(name, "col2im_generic")) {
+        g_tuning.col2im_generic = v[0] == '1';
+    } else if (!std::strcmp(name, "pool_bwd_direct")) {
+        g_tuning.pool_bwd_direct = v[0] == '1';
+    } else {
+        return fail("thgpu_debug_set: unknown switch '%s'", name);
+    }
+    return 0;
+}
+
+const Tuning &tuning() {
+    if (!g_tuning_read) {
+        g_tuning_read = true;
+        static const char *const kEnv[][2] = {
+            {"THGPU_GEMM_TILE", "gemm_tile"},           {"THGPU_GEMM_SPLIT", "gemm_split"},
+            {"THGPU_IM2COL_KERNEL", "im2col_kernel"},   {"THGPU_IM2COL_PLAN", "im2col_plan"},
+            {"THGPU_COL2IM_GENERIC", "col2im_generic"}, {"THGPU_POOL_BWD_DIRECT", "pool_bwd_direct"}};
+        for (auto &e : kEnv)
+            if (const char *v = std::getenv(e[0])) (void)tuning_set(e[1], v);
+    }
+    return g_tuning;
+}
+
 // ---- stream / device ----------------------------------------------------------
 static hipStream_t g_stream = nullptr;
 static bool g_init_done = false, g_init_ok = false;
@@ -56,6 +94,7 @@ static int init_once() {
     g_cus = prop.multiProcessorCount;
     // Default priority; non-blocking with respect to the legacy null stream.
     THGPU_HIP_TRY(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+    (void)tuning();
     g_init_ok = true;
     return 0;
 }
@@ -84,8 +123,10 @@ float *workspace(size_t bytes) {
         g_ws_bytes = 0;
     }
     size_t want = bytes + bytes / 4;
-    if (hipMalloc(reinterpret_cast<void **>(&g_ws), want) != hipSuccess) {
-        fail("workspace allocation of %zu bytes failed", want);
+    const hipError_t e = hipMalloc(reinterpret_cast<void **>(&g_ws), want);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();  // or the next launch check would report this failure as its own
+        fail("workspace allocation of %zu bytes failed: %s", want, hipGetErrorString(e));
         g_ws = nullptr;
         return nullptr;
     }
@@ -162,6 +203,12 @@ void THGPUSetErrorHandler(THGPUErrorHandler handler, void *data) {
 const char *thgpu_last_error(void) { return g_last_error; }
 
 int thgpu_init(void) { return init_once(); }
+
+int thgpu_debug_set(const char *name, const char *value) {
+    if (!name) return fail("thgpu_debug_set: null name");
+    (void)tuning();  // the environment is read first, so that it never overrides a later call
+    return tuning_set(name, value);
+}
 
 int thgpu_synchronize(void) {
     if (!stream()) return 1;

@@ -199,7 +199,7 @@ int forward(const char *name, bool subsample, THGPUTensor *input, THGPUTensor *w
     else THGPUTensor_resize3d(output, s.C, s.Ho, s.Wo);
     const long total = s.B * s.C * s.Ho * s.Wo;
     int rc = 0;
-    if (!THGPUTensor_isContiguous(output) || THGPUTensor_nElement(output) != total)
+    if (!tensor_ready(output, total))
         rc = fail("%s: could not size output", name);
     if (!rc && total > 0) {
         const char *family = subsample ? "subsample_fwd" : "avgpool_fwd";
@@ -243,7 +243,7 @@ int backward(const char *name, bool subsample, THGPUTensor *input, THGPUTensor *
     THGPUTensor_resizeAs(gradInput, input);
     const long total = s.B * s.C * (long)s.H * s.W;
     int rc = 0;
-    if (!THGPUTensor_isContiguous(gradInput) || THGPUTensor_nElement(gradInput) != total)
+    if (!tensor_ready(gradInput, total))
         rc = fail("%s: could not size gradInput", name);
     if (!rc && total > 0) {
         const char *family = subsample ? "subsample_bwd" : "avgpool_bwd";

@@ -55,25 +55,43 @@ void raw_resize(THGPUTensor *self, int nDimension, const long *size, const long 
     if (same) return;
 
     if (nDimension > 0) {
+        // Transactional: work out the new strides and extent, grow the storage first, and commit the new
+        // shape only when that succeeded.  A failed allocation (the error handler may return) leaves the
+        // tensor exactly as it was, so no caller can be left holding a shape its storage does not back.
+        if (nDimension > THGPU_MAX_DIMS * 4) {
+            raise("Tensor: too many dimensions (%d)", nDimension);
+            return;
+        }
+        long new_stride[THGPU_MAX_DIMS * 4];
+        long total = 1;
+        for (d = nDimension - 1; d >= 0; d--) {
+            if (stride && (stride[d] >= 0))
+                new_stride[d] = stride[d];
+            else
+                new_stride[d] = (d == nDimension - 1) ? 1 : size[d + 1] * new_stride[d + 1];
+            total += (size[d] - 1) * new_stride[d];
+        }
+        // Storage only ever grows here (THCTensor.cpp:677-683).
+        if (total + self->storageOffset > 0) {
+            if (!self->storage) self->storage = THGPUStorage_new();
+            if (!self->storage) return;
+            if (total + self->storageOffset > self->storage->size) {
+                if (!(self->storage->flag & TH_STORAGE_RESIZABLE)) {
+                    raise("Tensor: the storage is too small for the new shape and is not resizable");
+                    return;
+                }
+                THGPUStorage_resize(self->storage, total + self->storageOffset);
+                if (total + self->storageOffset > self->storage->size) return;  // the allocation failed (reported)
+            }
+        }
         if (nDimension != self->nDimension) {
             self->size = static_cast<long *>(std::realloc(self->size, sizeof(long) * nDimension));
             self->stride = static_cast<long *>(std::realloc(self->stride, sizeof(long) * nDimension));
             self->nDimension = nDimension;
         }
-        long total = 1;
-        for (d = nDimension - 1; d >= 0; d--) {
+        for (d = 0; d < nDimension; d++) {
             self->size[d] = size[d];
-            if (stride && (stride[d] >= 0))
-                self->stride[d] = stride[d];
-            else
-                self->stride[d] = (d == nDimension - 1) ? 1 : self->size[d + 1] * self->stride[d + 1];
-            total += (self->size[d] - 1) * self->stride[d];
-        }
-        // Storage only ever grows here (THCTensor.cpp:677-683).
-        if (total + self->storageOffset > 0) {
-            if (!self->storage) self->storage = THGPUStorage_new();
-            if (self->storage && total + self->storageOffset > self->storage->size)
-                THGPUStorage_resize(self->storage, total + self->storageOffset);
+            self->stride[d] = new_stride[d];
         }
     } else
         self->nDimension = 0;

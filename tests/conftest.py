@@ -27,3 +27,21 @@ def _conv_mode_fixture(mode):
 
 columns_route = _conv_mode_fixture(0)    # im2col / GEMM / col2im: finput and fgradInput hold columns
 gathered_route = _conv_mode_fixture(2)   # gathered GEMMs wherever the shape fits
+
+
+@pytest.fixture
+def switches():
+    """Sets testing switches of the library (thgpu_debug_set) for one test; the library's own choices are restored
+    afterwards.  Usage: switches("gemm_tile", "128x128")."""
+    import mcw_cppamp_torch_amd as pkg
+    lib = pkg._lib.lib
+    used = []
+
+    def set_switch(name, value):
+        used.append(name)
+        rc = lib.thgpu_debug_set(name.encode(), None if value is None else str(value).encode())
+        assert rc == 0, lib.thgpu_last_error()
+
+    yield set_switch
+    for name in used:
+        assert lib.thgpu_debug_set(name.encode(), None) == 0

@@ -152,6 +152,40 @@ def rel_err(got, ref):
     return float(np.max(np.abs(got - ref))) / denom
 
 
+def elem_rel_err(got, ref):
+    """Element-wise max relative error over the elements with |ref| > 1e-3 * max|ref| (smaller ones are
+    dominated by cancellation and carry no relative meaning)."""
+    got = np.asarray(got, np.float64)
+    ref = np.asarray(ref, np.float64)
+    top = float(np.max(np.abs(ref)))
+    mask = np.abs(ref) > 1e-3 * top
+    if not mask.any():
+        return 0.0
+    return float(np.max(np.abs(got - ref)[mask] / np.abs(ref)[mask]))
+
+
+MARGIN_LOG = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out",
+                          "parity_margins.jsonl")
+
+
+def check_close(tag, got, ref, k_red):
+    """Asserts the norm-wise bound 1e-4*sqrt(k_red) and puts the observed norm-wise and element-wise errors on
+    record (printed, and appended to gpurun_out/parity_margins.jsonl) so the margin under the bound is known."""
+    norm, elem, bound = rel_err(got, ref), elem_rel_err(got, ref), gemm_tol(k_red)
+    rec = {"case": tag, "k_red": int(k_red), "bound": bound, "norm_rel_err": norm, "elem_rel_err": elem,
+           "bound_used": norm / bound}
+    print("parity %s: norm-wise %.3e, element-wise %.3e, bound %.3e (%.1f %% used)"
+          % (tag, norm, elem, bound, 100.0 * norm / bound), flush=True)
+    try:
+        os.makedirs(os.path.dirname(MARGIN_LOG), exist_ok=True)
+        with open(MARGIN_LOG, "a") as f:
+            f.write(json.dumps(rec) + "\n")
+    except OSError:
+        pass
+    assert norm < bound, rec
+    return rec
+
+
 def gemm_tol(k_red):
     """Parity bound for fp32 GEMM results: 1e-4 * sqrt(reduction length)."""
     return 1e-4 * math.sqrt(max(int(k_red), 1))

@@ -103,6 +103,30 @@ def test_ops_reject_bad_arguments_without_a_device(pkg):
         nn.Threshold("a", 1)
 
 
+def test_switches_are_set_by_name(pkg):
+    L = pkg._lib
+    assert L.lib.thgpu_debug_set(b"no_such_switch", b"1") != 0
+    assert L.lib.thgpu_debug_set(b"gemm_tile", b"128x128") == 0 and L.lib.thgpu_debug_set(b"gemm_tile", None) == 0
+
+
+def test_failed_resize_leaves_the_tensor_unchanged_and_operators_refuse_it(pkg):
+    """A resize whose allocation fails (here: 2^46 floats, or no device at all) must not leave the tensor claiming
+    the new shape over the old buffer; an operator handed such tensors returns an error before any launch."""
+    L = pkg._lib
+    t = pkg.GPUTensor()
+    before = (t.dim(), t.nElement())
+    with pytest.raises(pkg.THGPUError):
+        L.lib.THGPUTensor_resize2d(t._p, 1 << 23, 1 << 23)
+        L.check()
+    assert (t.dim(), t.nElement()) == before
+    assert t._p.contents.nDimension == 0
+    st = t._p.contents.storage
+    assert not st or st.contents.size == 0
+    # the operator sees the old (empty) shape, not a 2^46-element claim over no memory, and refuses it
+    out, ind = pkg.GPUTensor(), pkg.GPUTensor()
+    assert L.lib.thgpu_SpatialMaxPooling_updateOutput(t._p, out._p, ind._p, 2, 2, 2, 2) != 0
+
+
 def test_module_defaults_follow_the_lua_constructors(pkg):
     nn = pkg.nn
     c = nn.SpatialConvolutionMM(3, 8, 5, 7)

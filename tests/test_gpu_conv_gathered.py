@@ -8,7 +8,7 @@ padded input kept in finput bit-exact; repeated runs bit-identical.
 import numpy as np
 import pytest
 
-from helpers import gemm_tol, oracle_stack, rel_err, rng_for, uniform
+from helpers import check_close, gemm_tol, oracle_stack, rel_err, rng_for, uniform
 
 pytestmark = pytest.mark.gpu
 
@@ -99,10 +99,12 @@ def test_gathered_conv_fwd_bwd_parity(gt, gathered_route, cfg):
         assert np.array_equal(bits(got["finput"]), bits(padded(x, pH, pW)))   # the padded input, not columns
     else:
         assert got["finput"].shape == (B, K, N)
-    assert rel_err(got["output"], out_ref) < gemm_tol(K)
-    assert rel_err(got["gradInput"], gi_ref) < gemm_tol(M * kH * kW)
-    assert rel_err(got["gradWeight"], gw_ref) < gemm_tol(B * N)
-    assert rel_err(got["gradBias"], gb_ref) < gemm_tol(B * N)
+    tag = "conv b%d %d->%d %dx%d k%dx%d p%dx%d s%dx%d gathered " % (B, C, M, H, W, kH, kW, pH, pW, sH, sW)
+    check_close(tag + "output", got["output"], out_ref, K)
+    # the gathered gradInput product sums over (output plane, tap) at once: that is its reduction length
+    check_close(tag + "gradInput", got["gradInput"], gi_ref, M * kH * kW)
+    check_close(tag + "gradWeight", got["gradWeight"], gw_ref, B * N)
+    check_close(tag + "gradBias", got["gradBias"], gb_ref, B * N)
 
 
 def test_gathered_matches_column_route_and_reruns_identically(gt, gathered_route):
@@ -198,11 +200,11 @@ def test_gathered_conv_random_geometry(gt, gathered_route, cfg):
 
 @pytest.mark.parametrize("split", [1, 3])
 @pytest.mark.parametrize("tile", ["128x128", "192x128", "64x256", "128x256", "256x128", "64x64"])
-def test_gathered_conv_every_tile_configuration(gt, gathered_route, tile, split, monkeypatch):
+def test_gathered_conv_every_tile_configuration(gt, gathered_route, tile, split, switches):
     """Every tile of the GEMM has its own gathering kernels (plain and reduction-batched); the library's choice
     would leave most of them to the large benchmark shapes, so each is forced here on a shape all of them fit."""
-    monkeypatch.setenv("THGPU_GEMM_TILE", tile)
-    monkeypatch.setenv("THGPU_GEMM_SPLIT", str(split))
+    switches("gemm_tile", tile)
+    switches("gemm_split", split)
     B, C, H, W, M, kH, kW = 2, 256, 12, 12, 256, 3, 3
     geo = (kH, kW, 1, 1, 1, 1)
     K = C * kH * kW
@@ -326,3 +328,54 @@ def test_gathered_alexnet_stack_matches_oracle(gt, gathered_route):
         if g is not None:
             assert rel_err(m.gradWeight.float(), g[0]) < 5e-3
             assert rel_err(m.gradBias.float(), g[1]) < 5e-3
+
+
+@pytest.mark.parametrize("mode", [0, 2], ids=["columns", "gathered"])
+def test_accgradparameters_depends_on_its_arguments_alone(gt, mode):
+    """forward(x1) then accGradParameters(x2): the reference GPU code re-extracts the columns from its `input`
+    argument on every call (gpunn-impl/SpatialConvolutionMM.cpp:388-396), so the result is the oracle's for x2, not
+    a product with the stale buffer of x1; likewise when two same-shaped modules share finput / fgradInput.  With
+    thgpu_conv_set_finput_reuse(1) the buffer is taken on trust, as the CPU module does."""
+    lib = gt._lib.lib
+    B, C, H, W, M, kH, kW = 3, 64, 11, 12, 80, 3, 3
+    geo = (kH, kW, 1, 1, 1, 1)
+    rng = rng_for(49)
+    x1, x2 = uniform(rng, (B, C, H, W)), uniform(rng, (B, C, H, W))
+    w, b = uniform(rng, (M, C * kH * kW), -0.05, 0.05), uniform(rng, (M,))
+    out2, cols2 = oracle.conv_updateOutput(x2, w, b, *geo)
+    go = uniform(rng, out2.shape)
+    gw_ref, gb_ref = np.zeros_like(w), np.zeros_like(b)
+    oracle.conv_accGradParameters(go, cols2, gw_ref, gb_ref, 1.0)
+    before = lib.thgpu_conv_get_mode()
+    assert lib.thgpu_conv_set_mode(mode) == 0 and lib.thgpu_conv_get_finput_reuse() == 0
+    try:
+        def module():
+            m = gt.nn.SpatialConvolutionMM(C, M, kW, kH, 1, 1, 1)
+            m._assign("weight", w)
+            m._assign("bias", b)
+            m.gradWeight[...] = 0
+            m.gradBias[...] = 0
+            return m.gpu()
+        m = module()
+        d1, d2, dgo = dev(gt, x1), dev(gt, x2), dev(gt, go)
+        m.forward(d1)
+        m.accGradParameters(d2, dgo, 1.0)
+        check_close("accGradParameters on another input than the forward's, mode %d" % mode, m.gradWeight.float(),
+                    gw_ref, B * H * W)
+        # two modules sharing their buffers, as memory-saving Torch scripts do
+        a, c = module(), module()
+        c.finput, c.fgradInput = a.finput, a.fgradInput
+        a.forward(d2)
+        c.forward(d1)                       # overwrites the shared finput with x1's
+        a.updateGradInput(d2, dgo)
+        a.accGradParameters(d2, dgo, 1.0)
+        check_close("accGradParameters with a shared finput, mode %d" % mode, a.gradWeight.float(), gw_ref, B * H * W)
+        # opt-in reuse: right after its own forward pass the buffer is the forward's and the result is the same
+        assert lib.thgpu_conv_set_finput_reuse(1) == 0
+        r = module()
+        r.forward(d2)
+        r.accGradParameters(d2, dgo, 1.0)
+        assert np.array_equal(bits(r.gradWeight.float()), bits(a.gradWeight.float()))
+    finally:
+        assert lib.thgpu_conv_set_finput_reuse(0) == 0
+        assert lib.thgpu_conv_set_mode(before) == 0

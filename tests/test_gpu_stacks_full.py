@@ -16,7 +16,7 @@ that path against the reference's plain loops).
 import numpy as np
 import pytest
 
-from helpers import gemm_tol, oracle_stack, rel_err, rng_for, uniform
+from helpers import check_close, oracle_stack, rng_for, uniform
 
 pytestmark = pytest.mark.gpu
 
@@ -90,12 +90,13 @@ def check_layers(gt, name, net, layers, B, x, go, outs, gins, grads, mode):
             _, cin, cout, kW, kH, dW, dH, pW, pH = l
             K = cin * kH * kW
             N = outs[i].shape[2] * outs[i].shape[3]
-            assert rel_err(out, outs[i]) < gemm_tol(K), (name, i)
+            tag = "%s b%d mode%d layer%d " % (name, B, mode, i)
+            check_close(tag + "output", out, outs[i], K)
             gathered = m.finput.dim() == 4   # [B, C, H+2pH, W+2pW] instead of [B, K, N]
             # the gathered gradInput product sums over (plane, tap) at once, the column route over planes
-            assert rel_err(gi, gins[i]) < gemm_tol(cout if mode == 0 else cout * kH * kW), (name, i)
-            assert rel_err(m.gradWeight.float(), grads[i][0]) < gemm_tol(B * N), (name, i)
-            assert rel_err(m.gradBias.float(), grads[i][1]) < gemm_tol(B * N), (name, i)
+            check_close(tag + "gradInput", gi, gins[i], cout if mode == 0 else cout * kH * kW)
+            check_close(tag + "gradWeight", m.gradWeight.float(), grads[i][0], B * N)
+            check_close(tag + "gradBias", m.gradBias.float(), grads[i][1], B * N)
             if gathered:
                 ref_pad = np.pad(ins[i], [(0, 0), (0, 0), (pH, pH), (pW, pW)])
                 assert np.array_equal(bits(m.finput.float()), bits(ref_pad)), (name, i)
