@@ -326,6 +326,20 @@ int thgpu_gemm_strided_batched(char transa, char transb, long m, long n, long k,
                                long stride_a, const float *b, long ldb, long stride_b, float beta, float *c, long ldc,
                                long stride_c, long batch);
 
+/* THGPUBlas_gemm for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments
+ * and result as THGPUBlas_gemm, status returned instead of the error handler being called.  The call
+ * allocates nothing: the partial sums of a split reduction, which THGPUBlas_gemm keeps in a workspace
+ * that grows with hipMalloc, go to a fixed array of THGPU_GEMM_NOALLOC_MAX_ELEMENTS floats (64 MiB) that
+ * the library holds on the GPU from load to exit, and the split is chosen among those whose partial sums
+ * fit it.  Limits: thgpu_init() must have been called (outside any capture; this call sets nothing up and
+ * fails otherwise); a result of more than THGPU_GEMM_NOALLOC_MAX_ELEMENTS elements (m * n) is rejected.
+ * Every call on the GPU shares the one array: calls that overlap in time (other streams or threads) race;
+ * calls through the library stream, which is what this function enqueues on, are ordered. */
+#define THGPU_GEMM_NOALLOC_MAX_ELEMENTS (16L << 20)
+int thgpu_gemm_noalloc(char transa, char transb, long m, long n, long k, float alpha, const float *a, long lda,
+                       const float *b, long ldb, float beta, float *c, long ldc);
+
 /* ---- flat operator entry points -------------------------------------------- */
 
 /* Batched im2col: im [B,C,H,W] -> col [B, C*kH*kW, Ho*Wo] (device pointers).

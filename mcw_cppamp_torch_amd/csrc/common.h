@@ -54,6 +54,9 @@ hipStream_t stream();
 // kernels that use it because everything runs on the one library stream.
 float *workspace(size_t bytes);
 int num_cus();
+// The fixed device array behind the entry points that must not allocate (runtime.hip): its device
+// address and size in floats once the library is initialised, nullptr before (never initialises).
+float *static_scratch(size_t *floats);
 
 // Testing and tuning switches.  Filled from the environment once, when the library initialises
 // (THGPU_GEMM_TILE, THGPU_GEMM_SPLIT, THGPU_IM2COL_KERNEL, THGPU_IM2COL_PLAN, THGPU_COL2IM_GENERIC,

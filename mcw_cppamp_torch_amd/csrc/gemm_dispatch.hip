@@ -136,6 +136,7 @@ GemmPlan plan_gemm(const GemmProblem &p, int steps_total) {
         for (int ns = 1; ns <= max_split; ++ns) {
             if (fsplit > 0 && ns != (fsplit < max_split ? fsplit : max_split)) continue;
             if (tiles * ns > 8L * cus * c.resident && ns > 1 && fsplit <= 0) break;
+            if (ns > 1 && p.ws_fixed && (long)ns * p.M * p.J > p.ws_fixed_floats) break;  // partial sums must fit
             const int sps = (int)cdiv(steps_total, ns);
             if ((int)cdiv(steps_total, sps) != ns) continue;  // would leave an empty split
             const double t = model_cycles(c, layout, p.M, p.J, steps_total, ns, cus);
@@ -212,6 +213,8 @@ int gemm_launch(const GemmProblem &p) {
         const long cap = g.steps_total / 8 > 0 ? g.steps_total / 8 : 1;
         if (want > cap) want = cap;
         if (want < 1) want = 1;
+        if (p.ws_fixed && want * p.M * p.J > p.ws_fixed_floats) want = p.ws_fixed_floats / ((long)p.M * p.J);
+        if (want < 1) want = 1;
         const int sps = (int)cdiv(g.steps_total, want);
         g.nsplit = (int)cdiv(g.steps_total, sps);
     }
@@ -224,7 +227,14 @@ int gemm_launch(const GemmProblem &p) {
     if (total <= 0 || total >= (1L << 31)) return fail("gemm: tile count %ld out of range", total);
     g.total = (unsigned)total;
     if (g.nsplit > 1) {
-        g.ws = workspace(sizeof(float) * (size_t)g.nsplit * p.M * p.J);
+        const size_t need = (size_t)g.nsplit * p.M * p.J;
+        if (p.ws_fixed) {
+            if ((long)need > p.ws_fixed_floats)
+                return fail("gemm: %zu floats of partial sums exceed the fixed workspace of %ld", need, p.ws_fixed_floats);
+            g.ws = p.ws_fixed;
+        } else {
+            g.ws = workspace(sizeof(float) * need);
+        }
         if (!g.ws) return 1;
     }
 
@@ -317,6 +327,26 @@ extern "C" void THGPUBlas_gemm(char transa, char transb, long m, long n, long k,
         return;
     }
     if (gemm_launch(p)) raise("%s", thgpu_last_error());
+}
+
+extern "C" int thgpu_gemm_noalloc(char transa, char transb, long m, long n, long k, float alpha, const float *a,
+                                  long lda, const float *b, long ldb, float beta, float *c, long ldc) {
+    // Nothing here may allocate, so neither may a lazy initialisation: the stream and the address of the
+    // static array exist only after thgpu_init.
+    size_t cap = 0;
+    float *ws = static_scratch(&cap);
+    if (!ws) return fail("thgpu_gemm_noalloc: call thgpu_init() first (this entry point sets nothing up itself)");
+    if (m > 0 && n > 0 && m * n > (long)cap)
+        return fail("thgpu_gemm_noalloc: a result of %ld x %ld elements exceeds the limit of %zu elements (%zu MiB)", m,
+                    n, cap, cap * sizeof(float) >> 20);
+    GemmProblem p;
+    const int rc = blas_problem(p, transa, transb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+    if (rc > 0) return 0;
+    if (rc < 0) return fail("thgpu_gemm_noalloc: dimension exceeds 2^31");
+    p.ws_fixed = ws;
+    p.ws_fixed_floats = (long)cap;
+    p.tag = "gemm_blas_noalloc";
+    return gemm_launch(p);
 }
 
 extern "C" int thgpu_gemm_strided_batched(char transa, char transb, long m, long n, long k, float alpha, const float *a,

@@ -48,6 +48,11 @@ struct GemmProblem {
     // convolution pass sets its algorithmic 2*M*N*K*B here, which a gathered gradInput product (one
     // column per input pixel) can exceed.
     double flops = 0.0;
+    // When non-null the split reduction keeps its partial sums in this caller-provided device buffer of
+    // ws_fixed_floats floats instead of the library's grow-only workspace, and only splits that fit it
+    // are considered: the launch then allocates nothing.
+    float *ws_fixed = nullptr;
+    long ws_fixed_floats = 0;
 };
 
 // Enqueues the GEMM on the library stream.  Returns 0 or a recorded error.

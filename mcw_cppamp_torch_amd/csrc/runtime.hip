@@ -76,6 +76,15 @@ const Tuning &tuning() {
     return g_tuning;
 }
 
+// ---- the array behind the entry points that must not allocate --------------------
+// Device memory the library holds from the moment its code object is loaded until the process
+// ends (64 MiB on every GPU the process uses).  `scratch` is only a host-side handle of the
+// symbol: the device address comes from hipGetSymbolAddress at initialisation and is the only
+// thing ever passed to a kernel.
+constexpr size_t kStaticScratchFloats = (size_t)THGPU_GEMM_NOALLOC_MAX_ELEMENTS;
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
+static float *g_scratch_ptr = nullptr;  // device address of scratch[] on device 0, the one device the library runs on
+
 // ---- stream / device ----------------------------------------------------------
 static hipStream_t g_stream = nullptr;
 static bool g_init_done = false, g_init_ok = false;
@@ -94,9 +103,18 @@ static int init_once() {
     g_cus = prop.multiProcessorCount;
     // Default priority; non-blocking with respect to the legacy null stream.
     THGPU_HIP_TRY(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+    // Device 0 is current: resolve where this device keeps its copy of scratch[].
+    void *sp = nullptr;
+    THGPU_HIP_TRY(hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch)));
+    g_scratch_ptr = static_cast<float *>(sp);
     (void)tuning();
     g_init_ok = true;
     return 0;
+}
+
+float *static_scratch(size_t *floats) {
+    if (floats) *floats = kStaticScratchFloats;
+    return g_init_ok ? g_scratch_ptr : nullptr;
 }
 
 hipStream_t stream() {

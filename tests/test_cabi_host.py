@@ -127,6 +127,13 @@ def test_failed_resize_leaves_the_tensor_unchanged_and_operators_refuse_it(pkg):
     assert L.lib.thgpu_SpatialMaxPooling_updateOutput(t._p, out._p, ind._p, 2, 2, 2, 2) != 0
 
 
+def test_noalloc_gemm_refuses_to_run_before_init_or_beyond_its_limit(pkg):
+    L = pkg._lib
+    null = ctypes.POINTER(ctypes.c_float)()
+    rc = L.lib.thgpu_gemm_noalloc(b"n", b"n", 4, 4, 4, 1.0, null, 4, null, 4, 0.0, null, 4)
+    assert rc != 0 and b"thgpu_init" in L.lib.thgpu_last_error()     # nothing in this CPU-side module initialises
+
+
 def test_module_defaults_follow_the_lua_constructors(pkg):
     nn = pkg.nn
     c = nn.SpatialConvolutionMM(3, 8, 5, 7)
