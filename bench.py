@@ -10,8 +10,13 @@ that are resident in HBM before the timed region starts.  Prints ONE JSON line.
 
 Beside the throughput the line carries
   roofline      the GEMM kernels (fp32 MFMA bound): algorithmic flops of all
-                GEMM launches of a step / their summed HIP-event durations,
-                measured in a second, instrumented run of the same K steps;
+                GEMM launches of a step (2*M*N*K*B per convolution pass, declared
+                at the convolution's launch sites) / their summed HIP-event
+                durations, measured in a second, instrumented run of the same K steps.
+                `traffic` is the HBM bytes per GEMM launch read from the committed
+                rocprofv3 --pmc summary under profiles/, and only when the GEMM
+                launches of this run (shapes, tiles, splits) are the ones that
+                summary was taken on;
   kernels       the same for every kernel family (HBM-bound ones in GB/s);
   gemm_shapes   every GEMM of the stack on its own (shape, chosen tile and split,
                 TFLOP/s): the small-K GEMMs of first layers are HBM-bound themselves;
@@ -24,10 +29,23 @@ Beside the throughput the line carries
   cpu_baseline  the CPU oracle (a port of the reference CPU nn path, OpenMP over
                 the batch + an optimised BLAS sgemm where one is found) timed
                 on this host on a reduced batch of the same stack.
+
+The stack runs with Sequential.fuse() (every ReLU applied by its neighbours as they store
+their results; bit-identical to the separate passes); --no-fuse runs the separate passes.
+
+Other modes
+  --workload ref_benchmark   the reference's own micro-benchmark (gpunn/test/benchmark.lua:7-91): seven single
+                             layers, updateOutput / updateGradInput / accGradParameters timed separately and
+                             reported with its GFLOP/s formula (:118).
+  --summarise kernel-trace|traffic|mfma ...   turns rocprofv3 CSV output into the text summaries kept under
+                             profiles/ (see summarise()).
 """
 import argparse
+import collections
+import csv
 import json
 import os
+import re
 import sys
 import time
 
@@ -37,12 +55,39 @@ sys.path.insert(0, ROOT)
 METRIC = "images/sec fwd+bwd, AlexNet-style conv stack b128 fp32; GEMM % fp32 MFMA peak"
 PEAK_MFMA_F32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per GEMM launch (average over the 15 launches of a step), from two rocprofv3 --pmc runs of this
-# script (FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0, the factors a plain copy kernel of known size gives);
-# the summary with the commands is profiles/hbm_traffic_alexnet_b128_pmc.txt.  Counters cannot be read
-# from inside the timed process, so the figure is carried here for the configuration it was measured on.
-MEASURED_GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("alexnet", 128, "auto"): 1.750e8, ("alexnet", 128, "columns"): 5.339e8}
 ROUTES = {"columns": 0, "auto": 1, "gathered": 2}   # thgpu_conv_set_mode values
+# rocprofv3's FETCH_SIZE / WRITE_SIZE read these fractions of the bytes a plain float4 copy kernel of known size
+# (64 MiB .. 2 GiB) loads / stores on this GPU: counters are scaled by the inverse.
+FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
+
+
+def traffic_profile_path(workload, batch, route):
+    tag = "" if route == "auto" else "_%s_route" % {"columns": "column", "gathered": "gathered"}[route]
+    return os.path.join(ROOT, "profiles", "hbm_traffic_%s_b%d%s_pmc.txt" % (workload, batch, tag))
+
+
+def measured_gemm_traffic(workload, batch, route, fused, gemm_labels):
+    """HBM bytes per GEMM launch from the committed rocprofv3 --pmc summary of this configuration, or (None, why).
+    The summary ends in a `bench_check:` JSON line naming the GEMM launches it was taken on; counters cannot be
+    read from inside the timed process, so the figure is only carried over when this run launched the same GEMMs."""
+    path = traffic_profile_path(workload, batch, route)
+    if not os.path.exists(path):
+        return None, "no traffic summary %s" % os.path.relpath(path, ROOT)
+    check = None
+    for line in open(path):
+        if line.startswith("bench_check:"):
+            check = json.loads(line[len("bench_check:"):])
+    if check is None:
+        return None, "%s has no bench_check line" % os.path.relpath(path, ROOT)
+    if bool(check.get("fused")) != bool(fused):
+        return None, "%s was measured with fused=%s" % (os.path.relpath(path, ROOT), check.get("fused"))
+    if sorted(check["gemm_launches"]) != sorted(gemm_labels):
+        missing = sorted(set(check["gemm_launches"]) - set(gemm_labels))
+        extra = sorted(set(gemm_labels) - set(check["gemm_launches"]))
+        return None, ("the GEMM launches of this run differ from the ones %s was measured on (not in this run: %s; "
+                      "new in this run: %s): re-run the two --pmc passes and bench.py --summarise traffic"
+                      % (os.path.relpath(path, ROOT), missing[:3], extra[:3]))
+    return check["gemm_bytes_per_launch"], None
 
 
 def cpu_baseline(workload, sample_batch, budget_s=12.0):
@@ -108,12 +153,184 @@ def cpu_baseline(workload, sample_batch, budget_s=12.0):
     }
 
 
+# The reference's micro-benchmark layer set (gpunn/test/benchmark.lua:7-91): ni, no, kw, kh, iw, ih, bs, dw, dh.
+REF_BENCHMARK_RUNS = [
+    (3, 96, 11, 11, 128, 128, 128, 1, 1),     # first layer
+    (64, 128, 9, 9, 64, 64, 128, 1, 1),       # second layer
+    (128, 128, 9, 9, 32, 32, 128, 1, 1),      # third layer
+    (128, 128, 7, 7, 16, 16, 128, 1, 1),      # fourth layer
+    (384, 384, 3, 3, 13, 13, 128, 1, 1),      # small inputs/kernels of the lower end of a network
+    (3, 96, 11, 11, 128, 128, 16, 1, 1),      # first layer, tiny batch
+    (64, 128, 9, 9, 64, 64, 16, 1, 1),        # second layer, tiny batch
+]
+
+
+def ref_benchmark(args, pkg):
+    """gpunn/test/benchmark.lua for nn.SpatialConvolutionMM (its BDHW rows): per layer, `steps` calls of updateOutput,
+    of updateGradInput and of accGradParameters, each loop between two synchronisations, GFLOP/s by the reference's
+    formula ni*no*kw*kh*(iw-kw+1)*(ih-kh+1)/dw/dh*bs*2/t (:118)."""
+    import numpy as np
+
+    from mcw_cppamp_torch_amd import gputorch, nn
+
+    rng = np.random.Generator(np.random.PCG64(77))
+    rows, tot_fl, tot_t = [], 0.0, 0.0
+    for ni, no, kw, kh, iw, ih, bs, dw, dh in REF_BENCHMARK_RUNS:
+        m = nn.SpatialConvolutionMM(ni, no, kw, kh, dw, dh, rng=rng).gpu()
+        x = pkg.FloatTensor(rng.standard_normal((bs, ni, ih, iw)).astype(np.float32)).gpu()
+        o = m.forward(x)
+        flops = ni * no * kw * kh * (iw - kw + 1) * (ih - kh + 1) / dw / dh * bs * 2
+        row = {"config": "input %dx%dx%d * ker %dx%dx%dx%d (bs = %d, stride = %d)" % (ni, iw, ih, ni, no, kw, kh, bs, dw)}
+        for name, call in (("updateOutput", lambda: m.updateOutput(x)),
+                           ("updateGradInput", lambda: m.updateGradInput(x, o)),
+                           ("accGradParameters", lambda: m.accGradParameters(x, o))):
+            for _ in range(args.warmup):
+                call()
+            gputorch.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                call()
+            gputorch.synchronize()
+            tm = (time.perf_counter() - t0) / args.steps
+            row[name] = {"gflops": round(flops / tm / 1e9, 1), "ms": round(tm * 1e3, 4),
+                         "frac_of_fp32_mfma_peak": round(flops / tm / 1e12 / PEAK_MFMA_F32_TFLOPS, 4)}
+            tot_fl += flops
+            tot_t += tm
+        rows.append(row)
+        del m, x, o
+    print(json.dumps({
+        "metric": "GFLOP/s of nn.SpatialConvolutionMM on the reference's benchmark layer set "
+                  "(gpunn/test/benchmark.lua), its own formula",
+        "value": round(tot_fl / tot_t / 1e9, 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(tot_t * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "seven single layers, three passes each timed on its own; value = all flops / all time",
+                   "device": gputorch.getDeviceProperties()["name"]},
+        "layers": rows}))
+
+
+# ---- rocprofv3 output -> the text summaries under profiles/ ----------------------------------------------------------
+
+def _short(name):
+    name = name.replace("thgpu::(anonymous namespace)::", "").replace("void ", "").replace("thgpu::", "")
+    return re.sub(r"\(.*", "", name)
+
+
+FAMILIES = [("gemm_fast", "gemm"), ("gemm_generic", "gemm"), ("im2col", "im2col"), ("col2im", "col2im"),
+            ("maxpool_bwd", "maxpool_bwd"), ("maxpool_fwd", "maxpool_fwd"), ("threshold_fwd", "threshold_fwd"),
+            ("threshold_bwd", "threshold_bwd"), ("split_reduce", "gemm_split_reduce"),
+            ("gradbias_partial", "gradbias"), ("gradbias_final", "gradbias_final"), ("fill_kernel", "fill"),
+            ("pad_planes", "pad_planes"), ("flip_weight", "flip_weight")]
+
+
+def _family(kernel_name):
+    for key, fam in FAMILIES:
+        if key in kernel_name:
+            return fam
+    return None
+
+
+def summarise(args):
+    """bench.py --summarise kernel-trace STATS.csv BENCH.json STEPS   (rocprofv3 --kernel-trace --stats ... _kernel_stats.csv)
+    bench.py --summarise traffic FETCH.csv WRITE.csv BENCH.json STEPS  (two --pmc runs' _counter_collection.csv)
+    bench.py --summarise mfma COUNTERS.csv                             (one --pmc run with the SQ_* counters)
+    BENCH.json is the line an ordinary run of the same configuration printed; STEPS the steps the profiled runs made
+    (warm-up included).  Writes the summary to stdout; `header` lines (the commands) come from --summary-header."""
+    kind, files = args.summarise[0], args.summarise[1:]
+    out = [l for l in (args.summary_header or "").split("\\n") if l] + [""]
+    if kind == "kernel-trace":
+        stats, bench, steps = files[0], json.load(open(files[1])), int(files[2])
+        out.append("%-66s %6s %12s %10s %6s" % ("kernel", "calls", "total_ms", "avg_us", "%"))
+        tot = gemm = 0.0
+        gcalls = 0
+        for r in csv.DictReader(open(stats)):
+            ms = float(r["TotalDurationNs"]) / 1e6
+            tot += ms
+            if _family(r["Name"]) == "gemm":
+                gemm += ms
+                gcalls += int(r["Calls"])
+            out.append("%-66s %6s %12.3f %10.1f %6.2f" % (_short(r["Name"])[:66], r["Calls"], ms,
+                                                           float(r["AverageNs"]) / 1e3, float(r["Percentage"])))
+        fl = bench["roofline"]["flops_per_step"]
+        out += ["", "All kernels: %.3f ms per step.  GEMM kernels (%d launches per step): %.3f ms per step"
+                % (tot / steps, gcalls / steps, gemm / steps),
+                "-> %.3f GFLOP of convolution GEMM work per step / %.3f ms = %.1f TFLOP/s = %.1f %% of the %.1f TFLOP/s "
+                "fp32 MFMA peak; average GEMM launch %.1f us."
+                % (fl / 1e9, gemm / steps, fl / (gemm / steps) / 1e9, fl / (gemm / steps) / 1e9 / PEAK_MFMA_F32_TFLOPS * 100,
+                   PEAK_MFMA_F32_TFLOPS, gemm / gcalls * 1e3),
+                "bench.py's own HIP-event measurement of the same launches in the same configuration: %.3f ms per step "
+                "(%.2f TFLOP/s); its throughput in that run: %.0f images/s (%.3f ms per step)."
+                % (bench["roofline"]["ms_per_step"], bench["roofline"]["achieved"], bench["value"], bench["ms_per_step"])]
+    elif kind == "traffic":
+        def load(path):
+            d = collections.OrderedDict()
+            for r in csv.DictReader(open(path)):
+                d[int(r["Dispatch_Id"])] = (r["Kernel_Name"], float(r["Counter_Value"]))
+            return d
+        fetch, write = load(files[0]), load(files[1])
+        bench, steps = json.load(open(files[2])), int(files[3])
+        fam = collections.OrderedDict()
+        for k, (name, v) in fetch.items():
+            f = _family(name)
+            if f is None or k not in write:
+                continue
+            a = fam.setdefault(f, [0, 0.0, 0.0])
+            a[0] += 1
+            a[1] += v * FETCH_SCALE / 1024
+            a[2] += write[k][1] * WRITE_SCALE / 1024
+        alg = {k: v["gbs"] * 1e6 * v["ms_per_step"] / 1048576 for k, v in bench["kernels"].items() if "gbs" in v}
+        out.append("Counters are KiB per dispatch; FETCH_SIZE is scaled by %.1f and WRITE_SIZE by %.1f, the factors a plain "
+                   "float4 copy kernel of known size (64 MiB .. 2 GiB) gives for the same counters on this GPU."
+                   % (FETCH_SCALE, WRITE_SCALE))
+        out += ["", "%-22s %9s %12s %12s %12s %15s %8s" % ("kernel family", "launches", "fetch MiB", "write MiB", "total MiB",
+                                                        "algorithmic MiB", "ratio"),
+                "%-22s %9s %12s %12s %12s %15s %8s" % ("", "per step", "per step", "per step", "per step", "per step", "")]
+        total = 0.0
+        for f, a in fam.items():
+            n, fe, wr = a[0] / steps, a[1] / steps, a[2] / steps
+            total += fe + wr
+            al = alg.get(f)
+            out.append("%-22s %9.1f %12.1f %12.1f %12.1f %15s %8s" % (f, n, fe, wr, fe + wr, ("%.1f" % al) if al else "-",
+                                                                    ("%.2f" % ((fe + wr) / al)) if al else "-"))
+        g = fam["gemm"]
+        per = (g[1] + g[2]) / g[0]
+        out += ["", "All kernels: %.1f MiB per step." % total,
+                "GEMM family: %.1f MiB per step over %d launches = %.1f MiB (%.4g bytes) per launch on average."
+                % ((g[1] + g[2]) / steps, g[0] / steps, per, per * 1048576),
+                "bench_check: " + json.dumps({
+                    "workload": bench["config"]["workload"].split(" ")[0], "batch": bench["config"]["batch"],
+                    "route": bench["config"]["conv_route"], "fused": bench["config"].get("relu_fused", False),
+                    "gemm_bytes_per_launch": round(per * 1048576), "gemm_launches": [s["gemm"] for s in bench["gemm_shapes"]]})]
+    elif kind == "mfma":
+        agg = collections.OrderedDict()
+        for r in csv.DictReader(open(files[0])):
+            if _family(r["Kernel_Name"]) != "gemm":
+                continue
+            key = (_short(r["Kernel_Name"]), r["Grid_Size"])
+            agg.setdefault(key, collections.defaultdict(float))[r["Counter_Name"]] += float(r["Counter_Value"])
+            agg[key]["_n_" + r["Counter_Name"]] += 1
+        out.append("%-58s %9s %9s %9s %9s %9s" % ("kernel (grid)", "launches", "mfma_busy", "wait_any", "wait_lds", "lds_confl"))
+        for (name, grid), c in agg.items():
+            n = c["_n_SQ_BUSY_CU_CYCLES"] or 1
+            busy = c["SQ_VALU_MFMA_BUSY_CYCLES"] / max(c["SQ_BUSY_CU_CYCLES"], 1) / 4   # per SIMD of a busy CU
+            wave = max(c["SQ_WAVE_CYCLES"], 1)
+            out.append("%-58s %9d %8.1f%% %8.1f%% %8.1f%% %8.2f%%" % (
+                ("%s (%s)" % (name, grid))[:58], n, 100 * busy, 100 * c["SQ_WAIT_INST_ANY"] / wave,
+                100 * c["SQ_WAIT_INST_LDS"] / wave, 100 * c["SQ_LDS_BANK_CONFLICT"] / max(c["SQ_ACTIVE_INST_LDS"], 1)))
+        out.append("mfma_busy = SQ_VALU_MFMA_BUSY_CYCLES / (4 * SQ_BUSY_CU_CYCLES); wait_* = SQ_WAIT_INST_* / SQ_WAVE_CYCLES; "
+                   "lds_confl = SQ_LDS_BANK_CONFLICT / SQ_ACTIVE_INST_LDS.")
+    else:
+        sys.exit("--summarise kernel-trace | traffic | mfma")
+    print("\n".join(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="alexnet", choices=["alexnet", "overfeat", "vgg_a", "conv1_b16"])
+    ap.add_argument("--workload", default="alexnet",
+                    choices=["alexnet", "overfeat", "vgg_a", "conv1_b16", "ref_benchmark"])
     ap.add_argument("--batch", type=int, default=None, help="override the workload's batch size")
     ap.add_argument("--cpu-sample-batch", type=int, default=128)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -122,7 +339,15 @@ def main():
                     help="how nn.SpatialConvolutionMM computes: im2col/GEMM/col2im columns, GEMMs that gather from "
                          "the padded image, or the library's choice per layer (its default)")
     ap.add_argument("--no-column-route", action="store_true", help="skip the second measurement on the column route")
+    ap.add_argument("--no-fuse", action="store_true", help="run every ReLU as a pass of its own (no Sequential.fuse())")
+    ap.add_argument("--reuse-finput", action="store_true",
+                    help="accGradParameters trusts the forward pass's finput (the CPU module's behaviour) instead of "
+                         "rebuilding it from its input (the reference GPU code's, the library's default)")
+    ap.add_argument("--summarise", nargs="+", metavar="ARG", help="see summarise()")
+    ap.add_argument("--summary-header", default=None, help="text put at the top of a --summarise output (\\n separated)")
     args = ap.parse_args()
+    if args.summarise:
+        return summarise(args)
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the path is built and measured on a single MI355X "
                  "(--gpus %d is not supported: every GPU box of this build has one GPU, and the value reported "
@@ -136,10 +361,16 @@ def main():
     lib = pkg._lib.lib
     if lib.thgpu_init() != 0:
         sys.exit("no GPU: " + lib.thgpu_last_error().decode())
+    lib.thgpu_conv_set_finput_reuse(1 if args.reuse_finput else 0)
+    if args.workload == "ref_benchmark":
+        return ref_benchmark(args, pkg)
 
     name = args.workload
     B = args.batch or stacks.STACKS[name]["batch"]
+    fused = not args.no_fuse
     net = stacks.build(name, seed_base=1000).gpu()
+    if fused:
+        net.fuse()
     x = pkg.FloatTensor(stacks.make_input(name, B, seed=1000)).gpu()
     rng = np.random.Generator(np.random.PCG64(1003))
     go = pkg.FloatTensor(rng.uniform(-1, 1, stacks.output_shape(name, B)).astype(np.float32)).gpu()
@@ -218,11 +449,18 @@ def main():
                 if by > 0:
                     ent.update(bound="hbm", gbs=round(by / ms / 1e6, 1), frac=round(by / ms / 1e6 / PEAK_HBM_GBS, 4))
         if g_ms > 0:
+            traffic, why = measured_gemm_traffic(name, B, route, fused, [s["gemm"] for s in gemm_shapes])
+            if why:
+                print("bench.py: roofline.traffic is null: " + why, file=sys.stderr)
+            algorithmic = stacks.work(name, B)["gemm_flops"]
+            if abs(g_fl - algorithmic) > 1e-6 * algorithmic:
+                sys.exit("bench.py: the GEMM launches of a step declare %.6g flops, the stack's 3 x 2*M*N*K*B is %.6g"
+                         % (g_fl, algorithmic))
             res["roofline"] = {
                 "bound": "mfma", "kernel": "gemm_fast_kernel<...> (all conv GEMM launches of a step)",
                 "achieved": round(g_fl / g_ms / 1e9, 2), "peak": PEAK_MFMA_F32_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(g_fl / g_ms / 1e9 / PEAK_MFMA_F32_TFLOPS, 4),
-                "traffic": MEASURED_GEMM_TRAFFIC_BYTES_PER_LAUNCH.get((name, B, route)),
+                "traffic": traffic, "traffic_note": why,
                 "launches_per_step": g_calls / steps, "ms_per_step": round(g_ms, 4),
                 "flops_per_step": g_fl,
             }
@@ -269,7 +507,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s conv stack, batch %d, input %s, fwd+bwd (zeroGradParameters, forward, "
                                "updateGradInput, accGradParameters)" % (name, B, "x".join(map(str, stacks.STACKS[name]["input"]))),
-                   "batch": B, "conv_route": args.conv_route, "device": gputorch.getDeviceProperties()["name"]},
+                   "batch": B, "conv_route": args.conv_route, "relu_fused": fused, "finput_reuse": bool(args.reuse_finput),
+                   "device": gputorch.getDeviceProperties()["name"]},
         "device_ms_per_step": round(main_run["device_ms_per_step"], 4),
         "transfers": {"h2d_input_ms": round(h2d_ms, 3), "d2h_gradinput_ms": round(d2h_ms, 3),
                       "images_per_s_including_transfers": round(B / ((ms_per_step + h2d_ms + d2h_ms) / 1e3), 1)},

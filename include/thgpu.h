@@ -108,9 +108,9 @@ int thgpu_init(void);
 
 /* Testing and tuning switches (no counterpart in the reference).  name: gemm_tile (a tile configuration such
  * as "128x128"), gemm_split (a reduction split count), im2col_kernel (unit | strip | direct), im2col_plan
- * ("v,PL,TG"), col2im_generic ("1"), pool_bwd_direct ("1"); value NULL or "" restores the library's own
- * choice.  The environment variables THGPU_GEMM_TILE, THGPU_GEMM_SPLIT, THGPU_IM2COL_KERNEL, THGPU_IM2COL_PLAN,
- * THGPU_COL2IM_GENERIC and THGPU_POOL_BWD_DIRECT give the initial values and are read once, when the library
+ * ("v,PL,TG"), col2im_generic ("1"), pool_fwd_wave ("1"), pool_bwd_direct ("1"); value NULL or "" restores the
+ * library's own choice.  The environment variables THGPU_GEMM_TILE, THGPU_GEMM_SPLIT, THGPU_IM2COL_KERNEL,
+ * THGPU_IM2COL_PLAN, THGPU_COL2IM_GENERIC, THGPU_POOL_FWD_WAVE and THGPU_POOL_BWD_DIRECT give the initial values and are read once, when the library
  * initialises; no operator call reads the environment. */
 int thgpu_debug_set(const char *name, const char *value);
 
@@ -381,6 +381,23 @@ int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor
                                                  THGPUTensor *finput, THGPUTensor *fgradInput, int kW, int kH,
                                                  int dW, int dH, int padW, int padH, float scale);
 
+/* nn.Threshold fused into its neighbours (no counterpart in the reference, where gpunn_Threshold_updateOutput /
+ * _updateGradInput, gpunn-impl/Threshold.cpp:16-81, always run as passes of their own).
+ * updateOutputThreshold: output = y > threshold ? y : val for every y = conv(input) + bias, applied as the
+ *   value is stored; bit-identical to updateOutput followed by thgpu_Threshold_updateOutput in place.
+ * updateGradInputMasked: gradInput = input > threshold ? g : 0 for every g of updateGradInput, applied as the
+ *   value is stored -- the backward of a Threshold in front of this module, whose output `input` is
+ *   (value <= threshold assumed, so that its output exceeds the threshold exactly where its input did);
+ *   bit-identical to updateGradInput followed by thgpu_Threshold_updateGradInput. */
+int thgpu_SpatialConvolutionMM_updateOutputThreshold(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias,
+                                                     THGPUTensor *finput, THGPUTensor *fgradInput,
+                                                     THGPUTensor *output, int kW, int kH, int dW, int dH, int padW,
+                                                     int padH, float threshold, float val);
+int thgpu_SpatialConvolutionMM_updateGradInputMasked(THGPUTensor *input, THGPUTensor *gradOutput,
+                                                     THGPUTensor *weight, THGPUTensor *finput,
+                                                     THGPUTensor *fgradInput, THGPUTensor *gradInput, int kW, int kH,
+                                                     int dW, int dH, int padW, int padH, float threshold);
+
 /* How the three entry points above compute (no counterpart in the reference, whose only route is
  * im2col + sgemm + col2im, gpunn-impl/SpatialConvolutionMM.cpp:110-429).
  *   mode 0: that route; finput and fgradInput hold the K x N columns as in the reference.
@@ -413,6 +430,12 @@ int thgpu_SpatialMaxPooling_updateOutput(THGPUTensor *input, THGPUTensor *output
                                          int kH, int dW, int dH);
 int thgpu_SpatialMaxPooling_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *gradInput,
                                             THGPUTensor *indices, int kW, int kH, int dW, int dH);
+
+/* updateGradInput with the backward of a Threshold in front of the pooling layer applied as gradInput is stored:
+ * gradInput = input > threshold ? g : 0 (see thgpu_SpatialConvolutionMM_updateGradInputMasked). */
+int thgpu_SpatialMaxPooling_updateGradInputMasked(THGPUTensor *input, THGPUTensor *gradOutput,
+                                                  THGPUTensor *gradInput, THGPUTensor *indices, int kW, int kH,
+                                                  int dW, int dH, float threshold);
 
 /* nn.Threshold / nn.ReLU.  Replace gpunn_Threshold_updateOutput /
  * _updateGradInput (gpunn-impl/Threshold.cpp:16-38, 53-81). */

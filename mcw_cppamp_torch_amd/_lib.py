@@ -187,6 +187,9 @@ _SIGNATURES = {
     "thgpu_SpatialConvolutionMM_updateOutput": (c_int, [TensorP] * 6 + [c_int] * 6),
     "thgpu_SpatialConvolutionMM_updateGradInput": (c_int, [TensorP] * 6 + [c_int] * 6),
     "thgpu_SpatialConvolutionMM_accGradParameters": (c_int, [TensorP] * 6 + [c_int] * 6 + [c_float]),
+    "thgpu_SpatialConvolutionMM_updateOutputThreshold": (c_int, [TensorP] * 6 + [c_int] * 6 + [c_float] * 2),
+    "thgpu_SpatialConvolutionMM_updateGradInputMasked": (c_int, [TensorP] * 6 + [c_int] * 6 + [c_float]),
+    "thgpu_SpatialMaxPooling_updateGradInputMasked": (c_int, [TensorP] * 4 + [c_int] * 4 + [c_float]),
     "thgpu_SpatialMaxPooling_updateOutput": (c_int, [TensorP] * 3 + [c_int] * 4),
     "thgpu_SpatialMaxPooling_updateGradInput": (c_int, [TensorP] * 4 + [c_int] * 4),
     "thgpu_Threshold_updateOutput": (c_int, [TensorP] * 2 + [c_float] * 2),

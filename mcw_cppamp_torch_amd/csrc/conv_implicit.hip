@@ -283,7 +283,7 @@ int pad_planes_launch(const float *in, long planes, int H, int W, int pH, int pW
 }
 
 int conv_implicit_forward(const float *padded, const float *weight, const float *bias, float *output, long B, int C,
-                          int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
+                          int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW, OutputThreshold act) {
     const int Hp = H + 2 * pH, Wp = W + 2 * pW;
     const int Ho = (Hp - kH) / sH + 1, Wo = (Wp - kW) / sW + 1;
     if (trim_tables()) return 1;
@@ -295,6 +295,9 @@ int conv_implicit_forward(const float *padded, const float *weight, const float 
     if (!p.rowtab || !p.coltab) return 1;
     p.C = output;
     p.bias = bias;
+    p.act = act.on;
+    p.act_threshold = act.threshold;
+    p.act_value = act.value;
     return gemm_launch(p);
 }
 
@@ -315,7 +318,7 @@ int conv_implicit_gradweight(const float *padded, const float *gradOutput, float
 }
 
 int conv_implicit_gradinput(const float *gradOutput, const float *weight, float *scratch, float *gradInput, long B,
-                            int C, int H, int W, int M, int kH, int kW, int pH, int pW) {
+                            int C, int H, int W, int M, int kH, int kW, int pH, int pW, InputMask mask) {
     hipStream_t s = stream();
     if (!s) return 1;
     const int Ho = H + 2 * pH - kH + 1, Wo = W + 2 * pW - kW + 1;
@@ -339,6 +342,8 @@ int conv_implicit_gradinput(const float *gradOutput, const float *weight, float 
     p.coltab = pixel_table(H, W, Wq, 1);
     if (!p.rowtab || !p.coltab) return 1;
     p.C = gradInput;
+    p.mask = mask.in;
+    p.mask_threshold = mask.threshold;
     return gemm_launch(p);
 }
 

@@ -15,7 +15,9 @@ namespace {
 __global__ __launch_bounds__(256) void split_reduce_kernel(const float *__restrict__ ws, float *__restrict__ C,
                                                            const float *__restrict__ bias, int M, int J, int N,
                                                            long sC, long bsC, FastDiv divJ, FastDiv divN, int nsplit,
-                                                           float alpha, float beta) {
+                                                           float alpha, float beta, int act, float act_threshold,
+                                                           float act_value, const float *__restrict__ mask,
+                                                           float mask_threshold) {
     unsigned idx = blockIdx.x * blockDim.x + threadIdx.x;
     const unsigned total = (unsigned)M * (unsigned)J;
     if (idx >= total) return;
@@ -42,6 +44,8 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(const float *__restri
     float val = alpha * sum;
     if (bias) val += bias[i];
     if (beta != 0.0f) val += beta * *c;
+    if (act) val = val > act_threshold ? val : act_value;
+    if (mask) val = mask[c - C] > mask_threshold ? val : 0.0f;
     *c = val;
 }
 
@@ -195,6 +199,11 @@ int gemm_launch(const GemmProblem &p) {
     g.divN = FastDiv((uint32_t)g.N);
     g.alpha = p.alpha;
     g.beta = p.beta;
+    g.act = p.act ? 1 : 0;
+    g.act_threshold = p.act_threshold;
+    g.act_value = p.act_value;
+    g.mask = p.mask;
+    g.mask_threshold = p.mask_threshold;
     g.steps_per_img = (p.R + GEMM_BK - 1) / GEMM_BK;
     g.steps_total = g.steps_per_img * (red ? p.nb : 1);
     g.divSpi = FastDiv((uint32_t)(g.steps_per_img > 0 ? g.steps_per_img : 1));
@@ -260,7 +269,7 @@ int gemm_launch(const GemmProblem &p) {
             LaunchScope scope("gemm_split_reduce", 0.0, 4.0 * n * (g.nsplit + 2));
             hipLaunchKernelGGL(split_reduce_kernel, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, s, g.ws, p.C, p.bias,
                                p.M, p.J, g.N, p.sC, p.bsC, FastDiv((uint32_t)p.J), g.divN, g.nsplit, p.alpha,
-                               p.beta);
+                               p.beta, g.act, g.act_threshold, g.act_value, g.mask, g.mask_threshold);
         }
         if (check_launch("gemm_split_reduce")) return 1;
     }

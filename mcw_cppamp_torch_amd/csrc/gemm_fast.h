@@ -349,6 +349,10 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         const long row_bytes = (MODE == 0 ? (long)g.J : g.sC) * 4;
         char *const out0 = MODE == 0 ? reinterpret_cast<char *>(g.ws + (long)split * g.M * g.J)
                                      : reinterpret_cast<char *>(g.C);
+        // Fused threshold / mask of the final value (uniform conditions; both off for partial sums).
+        const bool act = MODE != 0 && g.act != 0;
+        const bool masked = MODE != 0 && g.mask != nullptr;
+        const long mask_delta = masked ? reinterpret_cast<const char *>(g.mask) - reinterpret_cast<const char *>(g.C) : 0L;
         unsigned img0 = 0, n0 = 0;
         const bool per_image = MODE != 0 && !RED && g.N != g.J;
         if (per_image) g.divN.divmod((unsigned)j0, img0, n0);
@@ -395,6 +399,11 @@ __global__ __launch_bounds__(WGM *WGN * 64)
                     float val = acc[a][b][v];
                     if (MODE != 0) val = val * g.alpha + bias_v[v];
                     if (MODE == 2) val += g.beta * *c;
+                    if (act) val = val > g.act_threshold ? val : g.act_value;
+                    if (masked) {
+                        const float mv = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(c) + mask_delta);
+                        val = mv > g.mask_threshold ? val : 0.0f;
+                    }
                     *c = val;
                 }
             }

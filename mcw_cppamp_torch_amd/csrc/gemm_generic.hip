@@ -211,6 +211,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_generic_kernel(const GemmA
                     val *= g.alpha;
                     if (g.bias) val += g.bias[i];
                     if (g.beta != 0.0f) val += g.beta * *c;
+                    if (g.act) val = val > g.act_threshold ? val : g.act_value;
+                    if (g.mask) val = g.mask[c - g.C] > g.mask_threshold ? val : 0.0f;
                     *c = val;
                 }
             }

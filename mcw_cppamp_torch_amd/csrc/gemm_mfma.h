@@ -43,6 +43,14 @@ struct GemmProblem {
     int nb = 1;
     long rbA = 0, rbB = 0;
     float alpha = 1.0f, beta = 0.0f;
+    // Fused into the store of the final value (after alpha, bias and beta), in this order:
+    //   act:  C = C > act_threshold ? C : act_value          (nn.Threshold applied to a convolution's output)
+    //   mask: C = mask[same offset as C] > mask_threshold ? C : 0
+    //         (nn.Threshold's backward applied to a convolution's gradInput; mask is laid out exactly like C)
+    bool act = false;
+    float act_threshold = 0.0f, act_value = 0.0f;
+    const float *mask = nullptr;
+    float mask_threshold = 0.0f;
     const char *tag = "gemm";     // name used by per-kernel timing
     // Flops the per-kernel timing credits the launch with; 0 means the product's own 2*M*J*R*nb.  A
     // convolution pass sets its algorithmic 2*M*N*K*B here, which a gathered gradInput product (one
@@ -83,6 +91,10 @@ struct GemmArgs {
     unsigned tilesM, tilesJ, total;
     FastDiv divN, divTilesM, divTilesJ, divSpi;
     float alpha, beta;
+    int act;  // see GemmProblem
+    float act_threshold, act_value;
+    const float *mask;
+    float mask_threshold;
 };
 
 // Workgroups are handed to the 8 XCDs round-robin by linear id.  Remap so that

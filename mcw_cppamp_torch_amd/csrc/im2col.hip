@@ -37,6 +37,7 @@
 #include <cstring>
 
 #include "common.h"
+#include "kernels.h"
 
 namespace thgpu {
 
@@ -352,7 +353,8 @@ __global__ __launch_bounds__(256) void im2col_tapvec_kernel(const float *__restr
 
 // One lane per image pixel; see the file comment for the order of additions.
 __global__ __launch_bounds__(256) void col2im_kernel(const float *__restrict__ col, float *__restrict__ im,
-                                                     const ConvGeom g, long total, int TH, int TW) {
+                                                     const ConvGeom g, long total, int TH, int TW,
+                                                     const InputMask mask) {
     long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     unsigned plane, pix, h, w;
@@ -390,6 +392,7 @@ __global__ __launch_bounds__(256) void col2im_kernel(const float *__restrict__ c
             for (int u = 0; u < 4; ++u) acc += ok[u] ? v[u] : 0.0f;
         }
     }
+    if (mask.in) acc = mask.in[idx] > mask.threshold ? acc : 0.0f;
     im[idx] = acc;
 }
 
@@ -442,7 +445,7 @@ __global__ __launch_bounds__(256) void im2col_unit_kernel(const float *__restric
 // kh ascending, kw ascending, out-of-range taps contributing +0.0f.
 template <int KH, int KW>
 __global__ __launch_bounds__(256) void col2im_unit_kernel(const float *__restrict__ col, float *__restrict__ im,
-                                                          const ConvGeom g, unsigned total) {
+                                                          const ConvGeom g, unsigned total, const InputMask mask) {
     const unsigned q0 = blockIdx.x * 256u;  // scalar
     const unsigned q = q0 + threadIdx.x;
     const unsigned plane_first = g.divHW.div(q0);
@@ -453,6 +456,8 @@ __global__ __launch_bounds__(256) void col2im_unit_kernel(const float *__restric
     const long plane_floats = (long)(KH * KW) * g.N;
     const unsigned voff = (unsigned)(((long)(plane - plane_first) * plane_floats + (long)hp * g.Wo + wp) * 4);
     const char *base = reinterpret_cast<const char *>(col + (long)plane_first * plane_floats);
+    float mv = 0.0f;
+    if (mask.in) mv = mask.in[q < total ? q : total - 1];  // requested together with the taps
     float v[KH][KW];
 #pragma unroll
     for (int kh = 0; kh < KH; ++kh) {
@@ -469,6 +474,7 @@ __global__ __launch_bounds__(256) void col2im_unit_kernel(const float *__restric
     for (int kh = 0; kh < KH; ++kh)
 #pragma unroll
         for (int kw = 0; kw < KW; ++kw) acc += v[kh][kw];
+    if (mask.in) acc = mv > mask.threshold ? acc : 0.0f;
     if (q < total) im[q] = acc;
 }
 
@@ -488,7 +494,8 @@ __global__ __launch_bounds__(256) void col2im_unit_kernel(const float *__restric
 template <int TH, int TW>
 __global__ __launch_bounds__(256) void col2im_strided_kernel(const float *__restrict__ col, float *__restrict__ im,
                                                              const ConvGeom g, int R, int Qw, int qtiles,
-                                                             const FastDiv divQw, const FastDiv divTiles) {
+                                                             const FastDiv divQw, const FastDiv divTiles,
+                                                             const InputMask mask) {
     extern __shared__ float rows[];  // [R*sH][W]
     unsigned plane, qt;
     divTiles.divmod(blockIdx.x, plane, qt);
@@ -533,7 +540,13 @@ __global__ __launch_bounds__(256) void col2im_strided_kernel(const float *__rest
     const int h_hi = h_base + R * g.sH < g.H ? h_base + R * g.sH : g.H;
     float *dst = im + ((long)plane * g.H + h_lo) * g.W;
     const float *from = rows + (h_lo - h_base) * g.W;
-    for (int i = threadIdx.x; i < (h_hi - h_lo) * g.W; i += blockDim.x) dst[i] = from[i];
+    if (mask.in) {
+        const float *m = mask.in + (dst - im);
+        for (int i = threadIdx.x; i < (h_hi - h_lo) * g.W; i += blockDim.x)
+            dst[i] = m[i] > mask.threshold ? from[i] : 0.0f;
+    } else {
+        for (int i = threadIdx.x; i < (h_hi - h_lo) * g.W; i += blockDim.x) dst[i] = from[i];
+    }
 }
 
 int make_geom(ConvGeom &g, long B, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW) {
@@ -703,7 +716,7 @@ long im2col_plan_selftest() {
 }
 
 int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW,
-                  float *im) {
+                  float *im, InputMask mask) {
     ConvGeom g;
     if (make_geom(g, B, C, H, W, kH, kW, pH, pW, sH, sW)) return 1;
     hipStream_t s = stream();
@@ -712,7 +725,7 @@ int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW,
     if (total == 0) return 0;
     const long blocks = (total + 255) / 256;
     if (blocks >= (1L << 31)) return fail("col2im: image batch too large for one launch");
-    const double bytes = 4.0 * ((double)total + (double)B * C * kH * kW * g.Ho * g.Wo);
+    const double bytes = 4.0 * ((mask.in ? 2.0 : 1.0) * (double)total + (double)B * C * kH * kW * g.Ho * g.Wo);
     // Lane offsets of the unit-stride kernel are 32-bit: the planes one workgroup can touch must span < 4 GiB.
     const long span_planes = 256 / ((long)H * W) + 2;
     // The col2im_generic switch forces the general kernel (a testing and tuning aid).
@@ -722,10 +735,10 @@ int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW,
             LaunchScope scope(geom_label("col2im", g, B), 0.0, bytes);
             if (kH == 3)
                 hipLaunchKernelGGL((col2im_unit_kernel<3, 3>), dim3((unsigned)blocks), dim3(256), 0, s, col, im, g,
-                                   (unsigned)total);
+                                   (unsigned)total, mask);
             else
                 hipLaunchKernelGGL((col2im_unit_kernel<5, 5>), dim3((unsigned)blocks), dim3(256), 0, s, col, im, g,
-                                   (unsigned)total);
+                                   (unsigned)total, mask);
         }
         return check_launch("col2im");
     }
@@ -747,10 +760,10 @@ int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW,
                 LaunchScope scope(geom_label("col2im", g, B), 0.0, bytes);
                 if (th == 3 || tw == 3)
                     hipLaunchKernelGGL((col2im_strided_kernel<3, 3>), grid, block, lds, s, col, im, g, R, Qw, qtiles,
-                                       FastDiv((uint32_t)Qw), FastDiv((uint32_t)qtiles));
+                                       FastDiv((uint32_t)Qw), FastDiv((uint32_t)qtiles), mask);
                 else
                     hipLaunchKernelGGL((col2im_strided_kernel<2, 2>), grid, block, lds, s, col, im, g, R, Qw, qtiles,
-                                       FastDiv((uint32_t)Qw), FastDiv((uint32_t)qtiles));
+                                       FastDiv((uint32_t)Qw), FastDiv((uint32_t)qtiles), mask);
             }
             return check_launch("col2im");
         }
@@ -758,7 +771,7 @@ int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW,
     {
         LaunchScope scope(geom_label("col2im", g, B), 0.0, bytes);
         hipLaunchKernelGGL(col2im_kernel, dim3((unsigned)blocks), dim3(256), 0, s, col, im, g, total,
-                           (kH + sH - 1) / sH, (kW + sW - 1) / sW);
+                           (kH + sH - 1) / sH, (kW + sW - 1) / sW, mask);
     }
     return check_launch("col2im");
 }
@@ -776,7 +789,7 @@ int thgpu_im2col(const float *im, long B, int C, int H, int W, int kH, int kW, i
 
 int thgpu_col2im(const float *col, long B, int C, int H, int W, int kH, int kW, int padH, int padW, int sH, int sW,
                  float *im) {
-    return col2im_launch(col, B, C, H, W, kH, kW, padH, padW, sH, sW, im);
+    return col2im_launch(col, B, C, H, W, kH, kW, padH, padW, sH, sW, im, InputMask());
 }
 
 }  // extern "C"

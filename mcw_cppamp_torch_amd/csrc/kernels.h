@@ -6,14 +6,21 @@
 
 namespace thgpu {
 
+// nn.Threshold's backward fused into the kernel that produces the gradient: an element of the result is kept
+// where `in` (same shape and layout as the result) exceeds `threshold` and zeroed elsewhere.  in == nullptr: off.
+struct InputMask {
+    const float *in = nullptr;
+    float threshold = 0.0f;
+};
+
 int im2col_launch(const float *im, long B, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW,
                   float *col);
 int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW,
-                  float *im);
+                  float *im, InputMask mask = InputMask());
 int maxpool_fwd_launch(const float *in, long planes, int H, int W, int kH, int kW, int dH, int dW, float *out,
                        float *indices);
 int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int H, int W, int Ho, int Wo, int kH,
-                       int kW, int dH, int dW, float *gin);
+                       int kW, int dH, int dW, float *gin, InputMask mask = InputMask());
 int threshold_fwd_launch(const float *in, float *out, long n, float th, float val);
 int threshold_bwd_launch(const float *in, const float *gout, float *gin, long n, float th);
 int gradbias_launch(const float *gout, float *gbias, long B, int M, long N, float scale);
@@ -29,12 +36,19 @@ bool conv_use_gathered(long B, int C, int H, int W, int M, int kH, int kW, int p
 bool conv_use_gathered_gradinput(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW);
 long conv_implicit_gradinput_scratch(long B, int C, int H, int W, int M, int kH, int kW);
 int pad_planes_launch(const float *in, long planes, int H, int W, int pH, int pW, float *out);
+// `act` applies nn.Threshold (threshold, value) to the output as it is stored; `mask` zeroes gradInput where the
+// convolution's input does not exceed a threshold (the backward of a Threshold in front of the convolution).
+struct OutputThreshold {
+    bool on = false;
+    float threshold = 0.0f, value = 0.0f;
+};
 int conv_implicit_forward(const float *padded, const float *weight, const float *bias, float *output, long B, int C,
-                          int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW);
+                          int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW,
+                          OutputThreshold act = OutputThreshold());
 int conv_implicit_gradweight(const float *padded, const float *gradOutput, float *gradWeight, long B, int C, int H,
                              int W, int M, int kH, int kW, int pH, int pW, int sH, int sW, float scale);
 int conv_implicit_gradinput(const float *gradOutput, const float *weight, float *scratch, float *gradInput, long B,
-                            int C, int H, int W, int M, int kH, int kW, int pH, int pW);
+                            int C, int H, int W, int M, int kH, int kW, int pH, int pW, InputMask mask = InputMask());
 
 // Host-only checks of the launch planners (no GPU needed); each returns the number of violations.
 long im2col_plan_selftest();

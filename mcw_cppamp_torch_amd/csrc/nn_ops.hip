@@ -87,13 +87,9 @@ int size_padded(THGPUTensor *t, const ConvShape &s, int padH, int padW) {
     return 0;
 }
 
-}  // namespace
-
-extern "C" {
-
-int thgpu_SpatialConvolutionMM_updateOutput(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias,
-                                            THGPUTensor *finput, THGPUTensor *fgradInput, THGPUTensor *output,
-                                            int kW, int kH, int dW, int dH, int padW, int padH) {
+int conv_update_output(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias, THGPUTensor *finput,
+                       THGPUTensor *fgradInput, THGPUTensor *output, int kW, int kH, int dW, int dH, int padW,
+                       int padH, OutputThreshold act) {
     (void)fgradInput;  // the reference uses it as a buffer of ones for the bias GEMM; the bias is fused here
     ConvShape s;
     if (conv_shape(s, input, weight, kW, kH, dW, dH, padW, padH)) return 1;
@@ -130,7 +126,7 @@ int thgpu_SpatialConvolutionMM_updateOutput(THGPUTensor *input, THGPUTensor *wei
         if (!rc) rc = pad_planes_launch(dptr(in), s.B * s.C, s.H, s.W, padH, padW, dptr(finput));
         if (!rc)
             rc = conv_implicit_forward(dptr(finput), dptr(weight), dptr(bias), dptr(output), s.B, s.C, s.H, s.W, s.M, kH,
-                                       kW, padH, padW, dH, dW);
+                                       kW, padH, padW, dH, dW, act);
         THGPUTensor_free(in);
         return rc;
     }
@@ -155,16 +151,19 @@ int thgpu_SpatialConvolutionMM_updateOutput(THGPUTensor *input, THGPUTensor *wei
         p.R = s.K;
         p.tag = "gemm_conv_fwd";
         p.flops = 2.0 * s.M * (double)s.N * s.K * s.B;
+        p.act = act.on;
+        p.act_threshold = act.threshold;
+        p.act_value = act.value;
         rc = gemm_launch(p);
     }
     THGPUTensor_free(in);
     return rc;
 }
 
-int thgpu_SpatialConvolutionMM_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *weight,
-                                               THGPUTensor *finput, THGPUTensor *fgradInput,
-                                               THGPUTensor *gradInput, int kW, int kH, int dW, int dH, int padW,
-                                               int padH) {
+// mask_on: gradInput is zeroed where `input` does not exceed mask_threshold.
+int conv_update_grad_input(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *weight, THGPUTensor *finput,
+                           THGPUTensor *fgradInput, THGPUTensor *gradInput, int kW, int kH, int dW, int dH,
+                           int padW, int padH, bool mask_on, float mask_threshold) {
     (void)finput;
     ConvShape s;
     if (conv_shape(s, input, weight, kW, kH, dW, dH, padW, padH)) return 1;
@@ -173,6 +172,25 @@ int thgpu_SpatialConvolutionMM_updateGradInput(THGPUTensor *input, THGPUTensor *
     if (require_contiguous(weight, "weight")) return 1;
     THGPUTensor *go = THGPUTensor_newContiguous(gradOutput);
     if (!go) return 1;
+    // The mask reads `input` element for element beside gradInput, so it needs the dense layout.
+    THGPUTensor *in = mask_on ? THGPUTensor_newContiguous(input) : nullptr;
+    if (mask_on && (!in || !tensor_backed(in))) {
+        if (in) THGPUTensor_free(in);
+        THGPUTensor_free(go);
+        return fail("SpatialConvolutionMM: input is not usable as a mask");
+    }
+    InputMask mask;
+    if (mask_on) {
+        mask.in = dptr(in);
+        mask.threshold = mask_threshold;
+    }
+    struct Release {  // frees the contiguous copies on every return path
+        THGPUTensor *a, *b;
+        ~Release() {
+            if (a) THGPUTensor_free(a);
+            if (b) THGPUTensor_free(b);
+        }
+    } release{go, in};
 
     if (conv_use_gathered_gradinput(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW)) {
         // fgradInput holds the padded gradOutput and the flipped kernels instead of the gradient columns
@@ -189,8 +207,7 @@ int thgpu_SpatialConvolutionMM_updateGradInput(THGPUTensor *input, THGPUTensor *
             rc = fail("SpatialConvolutionMM: a tensor's shape exceeds its storage");
         if (!rc)
             rc = conv_implicit_gradinput(dptr(go), dptr(weight), dptr(fgradInput), dptr(gradInput), s.B, s.C, s.H, s.W,
-                                         s.M, kH, kW, padH, padW);
-        THGPUTensor_free(go);
+                                         s.M, kH, kW, padH, padW, mask);
         return rc;
     }
     if (s.batched) {
@@ -227,9 +244,47 @@ int thgpu_SpatialConvolutionMM_updateGradInput(THGPUTensor *input, THGPUTensor *
         p.flops = 2.0 * s.M * (double)s.N * s.K * s.B;
         rc = gemm_launch(p);
     }
-    if (!rc) rc = col2im_launch(dptr(fgradInput), s.B, s.C, s.H, s.W, kH, kW, padH, padW, dH, dW, dptr(gradInput));
-    THGPUTensor_free(go);
+    if (!rc)
+        rc = col2im_launch(dptr(fgradInput), s.B, s.C, s.H, s.W, kH, kW, padH, padW, dH, dW, dptr(gradInput), mask);
     return rc;
+}
+
+}  // namespace
+
+extern "C" {
+
+int thgpu_SpatialConvolutionMM_updateOutput(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias,
+                                            THGPUTensor *finput, THGPUTensor *fgradInput, THGPUTensor *output,
+                                            int kW, int kH, int dW, int dH, int padW, int padH) {
+    return conv_update_output(input, weight, bias, finput, fgradInput, output, kW, kH, dW, dH, padW, padH,
+                              OutputThreshold());
+}
+
+int thgpu_SpatialConvolutionMM_updateOutputThreshold(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias,
+                                                     THGPUTensor *finput, THGPUTensor *fgradInput,
+                                                     THGPUTensor *output, int kW, int kH, int dW, int dH, int padW,
+                                                     int padH, float threshold, float val) {
+    OutputThreshold act;
+    act.on = true;
+    act.threshold = threshold;
+    act.value = val;
+    return conv_update_output(input, weight, bias, finput, fgradInput, output, kW, kH, dW, dH, padW, padH, act);
+}
+
+int thgpu_SpatialConvolutionMM_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *weight,
+                                               THGPUTensor *finput, THGPUTensor *fgradInput,
+                                               THGPUTensor *gradInput, int kW, int kH, int dW, int dH, int padW,
+                                               int padH) {
+    return conv_update_grad_input(input, gradOutput, weight, finput, fgradInput, gradInput, kW, kH, dW, dH, padW,
+                                  padH, false, 0.0f);
+}
+
+int thgpu_SpatialConvolutionMM_updateGradInputMasked(THGPUTensor *input, THGPUTensor *gradOutput,
+                                                     THGPUTensor *weight, THGPUTensor *finput,
+                                                     THGPUTensor *fgradInput, THGPUTensor *gradInput, int kW, int kH,
+                                                     int dW, int dH, int padW, int padH, float threshold) {
+    return conv_update_grad_input(input, gradOutput, weight, finput, fgradInput, gradInput, kW, kH, dW, dH, padW,
+                                  padH, true, threshold);
 }
 
 int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor *gradOutput,
@@ -340,8 +395,9 @@ int thgpu_SpatialMaxPooling_updateOutput(THGPUTensor *input, THGPUTensor *output
     return rc;
 }
 
-int thgpu_SpatialMaxPooling_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *gradInput,
-                                            THGPUTensor *indices, int kW, int kH, int dW, int dH) {
+static int pool_update_grad_input(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *gradInput,
+                                  THGPUTensor *indices, int kW, int kH, int dW, int dH, bool mask_on,
+                                  float mask_threshold) {
     if (!input || !gradOutput || !gradInput || !indices) return fail("SpatialMaxPooling: null tensor");
     if (!(input->nDimension == 3 || input->nDimension == 4)) return fail("3D or 4D (batch) tensor expected");
     if (kW <= 0 || kH <= 0 || dW <= 0 || dH <= 0) return fail("SpatialMaxPooling: invalid kernel/stride");
@@ -363,10 +419,31 @@ int thgpu_SpatialMaxPooling_updateGradInput(THGPUTensor *input, THGPUTensor *gra
     int rc = 0;
     if (!tensor_ready(gradInput, B * C * H * W) || !tensor_backed(go))
         rc = fail("SpatialMaxPooling: could not size gradInput");
+    THGPUTensor *in = (!rc && mask_on) ? THGPUTensor_newContiguous(input) : nullptr;
+    InputMask mask;
+    if (!rc && mask_on) {
+        if (!in || !tensor_backed(in)) rc = fail("SpatialMaxPooling: input is not usable as a mask");
+        else {
+            mask.in = dptr(in);
+            mask.threshold = mask_threshold;
+        }
+    }
     if (!rc)
-        rc = maxpool_bwd_launch(dptr(go), dptr(indices), B * C, H, W, Ho, Wo, kH, kW, dH, dW, dptr(gradInput));
+        rc = maxpool_bwd_launch(dptr(go), dptr(indices), B * C, H, W, Ho, Wo, kH, kW, dH, dW, dptr(gradInput), mask);
+    if (in) THGPUTensor_free(in);
     THGPUTensor_free(go);
     return rc;
+}
+
+int thgpu_SpatialMaxPooling_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *gradInput,
+                                            THGPUTensor *indices, int kW, int kH, int dW, int dH) {
+    return pool_update_grad_input(input, gradOutput, gradInput, indices, kW, kH, dW, dH, false, 0.0f);
+}
+
+int thgpu_SpatialMaxPooling_updateGradInputMasked(THGPUTensor *input, THGPUTensor *gradOutput,
+                                                  THGPUTensor *gradInput, THGPUTensor *indices, int kW, int kH,
+                                                  int dW, int dH, float threshold) {
+    return pool_update_grad_input(input, gradOutput, gradInput, indices, kW, kH, dW, dH, true, threshold);
 }
 
 int thgpu_Threshold_updateOutput(THGPUTensor *input, THGPUTensor *output, float threshold, float val) {

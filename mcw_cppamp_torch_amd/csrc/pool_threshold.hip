@@ -1,26 +1,30 @@
 // nn.SpatialMaxPooling and nn.Threshold kernels.
 //
-// Max-pool forward: one lane per output element, lanes along the output row;
-// the window is scanned ky ascending, kx ascending with a strict '>' from -inf,
-// so the first maximum wins ties exactly as the CPU module's scan does
-// (mcw_nn/generic/SpatialMaxPooling.c:30-45).  The two index planes hold
-// ky+1 and kx+1 as floats (:51-52).
+// Max-pool forward, wavefront-level formulation (maxpool_fwd_tile_kernel; the default is the direct kernel, see
+// there): a workgroup stages a group of small planes (or a strip of rows of a large one) in
+// LDS with one contiguous, coalesced read -- every input row leaves memory once -- and its wavefronts
+// then take output rows one at a time with their lanes along the INPUT columns: a lane reduces its
+// column over the window rows (ky ascending, strict '>' from -inf, so the smallest ky wins a tie), and
+// output lane j combines the kW columns j*dW + kx through cross-lane reads, keeping the larger value
+// and, between equal values, the smaller (ky, kx) pair.  That is the first maximum of the CPU module's
+// row-major strict-'>' scan (mcw_nn/generic/SpatialMaxPooling.c:30-45).  Planes narrower than half a
+// wavefront are packed side by side.  The two index planes hold ky+1 and kx+1 as floats (:51-52).
 //
-// Max-pool backward is index driven and atomics-free: every input pixel visits
-// the windows that cover it in (i ascending, j ascending) order and adds
-// gradOutput where the saved argmax points back at the pixel.  This is the
-// float addition order of the CPU module's scatter (:165-174), so overlapping
-// windows give bit-identical sums, and no zero-fill pass is needed.  It
-// replaces gpunn-impl/SpatialMaxPooling.cpp:87-203, which only handled
-// non-overlapping windows.  A workgroup takes a strip of pixel rows of one
-// plane (or several small planes), turns the windows that can reach it into
-// (target pixel, gradient) pairs in LDS -- padded with pairs that target no
-// pixel, so the pixel loop has no bounds to check -- and then each pixel
-// compares at most ceil(kH/dH)*ceil(kW/dW) pairs against its own index.
+// Max-pool backward is an index-driven scatter without atomics and without a zero-fill pass over
+// memory: a workgroup owns the pixels of a group of planes (or a strip of rows) as a zeroed LDS tile,
+// reads the windows that can reach them once (contiguous reads of the three window arrays), and adds
+// each gradient at the pixel its saved argmax names.  The adds happen in ceil(kH/dH)*ceil(kW/dW)
+// phases: a window whose argmax is pixel (h, w) belongs to phase (h/dH - i, w/dW - j), phases run with
+// both differences descending, and inside one phase no two windows name the same pixel -- so every
+// pixel receives its gradients in (i ascending, j ascending) order, the float addition order of the
+// CPU module's scatter (:165-174), and overlapping windows give bit-identical sums.  It replaces
+// gpunn-impl/SpatialMaxPooling.cpp:87-203, which only handled non-overlapping windows.  The tile is
+// written out as one contiguous stream; the backward of a Threshold in front of the pooling layer can
+// be applied on the way (InputMask).
 #include "common.h"
+#include "kernels.h"
 
 #include <cmath>
-#include <cstdlib>
 
 namespace thgpu {
 
@@ -37,12 +41,18 @@ inline const char *pool_label(const char *family, const PoolGeom &g, long planes
     return prof_label("%s planes=%ld %dx%d k=%dx%d s=%dx%d", family, planes, g.H, g.W, g.kH, g.kW, g.dH, g.dW);
 }
 
-// KH, KW > 0 fix the window at compile time (fully unrolled: all loads of a
-// window are in flight before the compare chain); 0 takes the run-time sizes.
+// ---- forward ---------------------------------------------------------------------------------------
+
+// The direct kernel: one lane per output element, lanes along the output row, scanning its own window in
+// global memory (neighbouring lanes share the rows through the vector cache).  KH, KW > 0 fix the window at
+// compile time (fully unrolled: all loads of a window are in flight before the compare chain); 0 takes the
+// run-time sizes.  Measured on gfx950 this is the fastest forward kernel on every geometry of the benchmark
+// stacks (at 13x13 .. 55x55 planes a launch lasts 10-35 us and is bound by its ramp-up, not by traffic), so it
+// is the default; the tile kernel below is the wavefront-level formulation, kept behind the pool_fwd_wave switch.
 template <int KH, int KW>
-__global__ __launch_bounds__(256) void maxpool_fwd_kernel(const float *__restrict__ in, float *__restrict__ out,
-                                                          float *__restrict__ indy, float *__restrict__ indx,
-                                                          const PoolGeom g, unsigned total) {
+__global__ __launch_bounds__(256) void maxpool_fwd_direct_kernel(const float *__restrict__ in, float *__restrict__ out,
+                                                                 float *__restrict__ indy, float *__restrict__ indx,
+                                                                 const PoolGeom g, unsigned total) {
     unsigned o = blockIdx.x * blockDim.x + threadIdx.x;
     if (o >= total) return;
     unsigned plane, rem, i, j;
@@ -85,167 +95,353 @@ __global__ __launch_bounds__(256) void maxpool_fwd_kernel(const float *__restric
     indx[o] = by < 0 ? 0.0f : (float)(bx + 1);
 }
 
-// Launch shape of the LDS-tile backward kernel.
+// Launch shape of the forward tile kernel.
+struct PoolFwdPlan {
+    int G;       // planes per workgroup (more than one only when a strip is the whole plane)
+    int SR;      // output rows per strip
+    int strips;  // strips per plane
+    int P;       // planes (or row items) a wavefront takes side by side: 64 / W when the row fits twice
+    int CO;      // outputs per column chunk: a wavefront covers (CO-1)*dW + kW input columns
+    int chunks;  // column chunks per output row
+    FastDiv divStrips, divItemRows, divChunks, divLaneW;
+};
+
+// The wavefront-level argmax described at the top of the file.  KH, KW, DH, DW > 0 fix the window at compile time;
+// 0 takes the run-time values.
+template <int KH, int KW, int DH, int DW>
+__global__ __launch_bounds__(256) void maxpool_fwd_tile_kernel(const float *__restrict__ in, float *__restrict__ out,
+                                                               float *__restrict__ indy, float *__restrict__ indx,
+                                                               const PoolGeom g, const PoolFwdPlan p, unsigned planes) {
+    extern __shared__ float tile[];  // [np][nh][W]: the staged input rows, then [3][np][ni][Wo]: the results
+    const int kH = KH > 0 ? KH : g.kH, kW = KW > 0 ? KW : g.kW, dH = DH > 0 ? DH : g.dH, dW = DW > 0 ? DW : g.dW;
+    const int tid = threadIdx.x;
+    unsigned grp, strip;
+    p.divStrips.divmod(blockIdx.x, grp, strip);
+    const unsigned plane0 = grp * (unsigned)p.G;
+    const int np = (int)(planes - plane0 < (unsigned)p.G ? planes - plane0 : (unsigned)p.G);
+    const int i0 = (int)strip * p.SR;
+    const int ni = g.Ho - i0 < p.SR ? g.Ho - i0 : p.SR;  // output rows of this strip
+    const int h0 = i0 * dH;
+    const int nh = p.G > 1 ? g.H : (ni - 1) * dH + kH;   // grouped planes are staged whole
+    const int rows_w = nh * g.W;
+    // results of the strip: values, ky+1, kx+1, each [np][ni][Wo], behind the staged rows
+    const int nout = np * ni * g.Wo;
+    float *res = tile + ((p.G * (p.G > 1 ? g.H : (p.SR - 1) * dH + kH) * g.W + 3) & ~3);
+
+    // ---- stage: one contiguous range (grouped planes lie back to back; a strip is a run of whole rows) ----
+    {
+        const float *src = in + (long)plane0 * g.H * g.W + (p.G > 1 ? 0 : (long)h0 * g.W);
+        const int n = np * rows_w;
+        // 128-bit reads from the first 16-byte boundary on; single floats before it and at the end
+        const int head = (int)(((16u - (unsigned)(reinterpret_cast<uintptr_t>(src) & 15u)) & 15u) >> 2);
+        const int lead = head < n ? head : n;
+        if (tid < lead) tile[tid] = src[tid];
+        const int nv = (n - lead) >> 2;
+        const float4 *src4 = reinterpret_cast<const float4 *>(src + lead);
+        for (int q0 = tid; q0 < nv; q0 += 4 * 256) {
+            float4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (q0 + u * 256 < nv) v[u] = src4[q0 + u * 256];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (q0 + u * 256 < nv) {
+                    const int e = lead + 4 * (q0 + u * 256);
+                    tile[e] = v[u].x;
+                    tile[e + 1] = v[u].y;
+                    tile[e + 2] = v[u].z;
+                    tile[e + 3] = v[u].w;
+                }
+        }
+        const int done = lead + 4 * nv;
+        if (tid < n - done) tile[done + tid] = src[done + tid];
+    }
+    __syncthreads();
+
+    // ---- wavefronts take (plane, output row, column chunk) items, P of them side by side ----------------------
+    const int lane = tid & 63, wave = tid >> 6;
+    unsigned sub, c;
+    p.divLaneW.divmod((unsigned)lane, sub, c);  // lane -> (which of the P items, input column inside the chunk)
+    const int span = (p.CO - 1) * dW + kW;      // input columns a chunk covers
+    const int items = np * ni * p.chunks;
+    for (int it0 = wave * p.P; it0 < items; it0 += 4 * p.P) {
+        const int it = it0 + (int)sub;
+        const bool live = (int)sub < p.P && it < items;
+        unsigned rowitem, chunk = 0, pl, il;
+        if (p.chunks > 1)
+            p.divChunks.divmod((unsigned)(live ? it : 0), rowitem, chunk);
+        else
+            rowitem = (unsigned)(live ? it : 0);
+        p.divItemRows.divmod(rowitem, pl, il);  // il: output row inside the strip
+        const int j0 = (int)chunk * p.CO;
+        const int col = j0 * dW + (int)c;       // the lane's input column
+        // column reduce over the window rows: smallest ky wins ties
+        float cv = -INFINITY;
+        int cky = -1;
+        if (live && (int)c < span && col < g.W) {
+            const float *colp = tile + (int)pl * rows_w + ((int)il * dH) * g.W + col;  // the tile starts at row i0*dH
+#pragma unroll
+            for (int ky = 0; ky < (KH > 0 ? KH : 8); ++ky) {
+                if (KH == 0 && ky >= kH) break;
+                const float v = colp[ky * g.W];
+                if (v > cv) {
+                    cv = v;
+                    cky = ky;
+                }
+            }
+            if (KH == 0)
+                for (int ky = 8; ky < kH; ++ky) {
+                    const float v = colp[ky * g.W];
+                    if (v > cv) {
+                        cv = v;
+                        cky = ky;
+                    }
+                }
+        }
+        // combine the kW columns of each output across lanes: larger value, then the smaller (ky, kx)
+        float best = -INFINITY;
+        int bky = -1, bkx = 0;
+        const int lane_base = lane - (int)c;  // first lane of this lane's item
+#pragma unroll
+        for (int kx = 0; kx < (KW > 0 ? KW : 8); ++kx) {
+            if (KW == 0 && kx >= kW) break;
+            int srcl = lane_base + (int)c * dW + kx;
+            srcl = srcl < 64 ? srcl : 63;       // lanes that are no output lanes read anything: discarded below
+            const float v = __shfl(cv, srcl, 64);
+            const int vy = __shfl(cky, srcl, 64);
+            if (v > best || (v == best && vy >= 0 && (bky < 0 || vy < bky))) {
+                best = v;
+                bky = vy;
+                bkx = kx;
+            }
+        }
+        if (KW == 0)
+            for (int kx = 8; kx < kW; ++kx) {
+                int srcl = lane_base + (int)c * dW + kx;
+                srcl = srcl < 64 ? srcl : 63;
+                const float v = __shfl(cv, srcl, 64);
+                const int vy = __shfl(cky, srcl, 64);
+                if (v > best || (v == best && vy >= 0 && (bky < 0 || vy < bky))) {
+                    best = v;
+                    bky = vy;
+                    bkx = kx;
+                }
+            }
+        const int j = j0 + (int)c;
+        if (live && (int)c < p.CO && j < g.Wo) {
+            const int o = ((int)pl * ni + (int)il) * g.Wo + j;
+            res[o] = best;
+            // a window that never updated the maximum (all NaN or -inf): the CPU code stores (1, 0)
+            res[nout + o] = bky < 0 ? 1.0f : (float)(bky + 1);
+            res[2 * nout + o] = bky < 0 ? 0.0f : (float)(bkx + 1);
+        }
+    }
+    __syncthreads();
+    // ---- the three result arrays leave as contiguous streams (grouped planes lie back to back; a strip is a run
+    // of whole output rows) ------------------------------------------------------------------------------------
+    const long obase = (long)plane0 * g.Ho * g.Wo + (p.G > 1 ? 0 : (long)i0 * g.Wo);
+    float *const dsts[3] = {out + obase, indy + obase, indx + obase};
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        float *dst = dsts[a];
+        const float *src = res + a * nout;
+        for (int e = tid; e < nout; e += 256) dst[e] = src[e];
+    }
+}
+
+constexpr long kPoolLdsBytes = 32 * 1024;  // the most LDS a pooling tile may ask for
+
+// Shape of the forward tile kernel; false when a window is wider than a wavefront or one strip row does not fit LDS.
+bool plan_pool_fwd(const PoolGeom &g, long planes, PoolFwdPlan &p) {
+    if (g.kW > 64 || g.kH > 64) return false;
+    const long plane_floats = (long)g.H * g.W;
+    auto strip_floats = [&](long SR) { return ((SR - 1) * g.dH + g.kH) * (long)g.W; };
+    if (strip_floats(1) * 4 > kPoolLdsBytes) return false;
+    const long want = 4096;  // floats per workgroup
+    p.G = 1;
+    if (plane_floats <= want / 2 && plane_floats * 4 <= kPoolLdsBytes) {
+        p.SR = g.Ho;
+        long G = want / plane_floats;
+        if (G > planes) G = planes;
+        while (G > 1 && G * plane_floats * 4 > kPoolLdsBytes) --G;
+        p.G = (int)(G < 1 ? 1 : G);
+    } else {
+        long SR = g.Ho;
+        while (SR > 1 && (strip_floats(SR) > want || strip_floats(SR) * 4 > kPoolLdsBytes)) --SR;
+        const long strips = (g.Ho + SR - 1) / SR;
+        p.SR = (int)((g.Ho + strips - 1) / strips);  // even strips
+    }
+    if (p.G == 1 && strip_floats(p.SR) * 4 > kPoolLdsBytes) return false;
+    p.strips = (g.Ho + p.SR - 1) / p.SR;
+    // staged rows plus three result arrays
+    if (((long)p.G * (p.G > 1 ? g.H : (p.SR - 1) * g.dH + g.kH) * g.W + 4 + 3L * p.G * p.SR * g.Wo) * 4 > 2 * kPoolLdsBytes)
+        return false;
+    // column chunks: a wavefront's 64 lanes cover (CO-1)*dW + kW input columns
+    if (g.W <= 64) {
+        p.CO = g.Wo;
+        p.chunks = 1;
+        p.P = 64 / g.W;
+    } else {
+        p.CO = (64 - g.kW) / g.dW + 1;
+        p.chunks = (g.Wo + p.CO - 1) / p.CO;
+        p.P = 1;
+    }
+    if (p.P < 1) p.P = 1;
+    p.divStrips = FastDiv((uint32_t)p.strips);
+    p.divItemRows = FastDiv((uint32_t)(p.G > 1 ? g.Ho : p.SR));
+    p.divChunks = FastDiv((uint32_t)p.chunks);
+    p.divLaneW = FastDiv((uint32_t)(p.P > 1 ? g.W : 64));
+    return true;
+}
+
+// ---- backward ----------------------------------------------------------------------------------------
+
+// Launch shape of the backward tile kernel.
 struct PoolBwdPlan {
     int G;      // planes per workgroup (more than one only when a strip is the whole plane)
     int PR;     // pixel rows per strip
     int tiles;  // strips per plane
-    int RW;     // window rows kept per strip (with TH-1 rows of history)
-    int CW;     // window columns kept per row (with TW-1 columns of history and the uncovered right edge)
-    FastDiv divTiles, divEnt, divCW, divPix;
-    FastDiv divW2, divPix2;  // pixel pairs (dW == 2): pairs per row, pairs per plane
+    FastDiv divTiles, divWo;
 };
 
-// TH x TW = the most windows that can cover one pixel.  Pixel (h, w) can only
-// be the argmax of windows (i_hi - a, j_hi - b), i_hi = h / dH, j_hi = w / dW,
-// a < TH, b < TW; visiting a and b downwards is (i ascending, j ascending).
-// PAIRS (horizontal stride 2): a lane takes the two pixels (h, 2k) and (h, 2k+1), which share j_hi = k and
-// with it all their candidate windows, so each staged pair is read once for both.
-template <int TH, int TW, bool PAIRS>
+constexpr int kPoolBwdWindowsPerLane = 4;  // windows a lane keeps in registers: a workgroup takes up to 1024
+constexpr int kPoolBwdPixelsPerLane = 16;  // pixels a lane writes (and mask values it holds): up to 4096 a workgroup
+
 __global__ __launch_bounds__(256) void maxpool_bwd_tile_kernel(const float *__restrict__ gout,
                                                                const float *__restrict__ indy,
                                                                const float *__restrict__ indx,
                                                                float *__restrict__ gin, const PoolGeom g,
-                                                               const PoolBwdPlan p, unsigned planes) {
-    extern __shared__ int2 ent[];  // [G][RW][CW]: (target pixel inside the plane or -1, gradient bits)
-    const int tid = threadIdx.x, nthr = blockDim.x;
+                                                               const PoolBwdPlan p, unsigned planes, int TH, int TW,
+                                                               const InputMask mask) {
+    extern __shared__ float px[];  // [np][nh][W]: the strip's gradInput
+    constexpr int U = kPoolBwdWindowsPerLane;
+    const int tid = threadIdx.x;
     unsigned grp, strip;
     p.divTiles.divmod(blockIdx.x, grp, strip);
     const unsigned plane0 = grp * (unsigned)p.G;
     const int np = (int)(planes - plane0 < (unsigned)p.G ? planes - plane0 : (unsigned)p.G);
     const int h0 = (int)strip * p.PR;
     const int nh = g.H - h0 < p.PR ? g.H - h0 : p.PR;
-    const int i_first = (int)g.divDH.div((unsigned)h0) - (TH - 1);
-    const int per_plane = p.RW * p.CW;
-    const int HoWo = g.Ho * g.Wo;
+    const int npix = np * nh * g.W;
+    // window rows that can reach pixel rows [h0, h0 + nh): i*dH + kH - 1 >= h0 and i*dH <= h0 + nh - 1
+    const int t0 = h0 - g.kH + g.dH;  // numerator of the ceiling
+    const int i_first = t0 <= 0 ? 0 : (int)g.divDH.div((unsigned)t0);
+    int i_last = (int)g.divDH.div((unsigned)(h0 + nh - 1));
+    if (i_last > g.Ho - 1) i_last = g.Ho - 1;
+    const int ni = i_last - i_first + 1;  // may be <= 0: rows no window reaches stay zero
+    const int per_plane = ni > 0 ? ni * g.Wo : 0;
+    const int nwin = np * per_plane;
 
-    // ---- windows -> (target, gradient) pairs ------------------------------------------------
-    const int E = np * per_plane;
-    for (int e0 = tid; e0 < E; e0 += 4 * nthr) {
-        float vy[4], vx[4], vg[4];
-        int wi[4], wj[4];
-        bool ok[4];
+    // ---- the mask values of the strip's pixels are requested first and used last ------------------------------
+    constexpr int PX = kPoolBwdPixelsPerLane;
+    const long base = (long)plane0 * g.H * g.W + (p.G > 1 ? 0 : (long)h0 * g.W);
+    float mv[PX];
+    if (mask.in) {
+        const float *m = mask.in + base;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int idx = e0 + u * nthr;
-            unsigned pl, rem, rr, cc;
-            p.divEnt.divmod((unsigned)(idx < E ? idx : 0), pl, rem);
-            p.divCW.divmod(rem, rr, cc);
-            wi[u] = i_first + (int)rr;
-            wj[u] = (int)cc - (TW - 1);
-            ok[u] = idx < E && wi[u] >= 0 && wi[u] < g.Ho && wj[u] >= 0 && wj[u] < g.Wo;
-            const long o = (long)(plane0 + pl) * HoWo + (ok[u] ? wi[u] * g.Wo + wj[u] : 0);
-            vy[u] = indy[o];
-            vx[u] = indx[o];
-            vg[u] = gout[o];
+        for (int u = 0; u < PX; ++u) {
+            const int e = tid + u * 256;
+            mv[u] = e < npix ? m[e] : 0.0f;
         }
+    }
+
+    // ---- the windows: three contiguous reads, all in flight before the tile is touched -----------------------
+    float wg[U];
+    int wt[U], wphase[U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int idx = e0 + u * nthr;
-            if (idx < E) {
-                const int t = (wi[u] * g.dH + (int)vy[u] - 1) * g.W + wj[u] * g.dW + (int)vx[u] - 1;
-                ent[idx] = make_int2(ok[u] ? t : -1, __float_as_int(vg[u]));
+    for (int u = 0; u < U; ++u) {
+        const int e = tid + u * 256;
+        wphase[u] = -1;
+        wt[u] = 0;
+        wg[u] = 0.0f;
+        if (e < nwin) {
+            unsigned pl = 0, rem = (unsigned)e, il, j;
+            if (p.G > 1) g.divHoWo.divmod((unsigned)e, pl, rem);  // grouped planes are whole: Ho*Wo windows each
+            p.divWo.divmod(rem, il, j);
+            const int i = i_first + (int)il;
+            const long o = ((long)(plane0 + pl) * g.Ho + i) * g.Wo + j;
+            const float fy = indy[o], fx = indx[o];
+            wg[u] = gout[o];
+            const int y = (int)fy - 1, x = (int)fx - 1;
+            const int h = i * g.dH + y, w = (int)j * g.dW + x;
+            // the argmax lies inside the window by construction; anything else (the (1, 0) a window of NaNs
+            // stores) names no pixel and is skipped
+            if (y >= 0 && y < g.kH && x >= 0 && x < g.kW && h >= h0 && h < h0 + nh && w < g.W) {
+                const int a = (int)g.divDH.div((unsigned)y), b = (int)g.divDW.div((unsigned)x);  // h/dH - i, w/dW - j
+                wphase[u] = (TH - 1 - a) * TW + (TW - 1 - b);  // both differences descending
+                wt[u] = ((int)pl * nh + (h - h0)) * g.W + w;
             }
         }
     }
+    for (int e = tid; e < npix; e += 256) px[e] = 0.0f;
     __syncthreads();
 
-    // ---- pixels ----------------------------------------------------------------------------------
-    if (PAIRS) {
-        const int W2 = (g.W + 1) / 2;
-        const int P2 = nh * W2;
-        const int total2 = np * P2;
-        for (int q = tid; q < total2; q += nthr) {
-            unsigned pl = 0, r = (unsigned)q, hh, w2;
-            if (p.G > 1) p.divPix2.divmod(r, pl, r);  // grouped planes are whole: P2 == H*W2
-            p.divW2.divmod(r, hh, w2);
-            const int h = h0 + (int)hh, w = 2 * (int)w2;
-            const int i_hi = (int)g.divDH.div((unsigned)h), j_hi = (int)w2;
-            const int2 *e = ent + (int)pl * per_plane + (i_hi - i_first) * p.CW + j_hi + (TW - 1);
-            const int pix = h * g.W + w;
-            float acc0 = 0.0f, acc1 = 0.0f;
+    // ---- scatter, phase by phase: inside one phase no two windows share a pixel ------------------------------
+    const int nphase = TH * TW;
+    for (int ph = 0; ph < nphase; ++ph) {
 #pragma unroll
-            for (int a = TH - 1; a >= 0; --a)
-#pragma unroll
-                for (int b = TW - 1; b >= 0; --b) {
-                    const int2 c = e[-a * p.CW - b];
-                    acc0 += c.x == pix ? __int_as_float(c.y) : 0.0f;
-                    acc1 += c.x == pix + 1 ? __int_as_float(c.y) : 0.0f;
-                }
-            float *out = gin + (long)(plane0 + pl) * g.H * g.W + pix;
-            out[0] = acc0;
-            if (w + 1 < g.W) out[1] = acc1;
-        }
-        return;
+        for (int u = 0; u < U; ++u)
+            if (wphase[u] == ph) px[wt[u]] += wg[u];
+        __syncthreads();
     }
-    const int P = nh * g.W;
-    const int total = np * P;
-    for (int q = tid; q < total; q += nthr) {
-        unsigned pl = 0, r = (unsigned)q, hh, w;
-        if (p.G > 1) p.divPix.divmod(r, pl, r);  // grouped planes are whole: P == H*W
-        g.divW.divmod(r, hh, w);
-        const int h = h0 + (int)hh;
-        const int i_hi = (int)g.divDH.div((unsigned)h), j_hi = (int)g.divDW.div(w);
-        const int2 *e = ent + (int)pl * per_plane + (i_hi - i_first) * p.CW + j_hi + (TW - 1);
-        const int pix = h * g.W + (int)w;
-        float acc = 0.0f;
+
+    // ---- the tile leaves as one contiguous stream --------------------------------------------------------------
+    float *dst = gin + base;
+    if (mask.in) {
 #pragma unroll
-        for (int a = TH - 1; a >= 0; --a)
+        for (int u = 0; u < PX; ++u) {
+            const int e = tid + u * 256;
+            if (e < npix) dst[e] = mv[u] > mask.threshold ? px[e] : 0.0f;
+        }
+    } else {
 #pragma unroll
-            for (int b = TW - 1; b >= 0; --b) {
-                const int2 c = e[-a * p.CW - b];
-                acc += c.x == pix ? __int_as_float(c.y) : 0.0f;
-            }
-        gin[(long)(plane0 + pl) * g.H * g.W + pix] = acc;
+        for (int u = 0; u < PX; ++u) {
+            const int e = tid + u * 256;
+            if (e < npix) dst[e] = px[e];
+        }
     }
 }
 
-// The most LDS the tile kernel may ask for.
-constexpr long kPoolBwdLdsBytes = 32 * 1024;
-
-// Strip shape of the tile kernel; false when one pixel row's windows do not fit in LDS.
-bool plan_pool_bwd(const PoolGeom &g, long planes, int TH, int TW, PoolBwdPlan &p) {
-    const int right = (g.W - 1) / g.dW - (g.Wo - 1);
-    p.CW = g.Wo + (TW - 1) + (right > 0 ? right : 0);
-    auto rows = [&](long PR) { return (PR + g.dH - 1) / g.dH + TH; };
-    auto bytes = [&](long G, long PR) { return G * rows(PR) * (long)p.CW * 8; };
-    if (bytes(1, 1) > kPoolBwdLdsBytes) return false;
-    const long want = 2048;  // pixels per workgroup
+// Strip shape of the backward tile kernel; false when one pixel row with its windows does not fit.
+bool plan_pool_bwd(const PoolGeom &g, long planes, int TH, PoolBwdPlan &p) {
+    const long max_win = 256L * kPoolBwdWindowsPerLane;
+    auto win_rows = [&](long PR) { return (PR + g.dH - 1) / g.dH + TH; };  // an upper bound
+    const long max_pix = 256L * kPoolBwdPixelsPerLane;
+    auto fits = [&](long G, long PR) {
+        return G * PR * (long)g.W <= max_pix && G * win_rows(PR) * (long)g.Wo <= max_win;
+    };
+    if (!fits(1, 1)) return false;
+    const long want = 4096;  // pixels per workgroup
     p.G = 1;
-    if ((long)g.H * g.W <= want / 2 && bytes(1, g.H) <= kPoolBwdLdsBytes) {
+    if (fits(1, g.H)) {
         p.PR = g.H;
+        // whole planes: the window count is exact, Ho*Wo per plane
         long G = want / ((long)g.H * g.W);
         if (G > planes) G = planes;
-        while (G > 1 && bytes(G, p.PR) > kPoolBwdLdsBytes) --G;
-        p.G = (int)(G < 1 ? 1 : G);
+        if (G < 1) G = 1;
+        while (G > 1 && (G * (long)g.H * g.W > max_pix || G * (long)g.Ho * g.Wo > max_win)) --G;
+        p.G = (int)G;
     } else {
         long PR = want / g.W;
         if (PR < 1) PR = 1;
         if (PR > g.H) PR = g.H;
-        while (PR > 1 && bytes(1, PR) > kPoolBwdLdsBytes) --PR;
+        while (PR > 1 && !fits(1, PR)) --PR;
         const long tiles = (g.H + PR - 1) / PR;
         p.PR = (int)((g.H + tiles - 1) / tiles);
     }
     p.tiles = (g.H + p.PR - 1) / p.PR;
-    p.RW = (int)rows(p.PR);
     p.divTiles = FastDiv((uint32_t)p.tiles);
-    p.divEnt = FastDiv((uint32_t)(p.RW * p.CW));
-    p.divCW = FastDiv((uint32_t)p.CW);
-    p.divPix = FastDiv((uint32_t)(g.H * g.W));
-    p.divW2 = FastDiv((uint32_t)((g.W + 1) / 2));
-    p.divPix2 = FastDiv((uint32_t)(g.H * ((g.W + 1) / 2)));
+    p.divWo = FastDiv((uint32_t)(g.Wo > 0 ? g.Wo : 1));
     return true;
 }
 
-// The direct kernel, for windows the tile kernel is not built for.
-// TH x TW = the most windows that can cover one pixel (ceil(kH/dH) x ceil(kW/dW));
-// candidates outside [lo, hi] are read at a clamped address and contribute +0.0f,
-// so the loads of all candidates are in flight together.
-template <int TH, int TW>
-__global__ __launch_bounds__(256) void maxpool_bwd_kernel(const float *__restrict__ gout,
-                                                          const float *__restrict__ indy,
-                                                          const float *__restrict__ indx, float *__restrict__ gin,
-                                                          const PoolGeom g, unsigned total, int th_rt, int tw_rt) {
+// The direct kernel, for geometries the tile kernel's plan does not take.  Every pixel visits the windows
+// covering it in (i ascending, j ascending) order.
+__global__ __launch_bounds__(256) void maxpool_bwd_direct_kernel(const float *__restrict__ gout,
+                                                                 const float *__restrict__ indy,
+                                                                 const float *__restrict__ indx,
+                                                                 float *__restrict__ gin, const PoolGeom g,
+                                                                 unsigned total, const InputMask mask) {
     unsigned p = blockIdx.x * blockDim.x + threadIdx.x;
     if (p >= total) return;
     unsigned plane, rem, h, w;
@@ -264,40 +460,15 @@ __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const float *__restric
     const float *iy = indy + (long)plane * g.Ho * g.Wo;
     const float *ix = indx + (long)plane * g.Ho * g.Wo;
     float acc = 0.0f;
-    if (TH > 0) {
-        float vy[TH > 0 ? TH : 1][TW > 0 ? TW : 1], vx[TH > 0 ? TH : 1][TW > 0 ? TW : 1],
-            vg[TH > 0 ? TH : 1][TW > 0 ? TW : 1];
-#pragma unroll
-        for (int a = 0; a < TH; ++a)
-#pragma unroll
-            for (int b = 0; b < TW; ++b) {
-                const int i = i_lo + a, j = j_lo + b;
-                const int o = (i <= i_hi && j <= j_hi) ? i * g.Wo + j : 0;
-                vy[a][b] = iy[o];
-                vx[a][b] = ix[o];
-                vg[a][b] = go[o];
-            }
-#pragma unroll
-        for (int a = 0; a < TH; ++a)
-#pragma unroll
-            for (int b = 0; b < TW; ++b) {
-                const int i = i_lo + a, j = j_lo + b;
-                const float wy = (float)((int)h - i * g.dH + 1), wx = (float)((int)w - j * g.dW + 1);
-                const bool hit = i <= i_hi && j <= j_hi && vy[a][b] == wy && vx[a][b] == wx;
-                acc += hit ? vg[a][b] : 0.0f;
-            }
-    } else {
-        (void)th_rt;
-        (void)tw_rt;
-        for (int i = i_lo; i <= i_hi; ++i) {
-            const float wy = (float)((int)h - i * g.dH + 1);  // 1-based ky that would hit this row
-            for (int j = j_lo; j <= j_hi; ++j) {
-                const int o = i * g.Wo + j;
-                const float wx = (float)((int)w - j * g.dW + 1);
-                if (iy[o] == wy && ix[o] == wx) acc += go[o];
-            }
+    for (int i = i_lo; i <= i_hi; ++i) {
+        const float wy = (float)((int)h - i * g.dH + 1);  // 1-based ky that would hit this row
+        for (int j = j_lo; j <= j_hi; ++j) {
+            const int o = i * g.Wo + j;
+            const float wx = (float)((int)w - j * g.dW + 1);
+            if (iy[o] == wy && ix[o] == wx) acc += go[o];
         }
     }
+    if (mask.in) acc = mask.in[p] > mask.threshold ? acc : 0.0f;
     gin[p] = acc;
 }
 
@@ -350,28 +521,44 @@ __global__ __launch_bounds__(256) void threshold_bwd_scalar(const float *__restr
 // in two fixed-shape stages so that reruns are bit-identical: stage 1 sums a
 // slice of the batch per workgroup into part[m][slice], stage 2 adds the slices
 // in order.
+struct __attribute__((packed, aligned(4))) gb_float4u {  // four floats at a 4-byte aligned address
+    float x, y, z, w;
+};
+
 __global__ __launch_bounds__(256) void gradbias_partial_kernel(const float *__restrict__ gout,
                                                                float *__restrict__ part, int B, int M, int N,
-                                                               int imgs_per_slice, int nslices, const FastDiv divN) {
+                                                               int imgs_per_slice, int nslices, const FastDiv divQ) {
     const int m = blockIdx.x, slice = blockIdx.y;
     const int b0 = slice * imgs_per_slice;
     const int b1 = b0 + imgs_per_slice < B ? b0 + imgs_per_slice : B;
-    // The slice is (b1-b0) rows of N floats, M*N apart; lanes walk it as one
-    // flat array, eight loads in flight each, whatever N is.
-    const unsigned total = (unsigned)(b1 - b0) * (unsigned)N;
+    // The slice is (b1-b0) rows of N floats, M*N apart.  Lanes walk it in quads of four consecutive floats of
+    // one row (one 128-bit load each; the last quad of a row is cut to the row's end), four quads in flight.
+    const int Q = (N + 3) >> 2;  // quads per row
+    const unsigned total = (unsigned)(b1 - b0) * (unsigned)Q;
     const float *base = gout + ((long)b0 * M + m) * N;
-    const long row_gap = (long)(M - 1) * N;  // from the end of one row to the start of the next
+    const long row_stride = (long)M * N;
     float sum = 0.0f;
-    for (unsigned f0 = threadIdx.x; f0 < total; f0 += 256 * 8) {
-        float v[8];
+    for (unsigned f0 = threadIdx.x; f0 < total; f0 += 256 * 4) {
+        float v[4][4];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
+        for (int u = 0; u < 4; ++u) {
             const unsigned f = f0 + 256u * u;
-            const unsigned row = divN.div(f < total ? f : 0);
-            v[u] = f < total ? base[f + row * row_gap] : 0.0f;
+            unsigned row, q;
+            divQ.divmod(f < total ? f : 0, row, q);
+            const float *src = base + (long)row * row_stride + 4 * q;
+            const int left = f < total ? N - 4 * (int)q : 0;  // floats of the row from this quad on
+            if (left >= 4) {
+                const gb_float4u t = *reinterpret_cast<const gb_float4u *>(src);
+                v[u][0] = t.x; v[u][1] = t.y; v[u][2] = t.z; v[u][3] = t.w;
+            } else {
+                v[u][0] = left > 0 ? src[0] : 0.0f;
+                v[u][1] = left > 1 ? src[1] : 0.0f;
+                v[u][2] = left > 2 ? src[2] : 0.0f;
+                v[u][3] = 0.0f;
+            }
         }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) sum += v[u];
+        for (int u = 0; u < 4; ++u) sum += (v[u][0] + v[u][1]) + (v[u][2] + v[u][3]);
     }
     __shared__ float red[256];
     red[threadIdx.x] = sum;
@@ -411,59 +598,99 @@ int maxpool_fwd_launch(const float *in, long planes, int H, int W, int kH, int k
     g.divHoWo = FastDiv((uint32_t)(g.Ho * g.Wo));
     g.divW = FastDiv((uint32_t)W);
     g.divHW = FastDiv((uint32_t)(H * W));
+    const double bytes = 4.0 * (planes * (double)H * W + 3.0 * total);
+    PoolFwdPlan plan;
+    // The pool_fwd_wave switch selects the wavefront-level tile kernel where its plan applies.
+    if (tuning().pool_fwd_wave && plan_pool_fwd(g, planes, plan)) {
+        const long blocks = ((planes + plan.G - 1) / plan.G) * plan.strips;
+        if (blocks < (1L << 31)) {
+            const long rows = plan.G > 1 ? H : (long)(plan.SR - 1) * dH + kH;
+            const long nres = (long)plan.G * (plan.G > 1 ? g.Ho : plan.SR) * g.Wo;
+            const size_t lds = sizeof(float) * (size_t)(((plan.G * rows * W + 3) & ~3L) + 3 * nres);
+            {
+                LaunchScope scope(pool_label("maxpool_fwd", g, planes), 0.0, bytes);
+                const dim3 grid((unsigned)blocks), block(256);
+                float *iy = indices, *ix = indices + total;
+#define THGPU_POOL_FWD(KH_, KW_, DH_, DW_)                                                                         \
+    hipLaunchKernelGGL((maxpool_fwd_tile_kernel<KH_, KW_, DH_, DW_>), grid, block, lds, s, in, out, iy, ix, g, plan, \
+                       (unsigned)planes)
+                if (kH == 3 && kW == 3 && dH == 2 && dW == 2) THGPU_POOL_FWD(3, 3, 2, 2);
+                else if (kH == 2 && kW == 2 && dH == 2 && dW == 2) THGPU_POOL_FWD(2, 2, 2, 2);
+                else THGPU_POOL_FWD(0, 0, 0, 0);
+#undef THGPU_POOL_FWD
+            }
+            return check_launch("maxpool_fwd");
+        }
+    }
     {
-        LaunchScope scope(pool_label("maxpool_fwd", g, planes), 0.0, 4.0 * (planes * (double)H * W + 3.0 * total));
+        LaunchScope scope(pool_label("maxpool_fwd", g, planes), 0.0, bytes);
         const dim3 grid((unsigned)((total + 255) / 256)), block(256);
         if (kH == 3 && kW == 3)
-            hipLaunchKernelGGL((maxpool_fwd_kernel<3, 3>), grid, block, 0, s, in, out, indices, indices + total, g,
+            hipLaunchKernelGGL((maxpool_fwd_direct_kernel<3, 3>), grid, block, 0, s, in, out, indices, indices + total, g,
                                (unsigned)total);
         else if (kH == 2 && kW == 2)
-            hipLaunchKernelGGL((maxpool_fwd_kernel<2, 2>), grid, block, 0, s, in, out, indices, indices + total, g,
+            hipLaunchKernelGGL((maxpool_fwd_direct_kernel<2, 2>), grid, block, 0, s, in, out, indices, indices + total, g,
                                (unsigned)total);
         else
-            hipLaunchKernelGGL((maxpool_fwd_kernel<0, 0>), grid, block, 0, s, in, out, indices, indices + total, g,
+            hipLaunchKernelGGL((maxpool_fwd_direct_kernel<0, 0>), grid, block, 0, s, in, out, indices, indices + total, g,
                                (unsigned)total);
     }
     return check_launch("maxpool_fwd");
 }
 
-// Host check of the backward tile planner: the window rows and columns a strip's pixels look up must
-// lie inside the staged tile, which must fit its LDS budget.
+// Host check of the tile planners: a strip's rows and windows must fit the LDS and register budgets the kernels
+// assume, and the strips must cover the plane.
 long pool_plan_selftest() {
     long bad = 0;
-    const int sizes[] = {2, 3, 6, 7, 12, 13, 14, 24, 27, 28, 55, 56, 112, 224, 231, 1000, 5000};
+    const int sizes[] = {2, 3, 6, 7, 12, 13, 14, 24, 27, 28, 55, 56, 64, 65, 112, 224, 231, 1000, 5000};
     for (int H : sizes)
         for (int W : sizes)
             for (int k = 1; k <= 4; ++k)
                 for (int kw : {k, 2})  // square windows, and every height against a width of 2
                     for (int d = 1; d <= 4; ++d)
                         for (int dw : {d, 2}) {
-                    // the tile kernel takes th == tw in {1, 2}, as the launcher requires
-                    const int th = (k + d - 1) / d, tw = (kw + dw - 1) / dw;
-                    if (H < k || W < kw || th != tw || !(th == 1 || th == 2)) continue;
+                    if (H < k || W < kw) continue;
+                    const int th = (k + d - 1) / d;
                     PoolGeom g;
                     g.H = H; g.W = W; g.kH = k; g.kW = kw; g.dH = d; g.dW = dw;
                     g.Ho = (H - k) / d + 1;
                     g.Wo = (W - kw) / dw + 1;
                     for (long planes : {1L, 5L, 4096L}) {
                         PoolBwdPlan p;
-                        if (!plan_pool_bwd(g, planes, th, tw, p)) continue;
-                        bool ok = p.G >= 1 && p.G <= planes && p.PR >= 1 && p.PR <= H && (p.G == 1 || p.PR == H) &&
-                                  (long)p.G * p.RW * p.CW * 8 <= kPoolBwdLdsBytes && (long)p.tiles * p.PR >= H &&
-                                  (long)(p.tiles - 1) * p.PR < H && p.CW >= (W - 1) / dw + tw;
-                        for (int t = 0; t < p.tiles && ok; ++t) {
-                            const int h0 = t * p.PR, h1 = (h0 + p.PR < H ? h0 + p.PR : H) - 1;
-                            const int i_first = h0 / d - (th - 1);
-                            ok = h1 / d - i_first < p.RW;  // the last pixel row's newest window row
+                        if (plan_pool_bwd(g, planes, th, p)) {
+                            bool ok = p.G >= 1 && p.G <= planes && p.PR >= 1 && p.PR <= H && (p.G == 1 || p.PR == H) &&
+                                      (long)p.G * p.PR * W <= 256L * kPoolBwdPixelsPerLane && (long)p.tiles * p.PR >= H &&
+                                      (long)(p.tiles - 1) * p.PR < H;
+                            for (int t = 0; t < p.tiles && ok; ++t) {
+                                const int h0 = t * p.PR, nh = (h0 + p.PR < H ? h0 + p.PR : H) - h0;
+                                const int t0 = h0 - k + d;
+                                const int i_first = t0 <= 0 ? 0 : t0 / d;
+                                int i_last = (h0 + nh - 1) / d;
+                                if (i_last > g.Ho - 1) i_last = g.Ho - 1;
+                                const long nwin = (long)p.G * (i_last - i_first + 1 > 0 ? i_last - i_first + 1 : 0) * g.Wo;
+                                ok = nwin <= 256L * kPoolBwdWindowsPerLane;
+                            }
+                            if (!ok) ++bad;
                         }
-                        if (!ok) ++bad;
+                        PoolFwdPlan f;
+                        if (plan_pool_fwd(g, planes, f)) {
+                            const long rows = f.G > 1 ? H : (long)(f.SR - 1) * d + k;
+                            bool ok = f.G >= 1 && f.G <= planes && f.SR >= 1 && f.SR <= g.Ho &&
+                                      (f.G == 1 || f.SR == g.Ho) && (long)f.G * rows * W * 4 <= kPoolLdsBytes &&
+                                      (long)f.strips * f.SR >= g.Ho && (long)(f.strips - 1) * f.SR < g.Ho &&
+                                      (long)f.chunks * f.CO >= g.Wo && (f.CO - 1) * dw + kw <= (W <= 64 ? W : 64) &&
+                                      f.P >= 1 && (f.P == 1 || f.P * W <= 64) && (f.P == 1 || f.chunks == 1);
+                            // the last strip's rows end inside the plane
+                            ok = ok && ((long)(g.Ho - 1) * d + k <= H);
+                            if (!ok) ++bad;
+                        }
                     }
                 }
     return bad;
 }
 
 int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int H, int W, int Ho, int Wo, int kH,
-                       int kW, int dH, int dW, float *gin) {
+                       int kW, int dH, int dW, float *gin, InputMask mask) {
     hipStream_t s = stream();
     if (!s) return 1;
     PoolGeom g;
@@ -478,42 +705,25 @@ int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int
     g.divDH = FastDiv((uint32_t)dH);
     g.divDW = FastDiv((uint32_t)dW);
     const int th = (kH + dH - 1) / dH, tw = (kW + dW - 1) / dW;
-    const double bytes = 4.0 * ((double)total + 3.0 * ototal);
+    const double bytes = 4.0 * ((mask.in ? 2.0 : 1.0) * (double)total + 3.0 * ototal);
     PoolBwdPlan plan;
     // The pool_bwd_direct switch forces the direct kernel (a testing and tuning aid).
-    if (!tuning().pool_bwd_direct && ((th == 2 && tw == 2) || (th == 1 && tw == 1)) &&
-        plan_pool_bwd(g, planes, th, tw, plan)) {
+    if (!tuning().pool_bwd_direct && Ho > 0 && Wo > 0 && th * tw <= 64 && plan_pool_bwd(g, planes, th, plan)) {
         const long blocks = ((planes + plan.G - 1) / plan.G) * plan.tiles;
         if (blocks < (1L << 31)) {
-            const size_t lds = sizeof(int2) * (size_t)plan.G * plan.RW * plan.CW;
+            const size_t lds = sizeof(float) * (size_t)plan.G * plan.PR * W;
             {
                 LaunchScope scope(pool_label("maxpool_bwd", g, planes), 0.0, bytes);
-                const dim3 grid((unsigned)blocks), block(256);
-                float *ix = const_cast<float *>(indices) + ototal;
-#define THGPU_POOL_BWD(TH_, TW_, PAIRS_)                                                                          \
-    hipLaunchKernelGGL((maxpool_bwd_tile_kernel<TH_, TW_, PAIRS_>), grid, block, lds, s, gout, indices, ix, gin, g, \
-                       plan, (unsigned)planes)
-                if (th == 2 && dW == 2) THGPU_POOL_BWD(2, 2, true);
-                else if (th == 2) THGPU_POOL_BWD(2, 2, false);
-                else if (dW == 2) THGPU_POOL_BWD(1, 1, true);
-                else THGPU_POOL_BWD(1, 1, false);
-#undef THGPU_POOL_BWD
+                hipLaunchKernelGGL(maxpool_bwd_tile_kernel, dim3((unsigned)blocks), dim3(256), lds, s, gout, indices,
+                                   indices + ototal, gin, g, plan, (unsigned)planes, th, tw, mask);
             }
             return check_launch("maxpool_bwd");
         }
     }
     {
         LaunchScope scope(pool_label("maxpool_bwd", g, planes), 0.0, bytes);
-        const dim3 grid((unsigned)((total + 255) / 256)), block(256);
-        if (th == 2 && tw == 2)
-            hipLaunchKernelGGL((maxpool_bwd_kernel<2, 2>), grid, block, 0, s, gout, indices, indices + ototal, gin, g,
-                               (unsigned)total, th, tw);
-        else if (th == 1 && tw == 1)
-            hipLaunchKernelGGL((maxpool_bwd_kernel<1, 1>), grid, block, 0, s, gout, indices, indices + ototal, gin, g,
-                               (unsigned)total, th, tw);
-        else
-            hipLaunchKernelGGL((maxpool_bwd_kernel<0, 0>), grid, block, 0, s, gout, indices, indices + ototal, gin, g,
-                               (unsigned)total, th, tw);
+        hipLaunchKernelGGL(maxpool_bwd_direct_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, gout,
+                           indices, indices + ototal, gin, g, (unsigned)total, mask);
     }
     return check_launch("maxpool_bwd");
 }
@@ -574,7 +784,7 @@ int gradbias_launch(const float *gout, float *gbias, long B, int M, long N, floa
     {
         LaunchScope scope("gradbias", 0.0, 4.0 * B * M * N);
         hipLaunchKernelGGL(gradbias_partial_kernel, dim3((unsigned)M, (unsigned)nslices), dim3(256), 0, s, gout,
-                           part, (int)B, M, (int)N, ips, (int)nslices, FastDiv((uint32_t)N));
+                           part, (int)B, M, (int)N, ips, (int)nslices, FastDiv((uint32_t)((N + 3) / 4)));
     }
     if (check_launch("gradbias")) return 1;
     {

@@ -55,6 +55,8 @@ static int tuning_set(const char *name, const char *value) {
         std::sscanf(v, "%d,%d,%d", &g_tuning.im2col_plan[0], &g_tuning.im2col_plan[1], &g_tuning.im2col_plan[2]);
     } else if (!std::strcmp(name, "col2im_generic")) {
         g_tuning.col2im_generic = v[0] == '1';
+    } else if (!std::strcmp(name, "pool_fwd_wave")) {
+        g_tuning.pool_fwd_wave = v[0] == '1';
     } else if (!std::strcmp(name, "pool_bwd_direct")) {
         g_tuning.pool_bwd_direct = v[0] == '1';
     } else {
@@ -69,7 +71,8 @@ const Tuning &tuning() {
         static const char *const kEnv[][2] = {
             {"THGPU_GEMM_TILE", "gemm_tile"},           {"THGPU_GEMM_SPLIT", "gemm_split"},
             {"THGPU_IM2COL_KERNEL", "im2col_kernel"},   {"THGPU_IM2COL_PLAN", "im2col_plan"},
-            {"THGPU_COL2IM_GENERIC", "col2im_generic"}, {"THGPU_POOL_BWD_DIRECT", "pool_bwd_direct"}};
+            {"THGPU_COL2IM_GENERIC", "col2im_generic"}, {"THGPU_POOL_FWD_WAVE", "pool_fwd_wave"},
+            {"THGPU_POOL_BWD_DIRECT", "pool_bwd_direct"}};
         for (auto &e : kEnv)
             if (const char *v = std::getenv(e[0])) (void)tuning_set(e[1], v);
     }

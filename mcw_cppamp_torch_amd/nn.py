@@ -191,6 +191,43 @@ class Sequential(Module):
         for m in self.modules:
             m.zeroGradParameters()
 
+    def fuse(self):
+        """Lets the neighbours of every nn.Threshold / nn.ReLU do its work while they store their own results: a
+        SpatialConvolutionMM in front applies the threshold to its output, a SpatialConvolutionMM or
+        SpatialMaxPooling behind zeroes its gradInput where its input (the Threshold's output) is not above the
+        threshold.  The Threshold module stays in place and passes tensors through, so the module API and every
+        result downstream are unchanged bit for bit; what changes is that the convolution's `output` holds the
+        thresholded values and no separate elementwise pass runs.  Needs value <= threshold (true of ReLU), so that
+        output > threshold exactly where input > threshold.  Returns self; unfuse() undoes it."""
+        self.unfuse()
+        mods = self.modules
+        for i, m in enumerate(mods):
+            if isinstance(m, Sequential):
+                m.fuse()
+            if not isinstance(m, Threshold) or not m.val <= m.threshold:
+                continue
+            if i > 0 and isinstance(mods[i - 1], SpatialConvolutionMM) and mods[i - 1].fusedThreshold is None:
+                mods[i - 1].fusedThreshold = (m.threshold, m.val)
+                m.fusedForward = True
+            if i + 1 < len(mods) and isinstance(mods[i + 1], (SpatialConvolutionMM, SpatialMaxPooling)):
+                mods[i + 1].inputThreshold = m.threshold
+                m.fusedBackward = True
+        return self
+
+    def unfuse(self):
+        for m in self.modules:
+            if isinstance(m, Sequential):
+                m.unfuse()
+            elif isinstance(m, Threshold):
+                if m.fusedForward or m.fusedBackward:
+                    m.output, m.gradInput = type(m.output)(), type(m.gradInput)()
+                m.fusedForward = m.fusedBackward = False
+            elif isinstance(m, SpatialConvolutionMM):
+                m.fusedThreshold = m.inputThreshold = None
+            elif isinstance(m, SpatialMaxPooling):
+                m.inputThreshold = None
+        return self
+
     def updateParameters(self, learningRate):
         # mcw_nn/Sequential.lua:91-95
         for m in self.modules:
@@ -244,6 +281,10 @@ class SpatialConvolutionMM(Module):
         self.gradBias = FloatTensor(nOutputPlane)
         self.finput = FloatTensor()
         self.fgradInput = FloatTensor()
+        # set by Sequential.fuse(): (threshold, value) of a following nn.Threshold applied as the output is stored,
+        # and the threshold of a preceding one whose backward is applied as gradInput is stored
+        self.fusedThreshold = None
+        self.inputThreshold = None
         self._rng = rng if rng is not None else np.random.default_rng()
         self.reset()
 
@@ -270,6 +311,11 @@ class SpatialConvolutionMM(Module):
 
     def updateOutput(self, input):
         _require_gpu(input, self.weight, self.bias, self.finput, self.fgradInput, self.output)
+        if self.fusedThreshold is not None:
+            _lib.check_status(lib.thgpu_SpatialConvolutionMM_updateOutputThreshold(
+                input._p, self.weight._p, self.bias._p, self.finput._p, self.fgradInput._p, self.output._p,
+                *(self._geom() + (float(self.fusedThreshold[0]), float(self.fusedThreshold[1])))))
+            return self.output
         _lib.check_status(lib.thgpu_SpatialConvolutionMM_updateOutput(
             input._p, self.weight._p, self.bias._p, self.finput._p, self.fgradInput._p, self.output._p,
             *self._geom()))
@@ -279,6 +325,11 @@ class SpatialConvolutionMM(Module):
         if self.gradInput is None:
             return None
         _require_gpu(input, gradOutput, self.weight, self.finput, self.fgradInput, self.gradInput)
+        if self.inputThreshold is not None:
+            _lib.check_status(lib.thgpu_SpatialConvolutionMM_updateGradInputMasked(
+                input._p, gradOutput._p, self.weight._p, self.finput._p, self.fgradInput._p, self.gradInput._p,
+                *(self._geom() + (float(self.inputThreshold),))))
+            return self.gradInput
         _lib.check_status(lib.thgpu_SpatialConvolutionMM_updateGradInput(
             input._p, gradOutput._p, self.weight._p, self.finput._p, self.fgradInput._p, self.gradInput._p,
             *self._geom()))
@@ -370,6 +421,7 @@ class SpatialMaxPooling(Module):
         self.dW = dW or kW
         self.dH = dH or kH
         self.indices = FloatTensor()
+        self.inputThreshold = None   # set by Sequential.fuse(): the threshold of a preceding nn.Threshold
 
     def updateOutput(self, input):
         _require_gpu(input, self.output, self.indices)
@@ -379,6 +431,11 @@ class SpatialMaxPooling(Module):
 
     def updateGradInput(self, input, gradOutput):
         _require_gpu(input, gradOutput, self.gradInput, self.indices)
+        if self.inputThreshold is not None:
+            _lib.check_status(lib.thgpu_SpatialMaxPooling_updateGradInputMasked(
+                input._p, gradOutput._p, self.gradInput._p, self.indices._p, self.kW, self.kH, self.dW, self.dH,
+                float(self.inputThreshold)))
+            return self.gradInput
         _lib.check_status(lib.thgpu_SpatialMaxPooling_updateGradInput(
             input._p, gradOutput._p, self.gradInput._p, self.indices._p, self.kW, self.kH, self.dW, self.dH))
         return self.gradInput
@@ -460,13 +517,22 @@ class Threshold(Module):
                 raise THGPUError("nn.Threshold(threshold, value)")
         self.threshold = 1e-6 if th is None else th
         self.val = 0 if v is None else v
+        # set by Sequential.fuse(): the neighbouring modules do this module's work as they store their results
+        self.fusedForward = False
+        self.fusedBackward = False
 
     def updateOutput(self, input):
+        if self.fusedForward:
+            self.output = input          # the convolution in front has already applied the threshold
+            return input
         _require_gpu(input, self.output)
         _lib.check_status(lib.thgpu_Threshold_updateOutput(input._p, self.output._p, self.threshold, self.val))
         return self.output
 
     def updateGradInput(self, input, gradOutput):
+        if self.fusedBackward:
+            self.gradInput = gradOutput  # the module behind has already zeroed it where the output is not above the threshold
+            return gradOutput
         _require_gpu(input, gradOutput, self.gradInput)
         _lib.check_status(lib.thgpu_Threshold_updateGradInput(input._p, gradOutput._p, self.gradInput._p,
                                                               self.threshold))

@@ -1,0 +1,173 @@
+"""nn.Threshold / nn.ReLU fused into the neighbouring modules (Sequential.fuse()): the convolution in front applies
+the threshold as it stores its output, the convolution or max-pooling layer behind zeroes its gradInput where the
+Threshold's output is not above the threshold.  The bar is bit-identity with the unfused modules (a threshold is a
+select, not arithmetic), on both convolution routes and with every kernel that carries the fused store forced."""
+import numpy as np
+import pytest
+
+from helpers import rng_for, uniform
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gt():
+    import mcw_cppamp_torch_amd as pkg
+    assert pkg._lib.lib.thgpu_init() == 0, pkg._lib.lib.thgpu_last_error()
+    return pkg
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+def dev(gt, a):
+    return gt.GPUTensor.from_numpy(np.ascontiguousarray(a, np.float32))
+
+
+def build(gt, spec, seed):
+    nn = gt.nn
+    rng = rng_for(seed)
+    net = nn.Sequential()
+    for l in spec:
+        if l[0] == "conv":
+            _, cin, cout, k, s, p = l
+            net.add(nn.SpatialConvolutionMM(cin, cout, k, k, s, s, p, rng=rng))
+        elif l[0] == "pool":
+            net.add(nn.SpatialMaxPooling(l[1], l[1], l[2], l[2]))
+        elif l[0] == "relu":
+            net.add(nn.ReLU())
+        else:
+            net.add(nn.Threshold(l[1], l[2]))
+    return net
+
+
+def run(gt, spec, x, seed, fused, go=None):
+    net = build(gt, spec, seed).gpu()
+    if fused:
+        net.fuse()
+    net.zeroGradParameters()
+    dx = dev(gt, x)
+    out = net.forward(dx).float()
+    if go is None:
+        go = uniform(rng_for(seed + 1), out.shape)
+    gi = net.backward(dx, dev(gt, go)).float()
+    outs = [m.output.float() for m in net.modules]
+    grads = [(m.gradWeight.float(), m.gradBias.float()) for m in net.modules if hasattr(m, "gradWeight")]
+    return net, out, gi, outs, grads, go
+
+
+SPEC = [("conv", 3, 64, 5, 2, 2), ("relu",), ("pool", 3, 2), ("conv", 64, 96, 3, 1, 1), ("relu",),
+        ("conv", 96, 64, 3, 1, 1), ("thr", 0.25, -3.0), ("pool", 2, 2), ("conv", 64, 70, 5, 1, 2), ("relu",)]
+
+
+@pytest.mark.parametrize("mode", [0, 2], ids=["columns", "gathered"])
+def test_fused_stack_is_bit_identical_to_unfused(gt, mode):
+    lib = gt._lib.lib
+    before = lib.thgpu_conv_get_mode()
+    assert lib.thgpu_conv_set_mode(mode) == 0
+    try:
+        x = uniform(rng_for(90), (3, 3, 45, 41))
+        net_u, out_u, gi_u, outs_u, grads_u, go = run(gt, SPEC, x, 91, False)
+        net_f, out_f, gi_f, outs_f, grads_f, _ = run(gt, SPEC, x, 91, True, go)
+        thr = [m for m in net_f.modules if isinstance(m, gt.nn.Threshold)]
+        assert [t.fusedForward for t in thr] == [True] * 4
+        assert [t.fusedBackward for t in thr] == [True, True, True, False]      # the last one has nothing behind it
+        assert np.array_equal(bits(out_u), bits(out_f))
+        assert np.array_equal(bits(gi_u), bits(gi_f))
+        for i, l in enumerate(SPEC):
+            if l[0] in ("relu", "thr", "pool"):
+                assert np.array_equal(bits(outs_u[i]), bits(outs_f[i])), i
+            if l[0] in ("relu", "thr"):         # the fused convolution's output is the thresholded one
+                assert np.array_equal(bits(outs_f[i - 1]), bits(outs_u[i])), i
+        for (gw_u, gb_u), (gw_f, gb_f) in zip(grads_u, grads_f):
+            assert np.array_equal(bits(gw_u), bits(gw_f)) and np.array_equal(bits(gb_u), bits(gb_f))
+        assert (out_u == 0).mean() > 0.2                # the threshold did bite
+        # unfuse() restores the separate passes
+        net_f.unfuse()
+        assert not any(t.fusedForward or t.fusedBackward for t in thr)
+        dx = dev(gt, x)
+        net_f.forward(dx)
+        assert np.array_equal(bits(net_f.modules[0].output.float()), bits(outs_u[0]))
+    finally:
+        assert lib.thgpu_conv_set_mode(before) == 0
+
+
+def test_threshold_with_value_above_threshold_is_not_fused(gt):
+    nn = gt.nn
+    net = nn.Sequential().add(nn.SpatialConvolutionMM(3, 4, 3, 3)).add(nn.Threshold(0.1, 0.5)) \
+        .add(nn.SpatialMaxPooling(2, 2)).fuse()
+    t = net.get(1)
+    assert not t.fusedForward and not t.fusedBackward
+    assert net.get(0).fusedThreshold is None and net.get(2).inputThreshold is None
+
+
+CASES = [
+    # what is forced                    conv spec behind the ReLU                 mode
+    ({"col2im_generic": "1"}, ("conv", 8, 16, 3, 1, 1), 0),
+    ({}, ("conv", 8, 16, 3, 1, 1), 0),                       # col2im_unit_kernel<3,3>
+    ({}, ("conv", 8, 16, 5, 1, 2), 0),                       # col2im_unit_kernel<5,5>
+    ({}, ("conv", 8, 16, 7, 3, 2), 0),                       # col2im_strided_kernel (W >= 64 below)
+    ({}, ("conv", 8, 16, 4, 2, 1), 0),
+    ({}, ("conv", 64, 64, 3, 1, 1), 2),                      # gathered gradInput: tiled GEMM epilogue
+    ({"gemm_split": "3"}, ("conv", 64, 64, 3, 1, 1), 2),     # ... through the split reduction's final pass
+    ({"gemm_tile": "64x64"}, ("conv", 64, 128, 3, 1, 1), 2),
+    ({"gemm_tile": "128x128", "gemm_split": "2"}, ("conv", 128, 128, 3, 1, 1), 2),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=[str(i) for i in range(len(CASES))])
+def test_every_kernel_that_stores_a_masked_gradient_or_a_thresholded_output(gt, case, switches):
+    forced, conv, mode = case
+    for k, v in forced.items():
+        switches(k, v)
+    cin = conv[1]
+    spec = [("conv", 3, cin, 3, 1, 1), ("relu",), conv, ("relu",)]
+    lib = gt._lib.lib
+    before = lib.thgpu_conv_get_mode()
+    assert lib.thgpu_conv_set_mode(mode) == 0
+    try:
+        x = uniform(rng_for(92), (2, 3, 20, 70))
+        _, out_u, gi_u, outs_u, grads_u, go = run(gt, spec, x, 93, False)
+        _, out_f, gi_f, outs_f, grads_f, _ = run(gt, spec, x, 93, True, go)
+        assert np.array_equal(bits(out_u), bits(out_f)) and np.array_equal(bits(gi_u), bits(gi_f))
+        for (gw_u, gb_u), (gw_f, gb_f) in zip(grads_u, grads_f):
+            assert np.array_equal(bits(gw_u), bits(gw_f)) and np.array_equal(bits(gb_u), bits(gb_f))
+    finally:
+        assert lib.thgpu_conv_set_mode(before) == 0
+
+
+@pytest.mark.parametrize("direct", [None, "1"], ids=["tile", "direct"])
+@pytest.mark.parametrize("pool", [(3, 2), (2, 2), (3, 1)])
+def test_masked_pooling_backward(gt, pool, direct, switches):
+    switches("pool_bwd_direct", direct)
+    spec = [("conv", 3, 8, 3, 1, 1), ("relu",), ("pool",) + pool]
+    x = uniform(rng_for(94), (3, 3, 29, 31))
+    _, out_u, gi_u, _, grads_u, go = run(gt, spec, x, 95, False)
+    _, out_f, gi_f, _, grads_f, _ = run(gt, spec, x, 95, True, go)
+    assert np.array_equal(bits(out_u), bits(out_f)) and np.array_equal(bits(gi_u), bits(gi_f))
+    assert np.array_equal(bits(grads_u[0][0]), bits(grads_f[0][0]))
+
+
+def test_full_size_alexnet_fused_equals_unfused(gt):
+    """The benchmark runs the fused stack: at its full size (batch 128) every result must equal the unfused stack's,
+    which tests/test_gpu_stacks_full.py holds to the oracle layer by layer."""
+    stacks = gt.stacks
+    name, B = "alexnet", 128
+    x = stacks.make_input(name, B, seed=4000)
+    go = uniform(rng_for(4003), stacks.output_shape(name, B))
+    res = []
+    for fused in (False, True):
+        net = stacks.build(name, seed_base=4000).gpu()
+        if fused:
+            net.fuse()
+        net.zeroGradParameters()
+        dx = dev(gt, x)
+        out = net.forward(dx).float()
+        gi = net.backward(dx, dev(gt, go)).float()
+        res.append((out, gi, [(m.gradWeight.float(), m.gradBias.float()) for m in net.modules if hasattr(m, "gradWeight")]))
+        del net, dx
+    (out_u, gi_u, gr_u), (out_f, gi_f, gr_f) = res
+    assert np.array_equal(bits(out_u), bits(out_f)) and np.array_equal(bits(gi_u), bits(gi_f))
+    for (gw_u, gb_u), (gw_f, gb_f) in zip(gr_u, gr_f):
+        assert np.array_equal(bits(gw_u), bits(gw_f)) and np.array_equal(bits(gb_u), bits(gb_f))

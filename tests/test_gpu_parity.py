@@ -297,12 +297,19 @@ def test_blas_gemm_every_tile_configuration_exact(gt, tile, ta, tb, split, switc
 POOLS = [(2, 3, 7, 7, 3, 3, 2, 2), (3, 2, 9, 8, 2, 2, 2, 2), (2, 2, 10, 11, 3, 2, 1, 3), (1, 1, 6, 6, 4, 4, 1, 1),
          (4, 16, 55, 55, 3, 3, 2, 2), (2, 8, 13, 13, 3, 3, 2, 2), (2, 4, 24, 24, 2, 2, 2, 2),
          (2, 3, 11, 12, 2, 2, 3, 3),       # windows smaller than the stride: uncovered pixels
-         (1, 2, 224, 224, 2, 2, 2, 2), (3, 5, 14, 9, 3, 3, 2, 2), (2, 2, 10, 10, 3, 3, 3, 3), (1, 1, 3, 300, 3, 3, 2, 2)]
+         (1, 2, 224, 224, 2, 2, 2, 2), (3, 5, 14, 9, 3, 3, 2, 2), (2, 2, 10, 10, 3, 3, 3, 3), (1, 1, 3, 300, 3, 3, 2, 2),
+         (37, 3, 13, 13, 3, 3, 2, 2),      # more planes than one workgroup groups, a ragged last group
+         (2, 3, 30, 31, 5, 4, 1, 1),       # dense overlap: 5 x 4 windows cover a pixel, 20 scatter phases
+         (1, 2, 9, 70, 3, 3, 2, 2),        # rows wider than a wavefront: column chunks
+         (2, 1, 120, 130, 4, 7, 3, 5),     # row strips and column chunks, stride below the window
+         (3, 2, 40, 64, 3, 3, 1, 2), (2, 2, 33, 33, 2, 2, 1, 1), (1, 1, 64, 64, 64, 64, 1, 1)]
 
 
 @pytest.fixture(params=[None, "1"], ids=["auto", "direct"])
 def pool_bwd_kernel(request, switches):
-    """Runs a test with the library's own backward kernel choice, then with the direct kernel forced."""
+    """Runs a test with the library's own forward and backward kernel choice (direct forward, tile backward), then with
+    the other pair forced (wavefront-level tile forward, direct backward)."""
+    switches("pool_fwd_wave", request.param)
     switches("pool_bwd_direct", request.param)
     return request.param
 
