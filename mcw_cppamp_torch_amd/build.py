@@ -56,5 +56,32 @@ def build(verbose=False, jobs=None):
     return LIB_PATH
 
 
+def _lua_include_dirs():
+    """Directories holding lua.h and luaT.h, or None: LUA_INCDIR / TORCH_INSTALL first, then the usual prefixes."""
+    roots = [os.environ.get("LUA_INCDIR"), os.path.join(os.environ.get("TORCH_INSTALL", ""), "include"),
+             "/usr/include/luajit-2.1", "/usr/include/luajit-2.0", "/usr/include/lua5.1", "/usr/local/include",
+             "/usr/include", os.path.expanduser("~/torch/install/include")]
+    roots = [r for r in roots if r and os.path.isdir(r)]
+    lua = next((r for r in roots if os.path.exists(os.path.join(r, "lua.h"))), None)
+    luat = next((r for r in roots if os.path.exists(os.path.join(r, "luaT.h"))), None)
+    return [lua, luat] if lua and luat else None
+
+
+def build_lua_glue(verbose=False):
+    """Compiles lua/gpunn_glue.cpp into libgpunn.so where the Lua and luaT headers exist; returns its path or None
+    (no Lua toolchain: the glue is source only, the Python mirror in nn.py / gputorch.py is the host side)."""
+    inc = _lua_include_dirs()
+    if inc is None:
+        if verbose:
+            print("lua.h / luaT.h not found: lua/gpunn_glue.cpp not built")
+        return None
+    out = os.path.join(HERE, "libgpunn.so")
+    cmd = ["g++", "-O2", "-fPIC", "-shared", "-std=c++11", os.path.join(HERE, "lua", "gpunn_glue.cpp"), "-o", out,
+           "-L" + HERE, "-lthgpu", "-lluaT", "-Wl,-rpath," + HERE] + ["-I" + d for d in dict.fromkeys(inc)]
+    subprocess.check_call(cmd)
+    return out
+
+
 if __name__ == "__main__":
     print(build(verbose="-v" in sys.argv))
+    build_lua_glue(verbose=True)

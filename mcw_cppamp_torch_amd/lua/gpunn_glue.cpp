@@ -1,0 +1,236 @@
+// luaT glue: registers libthgpu's operators under the names, and reading the module fields, that the reference's
+// gpunn does, so that a Torch7 install can `require 'gpunn'` with this library behind it.
+//
+// Replaces gpunn/init.cpp:5-11 (luaopen_libgpunn -> open_libgpunn, gputorch/lib/THC/gpunn-impl/init.cpp:34-65) and the
+// luaT halves of gpunn-impl/SpatialConvolutionMM.cpp:110-443, SpatialMaxPooling.cpp:205-396, Threshold.cpp:16-94,
+// SpatialAveragePooling.cpp:67-248, SpatialSubSampling.cpp:246-452, LogSoftMax.cpp:115-194 and
+// ClassNLLCriterion.cpp:96-198.  Every function is called from Lua as input.nn.<Name>(self, input[, gradOutput[,
+// scale]]) (mcw_nn/SpatialConvolutionMM.lua:48-60): argument 1 is the module table, whose fields are read by the
+// names the reference reads (SpatialConvolutionMM.cpp:116-128).
+//
+// Built by mcw_cppamp_torch_amd/build.py only where lua.h and luaT.h are found (LUA_INCDIR / TORCH_INSTALL, or the
+// usual prefixes); link with -lthgpu -lluaT.  Optional module fields beyond the reference's:
+//   padW, padH        separate paddings (default: the reference's single `padding`)
+//   fusedThreshold, fusedValue   set by gpunn.fuse(net) on a convolution followed by nn.Threshold: the threshold is
+//                     applied as the output is stored
+//   inputThreshold    set by gpunn.fuse(net) on a convolution / max-pooling layer preceded by nn.Threshold: gradInput
+//                     is zeroed where the input is not above it
+extern "C" {
+#include <lua.h>
+#include <lauxlib.h>
+#include <luaT.h>
+}
+#include "../../include/thgpu.h"
+
+namespace {
+
+const char *const kTensor = "torch.GPUTensor";
+
+int fail(lua_State *L, int rc) { return rc ? luaL_error(L, "%s", thgpu_last_error()) : 0; }
+
+THGPUTensor *field(lua_State *L, const char *name) {
+    return static_cast<THGPUTensor *>(luaT_getfieldcheckudata(L, 1, name, kTensor));
+}
+THGPUTensor *arg(lua_State *L, int idx) { return static_cast<THGPUTensor *>(luaT_checkudata(L, idx, kTensor)); }
+
+bool has_field(lua_State *L, const char *name) {
+    lua_getfield(L, 1, name);
+    const bool present = !lua_isnil(L, -1);
+    lua_pop(L, 1);
+    return present;
+}
+double opt_number(lua_State *L, const char *name, double dflt) {
+    lua_getfield(L, 1, name);
+    const double v = lua_isnil(L, -1) ? dflt : lua_tonumber(L, -1);
+    lua_pop(L, 1);
+    return v;
+}
+
+struct ConvFields {
+    int kW, kH, dW, dH, padW, padH;
+};
+ConvFields conv_fields(lua_State *L) {
+    ConvFields f;
+    f.kW = luaT_getfieldcheckint(L, 1, "kW");
+    f.kH = luaT_getfieldcheckint(L, 1, "kH");
+    f.dW = luaT_getfieldcheckint(L, 1, "dW");
+    f.dH = luaT_getfieldcheckint(L, 1, "dH");
+    const int pad = luaT_getfieldcheckint(L, 1, "padding");
+    f.padW = static_cast<int>(opt_number(L, "padW", pad));
+    f.padH = static_cast<int>(opt_number(L, "padH", pad));
+    return f;
+}
+struct PoolFields {
+    int kW, kH, dW, dH;
+};
+PoolFields pool_fields(lua_State *L) {
+    return PoolFields{luaT_getfieldcheckint(L, 1, "kW"), luaT_getfieldcheckint(L, 1, "kH"),
+                      luaT_getfieldcheckint(L, 1, "dW"), luaT_getfieldcheckint(L, 1, "dH")};
+}
+
+// ---- nn.SpatialConvolutionMM -------------------------------------------------------------------------------------
+int conv_updateOutput(lua_State *L) {
+    THGPUTensor *input = arg(L, 2);
+    const ConvFields f = conv_fields(L);
+    if (has_field(L, "fusedThreshold"))
+        fail(L, thgpu_SpatialConvolutionMM_updateOutputThreshold(
+                    input, field(L, "weight"), field(L, "bias"), field(L, "finput"), field(L, "fgradInput"),
+                    field(L, "output"), f.kW, f.kH, f.dW, f.dH, f.padW, f.padH,
+                    static_cast<float>(opt_number(L, "fusedThreshold", 0)), static_cast<float>(opt_number(L, "fusedValue", 0))));
+    else
+        fail(L, thgpu_SpatialConvolutionMM_updateOutput(input, field(L, "weight"), field(L, "bias"), field(L, "finput"),
+                                                        field(L, "fgradInput"), field(L, "output"), f.kW, f.kH, f.dW,
+                                                        f.dH, f.padW, f.padH));
+    return 1;
+}
+int conv_updateGradInput(lua_State *L) {
+    THGPUTensor *input = arg(L, 2), *gradOutput = arg(L, 3);
+    const ConvFields f = conv_fields(L);
+    if (has_field(L, "inputThreshold"))
+        fail(L, thgpu_SpatialConvolutionMM_updateGradInputMasked(
+                    input, gradOutput, field(L, "weight"), field(L, "finput"), field(L, "fgradInput"),
+                    field(L, "gradInput"), f.kW, f.kH, f.dW, f.dH, f.padW, f.padH,
+                    static_cast<float>(opt_number(L, "inputThreshold", 0))));
+    else
+        fail(L, thgpu_SpatialConvolutionMM_updateGradInput(input, gradOutput, field(L, "weight"), field(L, "finput"),
+                                                           field(L, "fgradInput"), field(L, "gradInput"), f.kW, f.kH,
+                                                           f.dW, f.dH, f.padW, f.padH));
+    return 1;
+}
+int conv_accGradParameters(lua_State *L) {
+    THGPUTensor *input = arg(L, 2), *gradOutput = arg(L, 3);
+    const float scale = static_cast<float>(luaL_optnumber(L, 4, 1));  // SpatialConvolutionMM.cpp:326
+    const ConvFields f = conv_fields(L);
+    fail(L, thgpu_SpatialConvolutionMM_accGradParameters(input, gradOutput, field(L, "gradWeight"), field(L, "gradBias"),
+                                                         field(L, "finput"), field(L, "fgradInput"), f.kW, f.kH, f.dW,
+                                                         f.dH, f.padW, f.padH, scale));
+    return 0;
+}
+
+// ---- nn.SpatialMaxPooling ------------------------------------------------------------------------------------------
+int pool_updateOutput(lua_State *L) {
+    const PoolFields f = pool_fields(L);
+    fail(L, thgpu_SpatialMaxPooling_updateOutput(arg(L, 2), field(L, "output"), field(L, "indices"), f.kW, f.kH, f.dW,
+                                                 f.dH));
+    return 1;
+}
+int pool_updateGradInput(lua_State *L) {
+    const PoolFields f = pool_fields(L);
+    if (has_field(L, "inputThreshold"))
+        fail(L, thgpu_SpatialMaxPooling_updateGradInputMasked(arg(L, 2), arg(L, 3), field(L, "gradInput"),
+                                                              field(L, "indices"), f.kW, f.kH, f.dW, f.dH,
+                                                              static_cast<float>(opt_number(L, "inputThreshold", 0))));
+    else
+        fail(L, thgpu_SpatialMaxPooling_updateGradInput(arg(L, 2), arg(L, 3), field(L, "gradInput"), field(L, "indices"),
+                                                        f.kW, f.kH, f.dW, f.dH));
+    return 1;
+}
+
+// ---- nn.Threshold / nn.ReLU ------------------------------------------------------------------------------------------
+int thr_updateOutput(lua_State *L) {
+    fail(L, thgpu_Threshold_updateOutput(arg(L, 2), field(L, "output"),
+                                         static_cast<float>(luaT_getfieldchecknumber(L, 1, "threshold")),
+                                         static_cast<float>(luaT_getfieldchecknumber(L, 1, "val"))));
+    return 1;
+}
+int thr_updateGradInput(lua_State *L) {
+    fail(L, thgpu_Threshold_updateGradInput(arg(L, 2), arg(L, 3), field(L, "gradInput"),
+                                            static_cast<float>(luaT_getfieldchecknumber(L, 1, "threshold"))));
+    return 1;
+}
+
+// ---- nn.SpatialAveragePooling / nn.SpatialSubSampling ------------------------------------------------------------------
+int avg_updateOutput(lua_State *L) {
+    const PoolFields f = pool_fields(L);
+    fail(L, thgpu_SpatialAveragePooling_updateOutput(arg(L, 2), field(L, "output"), f.kW, f.kH, f.dW, f.dH));
+    return 1;
+}
+int avg_updateGradInput(lua_State *L) {
+    const PoolFields f = pool_fields(L);
+    fail(L, thgpu_SpatialAveragePooling_updateGradInput(arg(L, 2), arg(L, 3), field(L, "gradInput"), f.kW, f.kH, f.dW,
+                                                        f.dH));
+    return 1;
+}
+int sub_updateOutput(lua_State *L) {
+    const PoolFields f = pool_fields(L);
+    fail(L, thgpu_SpatialSubSampling_updateOutput(arg(L, 2), field(L, "weight"), field(L, "bias"), field(L, "output"),
+                                                  f.kW, f.kH, f.dW, f.dH));
+    return 1;
+}
+int sub_updateGradInput(lua_State *L) {
+    const PoolFields f = pool_fields(L);
+    fail(L, thgpu_SpatialSubSampling_updateGradInput(arg(L, 2), arg(L, 3), field(L, "weight"), field(L, "gradInput"),
+                                                     f.kW, f.kH, f.dW, f.dH));
+    return 1;
+}
+int sub_accGradParameters(lua_State *L) {
+    const PoolFields f = pool_fields(L);
+    fail(L, thgpu_SpatialSubSampling_accGradParameters(arg(L, 2), arg(L, 3), field(L, "gradWeight"), field(L, "gradBias"),
+                                                       f.kW, f.kH, f.dW, f.dH,
+                                                       static_cast<float>(luaL_optnumber(L, 4, 1))));
+    return 0;
+}
+
+// ---- nn.LogSoftMax / nn.ClassNLLCriterion ----------------------------------------------------------------------------------
+int lsm_updateOutput(lua_State *L) {
+    fail(L, thgpu_LogSoftMax_updateOutput(arg(L, 2), field(L, "output")));
+    return 1;
+}
+int lsm_updateGradInput(lua_State *L) {
+    fail(L, thgpu_LogSoftMax_updateGradInput(arg(L, 3), field(L, "output"), field(L, "gradInput")));
+    return 1;
+}
+int nll_updateOutput(lua_State *L) {
+    fail(L, thgpu_ClassNLLCriterion_updateOutput(arg(L, 2), arg(L, 3), field(L, "outputTensor"),
+                                                 luaT_getfieldcheckboolean(L, 1, "sizeAverage")));
+    return 1;
+}
+int nll_updateGradInput(lua_State *L) {
+    fail(L, thgpu_ClassNLLCriterion_updateGradInput(arg(L, 2), arg(L, 3), field(L, "gradInput"),
+                                                    luaT_getfieldcheckboolean(L, 1, "sizeAverage")));
+    return 1;
+}
+
+const struct luaL_Reg kOps[] = {
+    {"SpatialConvolutionMM_updateOutput", conv_updateOutput},
+    {"SpatialConvolutionMM_updateGradInput", conv_updateGradInput},
+    {"SpatialConvolutionMM_accGradParameters", conv_accGradParameters},
+    {"SpatialMaxPooling_updateOutput", pool_updateOutput},
+    {"SpatialMaxPooling_updateGradInput", pool_updateGradInput},
+    {"Threshold_updateOutput", thr_updateOutput},
+    {"Threshold_updateGradInput", thr_updateGradInput},
+    {"SpatialAveragePooling_updateOutput", avg_updateOutput},
+    {"SpatialAveragePooling_updateGradInput", avg_updateGradInput},
+    {"SpatialSubSampling_updateOutput", sub_updateOutput},
+    {"SpatialSubSampling_updateGradInput", sub_updateGradInput},
+    {"SpatialSubSampling_accGradParameters", sub_accGradParameters},
+    {"LogSoftMax_updateOutput", lsm_updateOutput},
+    {"LogSoftMax_updateGradInput", lsm_updateGradInput},
+    {"ClassNLLCriterion_updateOutput", nll_updateOutput},
+    {"ClassNLLCriterion_updateGradInput", nll_updateGradInput},
+    {NULL, NULL}};
+
+// gputorch.synchronize() / the library's own switches, as a small table `gpunn.thgpu`.
+int l_synchronize(lua_State *L) { return fail(L, thgpu_synchronize()); }
+int l_conv_mode(lua_State *L) { return fail(L, thgpu_conv_set_mode(static_cast<int>(luaL_checkinteger(L, 1)))); }
+int l_finput_reuse(lua_State *L) { return fail(L, thgpu_conv_set_finput_reuse(lua_toboolean(L, 1))); }
+const struct luaL_Reg kLib[] = {
+    {"synchronize", l_synchronize}, {"setConvMode", l_conv_mode}, {"setFinputReuse", l_finput_reuse}, {NULL, NULL}};
+
+void lua_error_handler(const char *msg, void *data) { luaL_error(static_cast<lua_State *>(data), "%s", msg); }
+
+}  // namespace
+
+extern "C" int luaopen_libgpunn(lua_State *L) {
+    // TH-named functions report through this handler, as luaopen_libtorch arranges for TH
+    // (mcw_torch7_core/init.c:38-55).
+    THGPUSetErrorHandler(lua_error_handler, L);
+    if (thgpu_init() != 0) return luaL_error(L, "%s", thgpu_last_error());
+    luaT_pushmetatable(L, kTensor);
+    luaT_registeratname(L, kOps, "nn");
+    lua_pop(L, 1);
+    lua_newtable(L);
+    luaL_register(L, NULL, kLib);
+    lua_setfield(L, LUA_GLOBALSINDEX, "thgpu");
+    return 0;
+}
