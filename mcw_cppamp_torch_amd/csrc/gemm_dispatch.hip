@@ -60,15 +60,26 @@ struct TileCfg {
     // measured launch times together with the occupancy factors of model_cycles.
     double eff[5];
     int (*launch)(const GemmArgs &, int, int, bool, hipStream_t);
+    // Fraction of that rate kept with k = 1..4 workgroups resident per CU (nullptr: the tables of model_cycles), and
+    // the row count from which the tile is no longer considered (0: no limit).
+    const double *occ;
+    int below_rows;
 };
 
+// The 64 x 128 tile's wavefronts own 64 x 32 outputs, half the MFMAs per reduction step of the large tiles: it needs all
+// four workgroups on a CU to keep the matrix pipe busy (measured on the 64-row products of the AlexNet-style stack: the
+// 64 x 4800 gathered gradInput runs 10 % faster in seven splits that fill every round than unsplit with three
+// workgroups per CU).  Taller tiles re-read the second operand less often, so it only stands in where they do not fit.
+const double kOccNarrow[5] = {0.0, 0.50, 0.75, 0.88, 1.0};
+
 const TileCfg kCfgs[] = {
-    {"128x128", 128, 128, 4, {0.90, 0.90, 0.88, 0.86, 0.90}, gemm_fast_128x128},
-    {"192x128", 192, 128, 3, {0.90, 0.90, 0.90, 0.86, 0.90}, gemm_fast_192x128},
-    {"64x256", 64, 256, 3, {0.76, 0.74, 0.90, 0.74, 0.70}, gemm_fast_64x256},
-    {"128x256", 128, 256, 2, {0.85, 0.87, 0.95, 0.85, 0.85}, gemm_fast_128x256},
-    {"256x128", 256, 128, 2, {0.90, 0.75, 0.95, 0.75, 0.90}, gemm_fast_256x128},
-    {"64x64", 64, 64, 4, {0.68, 0.60, 0.74, 0.60, 0.72}, gemm_fast_64x64},
+    {"128x128", 128, 128, 4, {0.90, 0.90, 0.88, 0.86, 0.90}, gemm_fast_128x128, nullptr, 0},
+    {"192x128", 192, 128, 3, {0.90, 0.90, 0.90, 0.86, 0.90}, gemm_fast_192x128, nullptr, 0},
+    {"64x256", 64, 256, 3, {0.76, 0.74, 0.90, 0.74, 0.70}, gemm_fast_64x256, nullptr, 0},
+    {"128x256", 128, 256, 2, {0.85, 0.87, 0.95, 0.85, 0.85}, gemm_fast_128x256, nullptr, 0},
+    {"256x128", 256, 128, 2, {0.90, 0.75, 0.95, 0.75, 0.90}, gemm_fast_256x128, nullptr, 0},
+    {"64x64", 64, 64, 4, {0.68, 0.60, 0.74, 0.60, 0.72}, gemm_fast_64x64, nullptr, 0},
+    {"64x128", 64, 128, 4, {0.84, 0.78, 0.84, 0.78, 0.86}, gemm_fast_64x128, kOccNarrow, 128},
 };
 
 inline long cdiv(long a, long b) { return (a + b - 1) / b; }
@@ -83,7 +94,7 @@ double model_cycles(const TileCfg &c, int layout, long M, long J, long steps_tot
     // busy as three: measured on the 192 x 1600 gradWeight product, 39 splits (two per CU) beat 59.
     static const double kOccDefault[5] = {0.0, 0.70, 0.88, 0.96, 1.0};
     static const double kOccBothR[5] = {0.0, 0.70, 0.98, 0.96, 1.0};
-    const double *kOcc = layout == 2 ? kOccBothR : kOccDefault;
+    const double *kOcc = c.occ ? c.occ : layout == 2 ? kOccBothR : kOccDefault;
     const long tiles = cdiv(M, c.bm) * cdiv(J, c.bn);
     const long wgs = tiles * nsplit;
     const long steps = cdiv(steps_total, nsplit);
@@ -135,6 +146,7 @@ GemmPlan plan_gemm(const GemmProblem &p, int steps_total) {
     for (const TileCfg &c : kCfgs) {
         if (!fast_ok || p.M < c.bm || p.J < c.bn || !offsets_fit(c.bm, c.bn)) continue;
         if (force && std::strcmp(force, c.name) != 0) continue;
+        if (!force && c.below_rows > 0 && p.M >= c.below_rows) continue;
         const long tiles = cdiv(p.M, c.bm) * cdiv(p.J, c.bn);
         const int max_split = (int)(steps_total / 8 > 0 ? (steps_total / 8 < 256 ? steps_total / 8 : 256) : 1);
         for (int ns = 1; ns <= max_split; ++ns) {

@@ -127,6 +127,7 @@ int gemm_fast_128x256(const GemmArgs &g, int la, int lb, bool red, hipStream_t s
 int gemm_fast_256x128(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
 int gemm_fast_64x64(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
 int gemm_fast_64x256(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
+int gemm_fast_64x128(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
 // The bounds-checked kernel for shapes smaller than a tile (gemm_generic.hip).
 int gemm_generic_64x64(const GemmArgs &g, bool a_rc, bool b_rc, bool red, hipStream_t s);
 

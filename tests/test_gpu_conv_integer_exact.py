@@ -21,7 +21,7 @@ pytestmark = pytest.mark.gpu
 import oracle  # noqa: E402
 
 TILES = {"128x128": (128, 128), "192x128": (192, 128), "64x256": (64, 256), "128x256": (128, 256),
-         "256x128": (256, 128), "64x64": (64, 64)}
+         "256x128": (256, 128), "64x64": (64, 64), "64x128": (64, 128)}
 
 SHAPES = {
     # name: B, C, H, W, M, kH, kW, pH, pW, sH, sW

@@ -250,7 +250,7 @@ def test_blas_gemm_integer_exact_beta0_ignores_nan_and_quick_returns(gt):
     assert np.array_equal(dc.float(), before * 3.0)
 
 
-GEMM_TILES = ["128x128", "192x128", "64x256", "128x256", "256x128", "64x64"]
+GEMM_TILES = ["128x128", "192x128", "64x256", "128x256", "256x128", "64x64", "64x128"]
 
 
 @pytest.mark.parametrize("split", [1, 3])
