@@ -269,6 +269,12 @@ float THGPUTensor_get4d(const THGPUTensor *tensor, long x0, long x1, long x2, lo
 void THGPUTensor_fill(THGPUTensor *self, float value);
 void THGPUTensor_zero(THGPUTensor *self);
 
+/* THGPUTensor_fill for `count` contiguous tensors in one kernel launch (no counterpart in the reference, where a
+ * network's gradients are zeroed tensor by tensor, mcw_nn/Module.lua:66-73, or flattened into one storage by
+ * getParameters first): what nn.Sequential:zeroGradParameters amounts to on a stack of small layers.  Returns 0
+ * or a status with thgpu_last_error() set; nothing is written when a tensor is rejected. */
+int thgpu_fill_many(THGPUTensor **tensors, int count, float value);
+
 /* gputorch/lib/THC/THCTensorCopy.h:7-23.  copy handles any strides
  * (THCTensorCopy.cpp:170-290); host<->device copies are blocking
  * (THCTensorCopy.cpp:20-36,64-80). */
@@ -383,20 +389,39 @@ int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor
 
 /* nn.Threshold fused into its neighbours (no counterpart in the reference, where gpunn_Threshold_updateOutput /
  * _updateGradInput, gpunn-impl/Threshold.cpp:16-81, always run as passes of their own).
- * updateOutputThreshold: output = y > threshold ? y : val for every y = conv(input) + bias, applied as the
- *   value is stored; bit-identical to updateOutput followed by thgpu_Threshold_updateOutput in place.
- * updateGradInputMasked: gradInput = input > threshold ? g : 0 for every g of updateGradInput, applied as the
- *   value is stored -- the backward of a Threshold in front of this module, whose output `input` is
+ * updateOutputFused, THGPU_FUSE_THRESHOLD: output = y > threshold ? y : val for every y = conv(input) + bias, applied
+ *   as the value is stored; bit-identical to updateOutput followed by thgpu_Threshold_updateOutput in place.
+ * updateGradInputFused, THGPU_FUSE_INPUT_MASK: gradInput = input > threshold ? g : 0 for every g of updateGradInput,
+ *   applied as the value is stored -- the backward of a Threshold in front of this module, whose output `input` is
  *   (value <= threshold assumed, so that its output exceeds the threshold exactly where its input did);
- *   bit-identical to updateGradInput followed by thgpu_Threshold_updateGradInput. */
-int thgpu_SpatialConvolutionMM_updateOutputThreshold(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias,
-                                                     THGPUTensor *finput, THGPUTensor *fgradInput,
-                                                     THGPUTensor *output, int kW, int kH, int dW, int dH, int padW,
-                                                     int padH, float threshold, float val);
-int thgpu_SpatialConvolutionMM_updateGradInputMasked(THGPUTensor *input, THGPUTensor *gradOutput,
-                                                     THGPUTensor *weight, THGPUTensor *finput,
-                                                     THGPUTensor *fgradInput, THGPUTensor *gradInput, int kW, int kH,
-                                                     int dW, int dH, int padW, int padH, float threshold);
+ *   bit-identical to updateGradInput followed by thgpu_Threshold_updateGradInput.
+ *
+ * The padded image without a copy.  On the gathered route (thgpu_conv_set_mode) updateOutput and accGradParameters
+ * read a copy of the input with a zero border of padH rows and padW columns.  A producer can write that image
+ * itself: SpatialConvolutionMM_updateOutput* and SpatialMaxPooling_updateOutput leave an `output` tensor that
+ * already has the right sizes as it is, also when it is a view with contiguous rows into a larger buffer (strides
+ * (C*P, P, pitch, 1)), and store into it.  With THGPU_INPUT_IN_PADDED_BUFFER the caller states that `input` is
+ * such a view: the interior of a [B, C, H + 2 padH, W + 2 padW] buffer whose border holds zeros.  The layout is
+ * checked, the zeros are the caller's word; no copy is made and finput stays untouched (a layer that does not
+ * gather copies the view into dense form first).  updateGradInputFused takes its mask from such a view as well. */
+#define THGPU_FUSE_THRESHOLD 1          /* updateOutputFused */
+#define THGPU_FUSE_INPUT_MASK 1         /* updateGradInputFused */
+#define THGPU_INPUT_IN_PADDED_BUFFER 2  /* updateOutputFused, accGradParametersFused */
+int thgpu_SpatialConvolutionMM_updateOutputFused(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias,
+                                                 THGPUTensor *finput, THGPUTensor *fgradInput, THGPUTensor *output,
+                                                 int kW, int kH, int dW, int dH, int padW, int padH, int flags,
+                                                 float threshold, float val);
+int thgpu_SpatialConvolutionMM_updateGradInputFused(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *weight,
+                                                    THGPUTensor *finput, THGPUTensor *fgradInput,
+                                                    THGPUTensor *gradInput, int kW, int kH, int dW, int dH, int padW,
+                                                    int padH, int flags, float threshold);
+int thgpu_SpatialConvolutionMM_accGradParametersFused(THGPUTensor *input, THGPUTensor *gradOutput,
+                                                      THGPUTensor *gradWeight, THGPUTensor *gradBias,
+                                                      THGPUTensor *finput, THGPUTensor *fgradInput, int kW, int kH,
+                                                      int dW, int dH, int padW, int padH, float scale, int flags);
+/* 1 when updateOutput / accGradParameters of a layer with these sizes would gather from the padded image in the
+ * current mode (and so profit from an input that already lies in a padded buffer), 0 otherwise. */
+int thgpu_conv_gathers(long B, int C, int H, int W, int M, int kW, int kH, int dW, int dH, int padW, int padH);
 
 /* How the three entry points above compute (no counterpart in the reference, whose only route is
  * im2col + sgemm + col2im, gpunn-impl/SpatialConvolutionMM.cpp:110-429).

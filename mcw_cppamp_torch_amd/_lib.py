@@ -164,6 +164,7 @@ _SIGNATURES = {
     "THGPUTensor_get3d": (c_float, [TensorP] + [c_long] * 3),
     "THGPUTensor_get4d": (c_float, [TensorP] + [c_long] * 4),
     "THGPUTensor_fill": (None, [TensorP, c_float]),
+    "thgpu_fill_many": (c_int, [ctypes.POINTER(TensorP), c_int, c_float]),
     "THGPUTensor_zero": (None, [TensorP]),
     "THGPUTensor_copy": (None, [TensorP, TensorP]),
     "THGPUTensor_copyGPU": (None, [TensorP, TensorP]),
@@ -187,8 +188,10 @@ _SIGNATURES = {
     "thgpu_SpatialConvolutionMM_updateOutput": (c_int, [TensorP] * 6 + [c_int] * 6),
     "thgpu_SpatialConvolutionMM_updateGradInput": (c_int, [TensorP] * 6 + [c_int] * 6),
     "thgpu_SpatialConvolutionMM_accGradParameters": (c_int, [TensorP] * 6 + [c_int] * 6 + [c_float]),
-    "thgpu_SpatialConvolutionMM_updateOutputThreshold": (c_int, [TensorP] * 6 + [c_int] * 6 + [c_float] * 2),
-    "thgpu_SpatialConvolutionMM_updateGradInputMasked": (c_int, [TensorP] * 6 + [c_int] * 6 + [c_float]),
+    "thgpu_SpatialConvolutionMM_updateOutputFused": (c_int, [TensorP] * 6 + [c_int] * 7 + [c_float] * 2),
+    "thgpu_SpatialConvolutionMM_updateGradInputFused": (c_int, [TensorP] * 6 + [c_int] * 7 + [c_float]),
+    "thgpu_SpatialConvolutionMM_accGradParametersFused": (c_int, [TensorP] * 6 + [c_int] * 6 + [c_float, c_int]),
+    "thgpu_conv_gathers": (c_int, [c_long] + [c_int] * 10),
     "thgpu_SpatialMaxPooling_updateGradInputMasked": (c_int, [TensorP] * 4 + [c_int] * 4 + [c_float]),
     "thgpu_SpatialMaxPooling_updateOutput": (c_int, [TensorP] * 3 + [c_int] * 4),
     "thgpu_SpatialMaxPooling_updateGradInput": (c_int, [TensorP] * 4 + [c_int] * 4),

@@ -283,7 +283,8 @@ int pad_planes_launch(const float *in, long planes, int H, int W, int pH, int pW
 }
 
 int conv_implicit_forward(const float *padded, const float *weight, const float *bias, float *output, long B, int C,
-                          int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW, OutputThreshold act) {
+                          int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW, OutputThreshold act,
+                          OutputLayout out) {
     const int Hp = H + 2 * pH, Wp = W + 2 * pW;
     const int Ho = (Hp - kH) / sH + 1, Wo = (Wp - kW) / sW + 1;
     if (trim_tables()) return 1;
@@ -298,6 +299,14 @@ int conv_implicit_forward(const float *padded, const float *weight, const float 
     p.act = act.on;
     p.act_threshold = act.threshold;
     p.act_value = act.value;
+    if (out.plane > 0) {
+        p.sC = out.plane;
+        p.bsC = (long)M * out.plane;
+    }
+    if (out.pitch > 0) {
+        p.c_pitch = out.pitch;
+        p.c_w = Wo;
+    }
     return gemm_launch(p);
 }
 
@@ -344,6 +353,14 @@ int conv_implicit_gradinput(const float *gradOutput, const float *weight, float 
     p.C = gradInput;
     p.mask = mask.in;
     p.mask_threshold = mask.threshold;
+    if (mask.in && mask.plane > 0) {
+        p.mask_sC = mask.plane;
+        p.mask_bsC = (long)C * mask.plane;
+    }
+    if (mask.in && mask.pitch > 0) {
+        p.mask_pitch = mask.pitch;
+        p.c_w = W;
+    }
     return gemm_launch(p);
 }
 

@@ -17,7 +17,8 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(const float *__restri
                                                            long sC, long bsC, FastDiv divJ, FastDiv divN, int nsplit,
                                                            float alpha, float beta, int act, float act_threshold,
                                                            float act_value, const float *__restrict__ mask,
-                                                           float mask_threshold) {
+                                                           float mask_threshold, int c_pitch, int mask_pitch,
+                                                           long mask_sC, long mask_bsC, FastDiv divCW) {
     unsigned idx = blockIdx.x * blockDim.x + threadIdx.x;
     const unsigned total = (unsigned)M * (unsigned)J;
     if (idx >= total) return;
@@ -34,18 +35,20 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(const float *__restri
     }
     unsigned i, j;
     divJ.divmod(idx, i, j);
-    long coff = j;
-    if (N != J) {
-        unsigned im, n;
+    long coff = j, moff = j;
+    if (N != J || c_pitch || mask_pitch) {
+        unsigned im, n, y, x;
         divN.divmod(j, im, n);
-        coff = (long)im * bsC + n;
+        divCW.divmod(n, y, x);
+        coff = (long)im * bsC + (c_pitch ? (long)y * c_pitch + x : (long)n);
+        moff = (long)im * mask_bsC + (mask_pitch ? (long)y * mask_pitch + x : (long)n);
     }
     float *c = C + (long)i * sC + coff;
     float val = alpha * sum;
     if (bias) val += bias[i];
     if (beta != 0.0f) val += beta * *c;
     if (act) val = val > act_threshold ? val : act_value;
-    if (mask) val = mask[c - C] > mask_threshold ? val : 0.0f;
+    if (mask) val = mask[(long)i * mask_sC + moff] > mask_threshold ? val : 0.0f;
     *c = val;
 }
 
@@ -216,6 +219,14 @@ int gemm_launch(const GemmProblem &p) {
     g.act_value = p.act_value;
     g.mask = p.mask;
     g.mask_threshold = p.mask_threshold;
+    if ((p.c_pitch || p.mask_pitch) && (p.c_w <= 0 || red || g.N % p.c_w != 0))
+        return fail("gemm: pitched rows need column batching and a plane width that divides the columns of an image");
+    g.c_w = p.c_w > 0 ? p.c_w : 1;
+    g.c_pitch = p.c_pitch;
+    g.mask_pitch = p.mask_pitch;
+    g.mask_sC = p.mask_sC ? p.mask_sC : p.sC;
+    g.mask_bsC = p.mask_bsC ? p.mask_bsC : p.bsC;
+    g.divCW = FastDiv((uint32_t)g.c_w);
     g.steps_per_img = (p.R + GEMM_BK - 1) / GEMM_BK;
     g.steps_total = g.steps_per_img * (red ? p.nb : 1);
     g.divSpi = FastDiv((uint32_t)(g.steps_per_img > 0 ? g.steps_per_img : 1));
@@ -281,7 +292,8 @@ int gemm_launch(const GemmProblem &p) {
             LaunchScope scope("gemm_split_reduce", 0.0, 4.0 * n * (g.nsplit + 2));
             hipLaunchKernelGGL(split_reduce_kernel, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, s, g.ws, p.C, p.bias,
                                p.M, p.J, g.N, p.sC, p.bsC, FastDiv((uint32_t)p.J), g.divN, g.nsplit, p.alpha,
-                               p.beta, g.act, g.act_threshold, g.act_value, g.mask, g.mask_threshold);
+                               p.beta, g.act, g.act_threshold, g.act_value, g.mask, g.mask_threshold, g.c_pitch,
+                               g.mask_pitch, g.mask_sC, g.mask_bsC, g.divCW);
         }
         if (check_launch("gemm_split_reduce")) return 1;
     }

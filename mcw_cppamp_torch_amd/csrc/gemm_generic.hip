@@ -187,13 +187,15 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_generic_kernel(const GemmA
     for (int b = 0; b < TN; ++b) {
         const int jg = j0 + wn * (TN * 32) + b * 32 + l32;
         if (jg >= g.J) continue;
-        long coff;
+        long coff, moff = jg;
         if (partial) {
             coff = (long)split * g.M * g.J + jg;
-        } else if (!RED && g.N != g.J) {
-            unsigned im, n;
+        } else if (!RED && (g.N != g.J || g.c_pitch || g.mask_pitch)) {
+            unsigned im, n, y, x;
             g.divN.divmod((unsigned)jg, im, n);
-            coff = (long)im * g.bsC + n;
+            g.divCW.divmod(n, y, x);
+            coff = (long)im * g.bsC + (g.c_pitch ? (long)y * g.c_pitch + x : (long)n);
+            moff = (long)im * g.mask_bsC + (g.mask_pitch ? (long)y * g.mask_pitch + x : (long)n);
         } else {
             coff = jg;
         }
@@ -212,7 +214,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_generic_kernel(const GemmA
                     if (g.bias) val += g.bias[i];
                     if (g.beta != 0.0f) val += g.beta * *c;
                     if (g.act) val = val > g.act_threshold ? val : g.act_value;
-                    if (g.mask) val = g.mask[c - g.C] > g.mask_threshold ? val : 0.0f;
+                    if (g.mask) val = g.mask[(long)i * g.mask_sC + moff] > g.mask_threshold ? val : 0.0f;
                     *c = val;
                 }
             }

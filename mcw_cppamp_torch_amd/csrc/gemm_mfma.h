@@ -51,6 +51,12 @@ struct GemmProblem {
     float act_threshold = 0.0f, act_value = 0.0f;
     const float *mask = nullptr;
     float mask_threshold = 0.0f;
+    // Column batching only: the N columns of an image are an image plane of width c_w, and C / mask keep it with
+    // rows c_pitch / mask_pitch floats apart (0: densely, column n at offset n): a result written into the
+    // interior of a zero-bordered buffer, a mask read from one.  The mask takes its own row and image strides
+    // (0: those of C).
+    int c_w = 0, c_pitch = 0, mask_pitch = 0;
+    long mask_sC = 0, mask_bsC = 0;
     const char *tag = "gemm";     // name used by per-kernel timing
     // Flops the per-kernel timing credits the launch with; 0 means the product's own 2*M*J*R*nb.  A
     // convolution pass sets its algorithmic 2*M*N*K*B here, which a gathered gradInput product (one
@@ -95,6 +101,9 @@ struct GemmArgs {
     float act_threshold, act_value;
     const float *mask;
     float mask_threshold;
+    int c_w, c_pitch, mask_pitch;
+    long mask_sC, mask_bsC;
+    FastDiv divCW;
 };
 
 // Workgroups are handed to the 8 XCDs round-robin by linear id.  Remap so that

@@ -11,14 +11,26 @@ namespace thgpu {
 struct InputMask {
     const float *in = nullptr;
     float threshold = 0.0f;
+    // Layout of `in` where a kernel accepts another than the result's dense one (the gathered convolution's
+    // gradInput store): floats between its planes (0: dense) and between its rows (0: dense).
+    long plane = 0;
+    int pitch = 0;
+};
+
+// Where a convolution's output planes go when not densely packed: floats between planes (images are
+// nOutputPlane planes apart) and between the rows of a plane (0: dense rows).
+struct OutputLayout {
+    long plane = 0;  // 0: dense
+    int pitch = 0;
 };
 
 int im2col_launch(const float *im, long B, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW,
                   float *col);
 int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW,
                   float *im, InputMask mask = InputMask());
+// out_plane / out_pitch: floats between the output's planes and rows when it is not densely packed (0: dense).
 int maxpool_fwd_launch(const float *in, long planes, int H, int W, int kH, int kW, int dH, int dW, float *out,
-                       float *indices);
+                       float *indices, long out_plane = 0, int out_pitch = 0);
 int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int H, int W, int Ho, int Wo, int kH,
                        int kW, int dH, int dW, float *gin, InputMask mask = InputMask());
 int threshold_fwd_launch(const float *in, float *out, long n, float th, float val);
@@ -44,7 +56,7 @@ struct OutputThreshold {
 };
 int conv_implicit_forward(const float *padded, const float *weight, const float *bias, float *output, long B, int C,
                           int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW,
-                          OutputThreshold act = OutputThreshold());
+                          OutputThreshold act = OutputThreshold(), OutputLayout out = OutputLayout());
 int conv_implicit_gradweight(const float *padded, const float *gradOutput, float *gradWeight, long B, int C, int H,
                              int W, int M, int kH, int kW, int pH, int pW, int sH, int sW, float scale);
 int conv_implicit_gradinput(const float *gradOutput, const float *weight, float *scratch, float *gradInput, long B,

@@ -87,77 +87,128 @@ int size_padded(THGPUTensor *t, const ConvShape &s, int padH, int padW) {
     return 0;
 }
 
+// An image tensor ([B,] C, H, W) whose rows are contiguous and whose planes follow each other at one fixed distance:
+// the dense layout (pitch == W, plane == H*W) or the interior of a larger buffer, e.g. one with a zero border.
+struct PlaneLayout {
+    long pitch = 0;  // floats between rows
+    long plane = 0;  // floats between planes; images are C planes apart
+    bool dense = false;
+};
+
+bool plane_layout(const THGPUTensor *t, PlaneLayout &l) {
+    if (!t || !(t->nDimension == 3 || t->nDimension == 4)) return false;
+    const int o = t->nDimension == 4 ? 1 : 0;
+    const long C = t->size[o], H = t->size[o + 1], W = t->size[o + 2];
+    if (C <= 0 || H <= 0 || W <= 0) return false;
+    if (W > 1 && t->stride[o + 2] != 1) return false;
+    l.pitch = H > 1 ? t->stride[o + 1] : W;
+    l.plane = C > 1 || o == 1 ? t->stride[o] : H * l.pitch;
+    if (C == 1 && o == 1 && t->size[0] > 1) l.plane = t->stride[0];  // single-plane images: the image stride is the plane's
+    if (l.pitch < W || l.plane < (H - 1) * l.pitch + W) return false;
+    if (o == 1 && t->size[0] > 1 && t->stride[0] != C * l.plane) return false;
+    l.dense = l.pitch == W && l.plane == H * W;
+    return tensor_backed(t);
+}
+
+// Whether `input` lies inside a buffer that keeps padH rows above and below and padW columns left and right of
+// every plane (the caller vouches for the zeros in them): then the buffer itself is the padded image.
+bool interior_of_padded(const THGPUTensor *input, const ConvShape &s, int padH, int padW, PlaneLayout &l) {
+    if (!plane_layout(input, l)) return false;
+    const long Hp = s.H + 2L * padH, Wp = s.W + 2L * padW;
+    if (l.pitch != Wp || l.plane != Hp * Wp) return false;
+    const long lead = (long)padH * Wp + padW;  // from the buffer's first element to the interior's
+    return input->storageOffset >= lead && input->storageOffset - lead + s.B * s.C * l.plane <= input->storage->size;
+}
+
+void set_output_layout(GemmProblem &p, const PlaneLayout &l, int planes_per_image, int width) {
+    p.sC = l.plane;
+    p.bsC = (long)planes_per_image * l.plane;
+    if (!l.dense) {
+        p.c_pitch = (int)l.pitch;
+        p.c_w = width;
+    }
+}
+
 int conv_update_output(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias, THGPUTensor *finput,
                        THGPUTensor *fgradInput, THGPUTensor *output, int kW, int kH, int dW, int dH, int padW,
-                       int padH, OutputThreshold act) {
+                       int padH, OutputThreshold act, bool input_in_padded_buffer) {
     (void)fgradInput;  // the reference uses it as a buffer of ones for the bias GEMM; the bias is fused here
     ConvShape s;
     if (conv_shape(s, input, weight, kW, kH, dW, dH, padW, padH)) return 1;
     if (!bias || !finput || !output) return fail("SpatialConvolutionMM: null tensor");
     if (THGPUTensor_nElement(bias) != s.M) return fail("SpatialConvolutionMM: bias must have nOutputPlane elements");
     if (require_contiguous(weight, "weight") || require_contiguous(bias, "bias")) return 1;
-    THGPUTensor *in = THGPUTensor_newContiguous(input);
-    if (!in) return 1;
+    PlaneLayout in_layout;
+    if (input_in_padded_buffer && !interior_of_padded(input, s, padH, padW, in_layout))
+        return fail("SpatialConvolutionMM: input is not the interior of a buffer padded by %d x %d", padH, padW);
 
     const bool gathered = conv_use_gathered(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW);
-    if (gathered) {
-        // finput holds the padded input instead of the columns
-        if (size_padded(finput, s, padH, padW)) {
-            THGPUTensor_free(in);
-            return 1;
+    const bool direct = gathered && input_in_padded_buffer;  // the input's own buffer is the padded image
+    THGPUTensor *in = direct ? nullptr : THGPUTensor_newContiguous(input);
+    if (!direct && !in) return 1;
+    struct Release {
+        THGPUTensor *t;
+        ~Release() {
+            if (t) THGPUTensor_free(t);
         }
+    } release{in};
+
+    if (direct) {
+        // finput is not needed: nothing is copied
+    } else if (gathered) {
+        // finput holds the padded input instead of the columns
+        if (size_padded(finput, s, padH, padW)) return 1;
     } else if (s.batched) {
         THGPUTensor_resize3d(finput, s.B, s.K, s.N);
     } else {
         THGPUTensor_resize2d(finput, s.K, s.N);
     }
+    // The output keeps the layout it comes with when it already has the right sizes: densely packed, or rows inside
+    // a larger buffer (the next layer's padded input).
     if (s.batched)
         THGPUTensor_resize4d(output, s.B, s.M, s.Ho, s.Wo);
     else
         THGPUTensor_resize3d(output, s.M, s.Ho, s.Wo);
-    int rc = 0;
-    if (!tensor_ready(finput, gathered ? s.B * s.C * (s.H + 2L * padH) * (s.W + 2L * padW) : s.B * s.K * s.N) ||
-        !tensor_ready(output, s.B * s.M * s.N))
-        rc = fail("SpatialConvolutionMM: could not size finput/output");
-    if (!rc && !(tensor_backed(in) && tensor_backed(weight) && tensor_backed(bias)))
-        rc = fail("SpatialConvolutionMM: a tensor's shape exceeds its storage");
+    PlaneLayout out_layout;
+    if (!plane_layout(output, out_layout) || THGPUTensor_nElement(output) != s.B * s.M * s.N)
+        return fail("SpatialConvolutionMM: could not size output");
+    if (!direct && !tensor_ready(finput, gathered ? s.B * s.C * (s.H + 2L * padH) * (s.W + 2L * padW) : s.B * s.K * s.N))
+        return fail("SpatialConvolutionMM: could not size finput");
+    if (!((direct || tensor_backed(in)) && tensor_backed(weight) && tensor_backed(bias)))
+        return fail("SpatialConvolutionMM: a tensor's shape exceeds its storage");
 
     if (gathered) {
-        if (!rc) rc = pad_planes_launch(dptr(in), s.B * s.C, s.H, s.W, padH, padW, dptr(finput));
-        if (!rc)
-            rc = conv_implicit_forward(dptr(finput), dptr(weight), dptr(bias), dptr(output), s.B, s.C, s.H, s.W, s.M, kH,
-                                       kW, padH, padW, dH, dW, act);
-        THGPUTensor_free(in);
-        return rc;
+        const float *padded = direct ? dptr(input) - ((long)padH * in_layout.pitch + padW) : dptr(finput);
+        if (!direct && pad_planes_launch(dptr(in), s.B * s.C, s.H, s.W, padH, padW, dptr(finput))) return 1;
+        OutputLayout ol;
+        ol.plane = out_layout.plane;
+        ol.pitch = out_layout.dense ? 0 : (int)out_layout.pitch;
+        return conv_implicit_forward(padded, dptr(weight), dptr(bias), dptr(output), s.B, s.C, s.H, s.W, s.M, kH, kW,
+                                     padH, padW, dH, dW, act, ol);
     }
-    if (!rc) rc = im2col_launch(dptr(in), s.B, s.C, s.H, s.W, kH, kW, padH, padW, dH, dW, dptr(finput));
-    if (!rc) {
-        // output[b][m][n] = bias[m] + sum_k weight[m][k] * finput[b][k][n]
-        GemmProblem p;
-        p.A = dptr(weight);
-        p.a_rc = true;
-        p.sA = s.K;
-        p.B = dptr(finput);
-        p.b_rc = false;
-        p.sB = s.N;
-        p.bsB = (long)s.K * s.N;
-        p.C = dptr(output);
-        p.sC = s.N;
-        p.bsC = (long)s.M * s.N;
-        p.bias = dptr(bias);
-        p.M = s.M;
-        p.J = (int)(s.B * s.N);
-        p.N = (int)s.N;
-        p.R = s.K;
-        p.tag = "gemm_conv_fwd";
-        p.flops = 2.0 * s.M * (double)s.N * s.K * s.B;
-        p.act = act.on;
-        p.act_threshold = act.threshold;
-        p.act_value = act.value;
-        rc = gemm_launch(p);
-    }
-    THGPUTensor_free(in);
-    return rc;
+    if (im2col_launch(dptr(in), s.B, s.C, s.H, s.W, kH, kW, padH, padW, dH, dW, dptr(finput))) return 1;
+    // output[b][m][n] = bias[m] + sum_k weight[m][k] * finput[b][k][n]
+    GemmProblem p;
+    p.A = dptr(weight);
+    p.a_rc = true;
+    p.sA = s.K;
+    p.B = dptr(finput);
+    p.b_rc = false;
+    p.sB = s.N;
+    p.bsB = (long)s.K * s.N;
+    p.C = dptr(output);
+    set_output_layout(p, out_layout, s.M, s.Wo);
+    p.bias = dptr(bias);
+    p.M = s.M;
+    p.J = (int)(s.B * s.N);
+    p.N = (int)s.N;
+    p.R = s.K;
+    p.tag = "gemm_conv_fwd";
+    p.flops = 2.0 * s.M * (double)s.N * s.K * s.B;
+    p.act = act.on;
+    p.act_threshold = act.threshold;
+    p.act_value = act.value;
+    return gemm_launch(p);
 }
 
 // mask_on: gradInput is zeroed where `input` does not exceed mask_threshold.
@@ -170,19 +221,29 @@ int conv_update_grad_input(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTen
     if (!gradOutput || !fgradInput || !gradInput) return fail("SpatialConvolutionMM: null tensor");
     if (check_grad_output(s, gradOutput)) return 1;
     if (require_contiguous(weight, "weight")) return 1;
+    const bool gathered = conv_use_gathered_gradinput(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW);
     THGPUTensor *go = THGPUTensor_newContiguous(gradOutput);
     if (!go) return 1;
-    // The mask reads `input` element for element beside gradInput, so it needs the dense layout.
-    THGPUTensor *in = mask_on ? THGPUTensor_newContiguous(input) : nullptr;
-    if (mask_on && (!in || !tensor_backed(in))) {
-        if (in) THGPUTensor_free(in);
-        THGPUTensor_free(go);
-        return fail("SpatialConvolutionMM: input is not usable as a mask");
-    }
+    // The mask is `input`, read element for element beside gradInput.  The gathered product's store takes it in
+    // any regular plane layout (dense, or the interior of a padded buffer); col2im wants it dense.
+    PlaneLayout mask_layout;
+    THGPUTensor *in = nullptr;
     InputMask mask;
     if (mask_on) {
-        mask.in = dptr(in);
+        if (gathered && plane_layout(input, mask_layout)) {
+            mask.in = dptr(input);
+        } else {
+            in = THGPUTensor_newContiguous(input);
+            if (!in || !plane_layout(in, mask_layout)) {
+                if (in) THGPUTensor_free(in);
+                THGPUTensor_free(go);
+                return fail("SpatialConvolutionMM: input is not usable as a mask");
+            }
+            mask.in = dptr(in);
+        }
         mask.threshold = mask_threshold;
+        mask.plane = mask_layout.plane;
+        mask.pitch = mask_layout.dense ? 0 : (int)mask_layout.pitch;
     }
     struct Release {  // frees the contiguous copies on every return path
         THGPUTensor *a, *b;
@@ -192,7 +253,7 @@ int conv_update_grad_input(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTen
         }
     } release{go, in};
 
-    if (conv_use_gathered_gradinput(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW)) {
+    if (gathered) {
         // fgradInput holds the padded gradOutput and the flipped kernels instead of the gradient columns
         const long need = conv_implicit_gradinput_scratch(s.B, s.C, s.H, s.W, s.M, kH, kW);
         if (s.batched)
@@ -200,15 +261,12 @@ int conv_update_grad_input(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTen
         else
             THGPUTensor_resize3d(gradInput, s.C, s.H, s.W);
         THGPUTensor_resize1d(fgradInput, need);
-        int rc = 0;
         if (!tensor_ready(fgradInput, need) || !tensor_ready(gradInput, s.B * (long)s.C * s.H * s.W))
-            rc = fail("SpatialConvolutionMM: could not size gradInput/fgradInput");
-        if (!rc && !(tensor_backed(go) && tensor_backed(weight)))
-            rc = fail("SpatialConvolutionMM: a tensor's shape exceeds its storage");
-        if (!rc)
-            rc = conv_implicit_gradinput(dptr(go), dptr(weight), dptr(fgradInput), dptr(gradInput), s.B, s.C, s.H, s.W,
-                                         s.M, kH, kW, padH, padW, mask);
-        return rc;
+            return fail("SpatialConvolutionMM: could not size gradInput/fgradInput");
+        if (!(tensor_backed(go) && tensor_backed(weight)))
+            return fail("SpatialConvolutionMM: a tensor's shape exceeds its storage");
+        return conv_implicit_gradinput(dptr(go), dptr(weight), dptr(fgradInput), dptr(gradInput), s.B, s.C, s.H, s.W,
+                                       s.M, kH, kW, padH, padW, mask);
     }
     if (s.batched) {
         THGPUTensor_resize4d(gradInput, s.B, s.C, s.H, s.W);
@@ -217,13 +275,11 @@ int conv_update_grad_input(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTen
         THGPUTensor_resize3d(gradInput, s.C, s.H, s.W);
         THGPUTensor_resize2d(fgradInput, s.K, s.N);
     }
-    int rc = 0;
     if (!tensor_ready(fgradInput, s.B * s.K * s.N) || !tensor_ready(gradInput, s.B * (long)s.C * s.H * s.W))
-        rc = fail("SpatialConvolutionMM: could not size gradInput/fgradInput");
-    if (!rc && !(tensor_backed(go) && tensor_backed(weight)))
-        rc = fail("SpatialConvolutionMM: a tensor's shape exceeds its storage");
-
-    if (!rc) {
+        return fail("SpatialConvolutionMM: could not size gradInput/fgradInput");
+    if (!(tensor_backed(go) && tensor_backed(weight)))
+        return fail("SpatialConvolutionMM: a tensor's shape exceeds its storage");
+    {
         // fgradInput[b][k][n] = sum_m weight[m][k] * gradOutput[b][m][n]
         GemmProblem p;
         p.A = dptr(weight);
@@ -242,55 +298,14 @@ int conv_update_grad_input(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTen
         p.R = s.M;
         p.tag = "gemm_conv_gradinput";
         p.flops = 2.0 * s.M * (double)s.N * s.K * s.B;
-        rc = gemm_launch(p);
+        if (gemm_launch(p)) return 1;
     }
-    if (!rc)
-        rc = col2im_launch(dptr(fgradInput), s.B, s.C, s.H, s.W, kH, kW, padH, padW, dH, dW, dptr(gradInput), mask);
-    return rc;
+    return col2im_launch(dptr(fgradInput), s.B, s.C, s.H, s.W, kH, kW, padH, padW, dH, dW, dptr(gradInput), mask);
 }
 
-}  // namespace
-
-extern "C" {
-
-int thgpu_SpatialConvolutionMM_updateOutput(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias,
-                                            THGPUTensor *finput, THGPUTensor *fgradInput, THGPUTensor *output,
-                                            int kW, int kH, int dW, int dH, int padW, int padH) {
-    return conv_update_output(input, weight, bias, finput, fgradInput, output, kW, kH, dW, dH, padW, padH,
-                              OutputThreshold());
-}
-
-int thgpu_SpatialConvolutionMM_updateOutputThreshold(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias,
-                                                     THGPUTensor *finput, THGPUTensor *fgradInput,
-                                                     THGPUTensor *output, int kW, int kH, int dW, int dH, int padW,
-                                                     int padH, float threshold, float val) {
-    OutputThreshold act;
-    act.on = true;
-    act.threshold = threshold;
-    act.value = val;
-    return conv_update_output(input, weight, bias, finput, fgradInput, output, kW, kH, dW, dH, padW, padH, act);
-}
-
-int thgpu_SpatialConvolutionMM_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *weight,
-                                               THGPUTensor *finput, THGPUTensor *fgradInput,
-                                               THGPUTensor *gradInput, int kW, int kH, int dW, int dH, int padW,
-                                               int padH) {
-    return conv_update_grad_input(input, gradOutput, weight, finput, fgradInput, gradInput, kW, kH, dW, dH, padW,
-                                  padH, false, 0.0f);
-}
-
-int thgpu_SpatialConvolutionMM_updateGradInputMasked(THGPUTensor *input, THGPUTensor *gradOutput,
-                                                     THGPUTensor *weight, THGPUTensor *finput,
-                                                     THGPUTensor *fgradInput, THGPUTensor *gradInput, int kW, int kH,
-                                                     int dW, int dH, int padW, int padH, float threshold) {
-    return conv_update_grad_input(input, gradOutput, weight, finput, fgradInput, gradInput, kW, kH, dW, dH, padW,
-                                  padH, true, threshold);
-}
-
-int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor *gradOutput,
-                                                 THGPUTensor *gradWeight, THGPUTensor *gradBias,
-                                                 THGPUTensor *finput, THGPUTensor *fgradInput, int kW, int kH,
-                                                 int dW, int dH, int padW, int padH, float scale) {
+int conv_acc_grad_parameters(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *gradWeight,
+                             THGPUTensor *gradBias, THGPUTensor *finput, THGPUTensor *fgradInput, int kW, int kH, int dW,
+                             int dH, int padW, int padH, float scale, bool input_in_padded_buffer) {
     (void)fgradInput;
     ConvShape s;
     if (!gradWeight || !gradBias || !finput || !gradOutput) return fail("SpatialConvolutionMM: null tensor");
@@ -298,46 +313,59 @@ int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor
     if (check_grad_output(s, gradOutput)) return 1;
     if (THGPUTensor_nElement(gradBias) != s.M) return fail("SpatialConvolutionMM: gradBias must have nOutputPlane elements");
     if (require_contiguous(gradWeight, "gradWeight") || require_contiguous(gradBias, "gradBias")) return 1;
+    PlaneLayout in_layout;
+    if (input_in_padded_buffer && !interior_of_padded(input, s, padH, padW, in_layout))
+        return fail("SpatialConvolutionMM: input is not the interior of a buffer padded by %d x %d", padH, padW);
+    const bool gathered = conv_use_gathered(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW);
+    const bool direct = gathered && input_in_padded_buffer;
     THGPUTensor *go = THGPUTensor_newContiguous(gradOutput);
     if (!go) return 1;
-    int rc = 0;
-    THGPUTensor *in = THGPUTensor_newContiguous(input);
-    if (!in) {
+    THGPUTensor *in = direct ? nullptr : THGPUTensor_newContiguous(input);
+    if (!direct && !in) {
         THGPUTensor_free(go);
         return 1;
     }
-    if (!(tensor_backed(in) && tensor_backed(go) && tensor_backed(gradWeight) && tensor_backed(gradBias)))
-        rc = fail("SpatialConvolutionMM: a tensor's shape exceeds its storage");
+    struct Release {
+        THGPUTensor *a, *b;
+        ~Release() {
+            if (a) THGPUTensor_free(a);
+            if (b) THGPUTensor_free(b);
+        }
+    } release{go, in};
+    if (!((direct || tensor_backed(in)) && tensor_backed(go) && tensor_backed(gradWeight) && tensor_backed(gradBias)))
+        return fail("SpatialConvolutionMM: a tensor's shape exceeds its storage");
     // finput is rebuilt from `input` on every call, as the reference GPU code does
     // (gpunn-impl/SpatialConvolutionMM.cpp:388-396): the result then depends on the arguments alone,
     // whatever input the last forward pass saw and whoever else shares the buffer.  With
     // thgpu_conv_set_finput_reuse(1) a finput of the right shape is taken to be the forward's, as the CPU
-    // module takes it (mcw_nn/generic/SpatialConvolutionMM.c:318,336).
+    // module takes it (mcw_nn/generic/SpatialConvolutionMM.c:318,336).  An input that lies in its own padded
+    // buffer needs neither: the gathered product reads it there.
     const bool reuse = g_finput_reuse;
-    if (!rc && conv_use_gathered(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW)) {
-        // finput holds the padded input
-        if (!(reuse && is_padded(finput, s, padH, padW) && tensor_backed(finput))) {
-            rc = size_padded(finput, s, padH, padW);
-            if (!rc) rc = pad_planes_launch(dptr(in), s.B * s.C, s.H, s.W, padH, padW, dptr(finput));
+    if (gathered) {
+        const float *padded;
+        if (direct) {
+            padded = dptr(input) - ((long)padH * in_layout.pitch + padW);
+        } else {
+            if (!(reuse && is_padded(finput, s, padH, padW) && tensor_backed(finput))) {
+                if (size_padded(finput, s, padH, padW)) return 1;
+                if (pad_planes_launch(dptr(in), s.B * s.C, s.H, s.W, padH, padW, dptr(finput))) return 1;
+            }
+            padded = dptr(finput);
         }
-        if (!rc)
-            rc = conv_implicit_gradweight(dptr(finput), dptr(go), dptr(gradWeight), s.B, s.C, s.H, s.W, s.M, kH, kW,
-                                          padH, padW, dH, dW, scale);
-        if (!rc) rc = gradbias_launch(dptr(go), dptr(gradBias), s.B, s.M, s.N, scale);
-        THGPUTensor_free(in);
-        THGPUTensor_free(go);
-        return rc;
+        if (conv_implicit_gradweight(padded, dptr(go), dptr(gradWeight), s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH,
+                                     dW, scale))
+            return 1;
+        return gradbias_launch(dptr(go), dptr(gradBias), s.B, s.M, s.N, scale);
     }
-    if (!rc && !(reuse && is_columns(finput, s) && tensor_backed(finput))) {
+    if (!(reuse && is_columns(finput, s) && tensor_backed(finput))) {
         if (s.batched)
             THGPUTensor_resize3d(finput, s.B, s.K, s.N);
         else
             THGPUTensor_resize2d(finput, s.K, s.N);
-        if (!tensor_ready(finput, s.B * s.K * s.N)) rc = fail("SpatialConvolutionMM: could not size finput");
-        if (!rc) rc = im2col_launch(dptr(in), s.B, s.C, s.H, s.W, kH, kW, padH, padW, dH, dW, dptr(finput));
+        if (!tensor_ready(finput, s.B * s.K * s.N)) return fail("SpatialConvolutionMM: could not size finput");
+        if (im2col_launch(dptr(in), s.B, s.C, s.H, s.W, kH, kW, padH, padW, dH, dW, dptr(finput))) return 1;
     }
-    THGPUTensor_free(in);
-    if (!rc) {
+    {
         // gradWeight[m][k] += scale * sum_b sum_n gradOutput[b][m][n] * finput[b][k][n]
         GemmProblem p;
         p.A = dptr(go);
@@ -359,11 +387,74 @@ int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor
         p.beta = 1.0f;
         p.tag = "gemm_conv_gradweight";
         p.flops = 2.0 * s.M * (double)s.N * s.K * s.B;
-        rc = gemm_launch(p);
+        if (gemm_launch(p)) return 1;
     }
-    if (!rc) rc = gradbias_launch(dptr(go), dptr(gradBias), s.B, s.M, s.N, scale);
-    THGPUTensor_free(go);
-    return rc;
+    return gradbias_launch(dptr(go), dptr(gradBias), s.B, s.M, s.N, scale);
+}
+
+}  // namespace
+
+extern "C" {
+
+int thgpu_SpatialConvolutionMM_updateOutput(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias,
+                                            THGPUTensor *finput, THGPUTensor *fgradInput, THGPUTensor *output,
+                                            int kW, int kH, int dW, int dH, int padW, int padH) {
+    return conv_update_output(input, weight, bias, finput, fgradInput, output, kW, kH, dW, dH, padW, padH,
+                              OutputThreshold(), false);
+}
+
+int thgpu_SpatialConvolutionMM_updateOutputFused(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias,
+                                                 THGPUTensor *finput, THGPUTensor *fgradInput, THGPUTensor *output,
+                                                 int kW, int kH, int dW, int dH, int padW, int padH, int flags,
+                                                 float threshold, float val) {
+    if (flags & ~(THGPU_FUSE_THRESHOLD | THGPU_INPUT_IN_PADDED_BUFFER)) return fail("SpatialConvolutionMM: unknown flags");
+    OutputThreshold act;
+    act.on = (flags & THGPU_FUSE_THRESHOLD) != 0;
+    act.threshold = threshold;
+    act.value = val;
+    return conv_update_output(input, weight, bias, finput, fgradInput, output, kW, kH, dW, dH, padW, padH, act,
+                              (flags & THGPU_INPUT_IN_PADDED_BUFFER) != 0);
+}
+
+int thgpu_SpatialConvolutionMM_updateGradInput(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *weight,
+                                               THGPUTensor *finput, THGPUTensor *fgradInput,
+                                               THGPUTensor *gradInput, int kW, int kH, int dW, int dH, int padW,
+                                               int padH) {
+    return conv_update_grad_input(input, gradOutput, weight, finput, fgradInput, gradInput, kW, kH, dW, dH, padW,
+                                  padH, false, 0.0f);
+}
+
+int thgpu_SpatialConvolutionMM_updateGradInputFused(THGPUTensor *input, THGPUTensor *gradOutput,
+                                                    THGPUTensor *weight, THGPUTensor *finput,
+                                                    THGPUTensor *fgradInput, THGPUTensor *gradInput, int kW, int kH,
+                                                    int dW, int dH, int padW, int padH, int flags, float threshold) {
+    if (flags & ~THGPU_FUSE_INPUT_MASK) return fail("SpatialConvolutionMM: unknown flags");
+    return conv_update_grad_input(input, gradOutput, weight, finput, fgradInput, gradInput, kW, kH, dW, dH, padW,
+                                  padH, (flags & THGPU_FUSE_INPUT_MASK) != 0, threshold);
+}
+
+int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor *gradOutput,
+                                                 THGPUTensor *gradWeight, THGPUTensor *gradBias,
+                                                 THGPUTensor *finput, THGPUTensor *fgradInput, int kW, int kH,
+                                                 int dW, int dH, int padW, int padH, float scale) {
+    return conv_acc_grad_parameters(input, gradOutput, gradWeight, gradBias, finput, fgradInput, kW, kH, dW, dH, padW,
+                                    padH, scale, false);
+}
+
+int thgpu_SpatialConvolutionMM_accGradParametersFused(THGPUTensor *input, THGPUTensor *gradOutput,
+                                                      THGPUTensor *gradWeight, THGPUTensor *gradBias,
+                                                      THGPUTensor *finput, THGPUTensor *fgradInput, int kW, int kH,
+                                                      int dW, int dH, int padW, int padH, float scale, int flags) {
+    if (flags & ~THGPU_INPUT_IN_PADDED_BUFFER) return fail("SpatialConvolutionMM: unknown flags");
+    return conv_acc_grad_parameters(input, gradOutput, gradWeight, gradBias, finput, fgradInput, kW, kH, dW, dH, padW,
+                                    padH, scale, (flags & THGPU_INPUT_IN_PADDED_BUFFER) != 0);
+}
+
+int thgpu_conv_gathers(long B, int C, int H, int W, int M, int kW, int kH, int dW, int dH, int padW, int padH) {
+    if (B <= 0 || C <= 0 || H <= 0 || W <= 0 || M <= 0 || kW <= 0 || kH <= 0 || dW <= 0 || dH <= 0 || padW < 0 ||
+        padH < 0 || H + 2 * padH < kH || W + 2 * padW < kW)
+        return 0;
+    return conv_use_gathered(B, C, H, W, M, kH, kW, padH, padW, dH, dW) ? 1 : 0;
 }
 
 int thgpu_SpatialMaxPooling_updateOutput(THGPUTensor *input, THGPUTensor *output, THGPUTensor *indices, int kW,
@@ -387,10 +478,16 @@ int thgpu_SpatialMaxPooling_updateOutput(THGPUTensor *input, THGPUTensor *output
         THGPUTensor_resize3d(output, C, Ho, Wo);
         THGPUTensor_resize4d(indices, 2, C, Ho, Wo);
     }
+    // The output keeps the layout it comes with when it already has the right sizes: densely packed, or rows inside
+    // a larger buffer (the next layer's padded input).
     int rc = 0;
-    if (!tensor_ready(output, B * C * Ho * Wo) || !tensor_ready(indices, 2 * B * C * Ho * Wo) || !tensor_backed(in))
+    PlaneLayout ol;
+    if (!plane_layout(output, ol) || THGPUTensor_nElement(output) != B * C * Ho * Wo ||
+        !tensor_ready(indices, 2 * B * C * Ho * Wo) || !tensor_backed(in))
         rc = fail("SpatialMaxPooling: could not size output/indices");
-    if (!rc) rc = maxpool_fwd_launch(dptr(in), B * C, H, W, kH, kW, dH, dW, dptr(output), dptr(indices));
+    if (!rc)
+        rc = maxpool_fwd_launch(dptr(in), B * C, H, W, kH, kW, dH, dW, dptr(output), dptr(indices), ol.plane,
+                                (int)ol.pitch);
     THGPUTensor_free(in);
     return rc;
 }

@@ -32,6 +32,8 @@ namespace {
 
 struct PoolGeom {
     int H, W, Ho, Wo, kH, kW, dH, dW;
+    long oplane;  // floats between the forward output's planes and rows (Ho*Wo and Wo when densely packed)
+    int opitch;
     FastDiv divWo, divHoWo, divW, divHW, divDH, divDW;
 };
 
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(256) void maxpool_fwd_direct_kernel(const float *__
             }
         }
     }
-    out[o] = best;
+    out[(long)plane * g.oplane + (long)i * g.opitch + j] = best;
     // A window of NaNs never updates the maximum; the CPU code then stores
     // (int)(-1 / kW) + 1 and (-1 % kW) + 1, i.e. (1, 0).
     indy[o] = by < 0 ? 1.0f : (float)(by + 1);
@@ -583,7 +585,7 @@ __global__ __launch_bounds__(256) void gradbias_final_kernel(const float *__rest
 }  // namespace
 
 int maxpool_fwd_launch(const float *in, long planes, int H, int W, int kH, int kW, int dH, int dW, float *out,
-                       float *indices) {
+                       float *indices, long out_plane, int out_pitch) {
     hipStream_t s = stream();
     if (!s) return 1;
     PoolGeom g;
@@ -599,9 +601,14 @@ int maxpool_fwd_launch(const float *in, long planes, int H, int W, int kH, int k
     g.divW = FastDiv((uint32_t)W);
     g.divHW = FastDiv((uint32_t)(H * W));
     const double bytes = 4.0 * (planes * (double)H * W + 3.0 * total);
+    const bool dense_out = (out_plane == 0 || out_plane == (long)g.Ho * g.Wo) && (out_pitch == 0 || out_pitch == g.Wo);
+    g.oplane = dense_out ? (long)g.Ho * g.Wo : out_plane;
+    g.opitch = dense_out ? g.Wo : out_pitch;
+    if (!dense_out && (out_pitch < g.Wo || out_plane < (long)(g.Ho - 1) * out_pitch + g.Wo))
+        return fail("SpatialMaxPooling: output planes overlap");
     PoolFwdPlan plan;
-    // The pool_fwd_wave switch selects the wavefront-level tile kernel where its plan applies.
-    if (tuning().pool_fwd_wave && plan_pool_fwd(g, planes, plan)) {
+    // The pool_fwd_wave switch selects the wavefront-level tile kernel where its plan applies (dense outputs only).
+    if (tuning().pool_fwd_wave && dense_out && plan_pool_fwd(g, planes, plan)) {
         const long blocks = ((planes + plan.G - 1) / plan.G) * plan.strips;
         if (blocks < (1L << 31)) {
             const long rows = plan.G > 1 ? H : (long)(plan.SR - 1) * dH + kH;
@@ -695,6 +702,8 @@ int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int
     if (!s) return 1;
     PoolGeom g;
     g.H = H; g.W = W; g.kH = kH; g.kW = kW; g.dH = dH; g.dW = dW; g.Ho = Ho; g.Wo = Wo;
+    g.oplane = (long)Ho * Wo;
+    g.opitch = Wo;
     long total = planes * (long)H * W, ototal = planes * (long)Ho * Wo;
     if (total == 0) return 0;
     if (total >= (1L << 31)) return fail("SpatialMaxPooling: tensor too large for 32-bit indexing");

@@ -41,6 +41,25 @@ int fill_device(float *p, long n, float v) {
     return check_launch("fill");
 }
 
+// One launch that fills several buffers (a network's gradient tensors): entry e owns the virtual index range
+// [start[e], start[e+1]) of the concatenation.
+constexpr int kFillManyMax = 32;
+struct FillMany {
+    float *p[kFillManyMax];
+    long start[kFillManyMax + 1];
+    int count;
+};
+
+__global__ __launch_bounds__(256) void fill_many_kernel(const FillMany f, float v) {
+    const long total = f.start[f.count];
+    const long stride = (long)gridDim.x * blockDim.x;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        int e = 0;
+        while (i >= f.start[e + 1]) ++e;  // at most 32 ranges
+        f.p[e][i - f.start[e]] = v;
+    }
+}
+
 // Blocking host<->device copies: stage through the caller's pageable memory
 // with hipMemcpyAsync on the library stream, then drain the stream, which is
 // what a blocking clEnqueue{Read,Write}Buffer gave the reference's callers
@@ -260,3 +279,37 @@ THGPU_STORAGE_COPY_VIA_FLOAT(Long, long)
 THGPU_STORAGE_COPY_VIA_FLOAT(Double, double)
 
 }  // extern "C"
+
+extern "C" int thgpu_fill_many(THGPUTensor **tensors, int count, float value) {
+    if (count < 0 || (count > 0 && !tensors)) return fail("thgpu_fill_many: invalid arguments");
+    hipStream_t s = stream();
+    if (!s) return 1;
+    for (int i = 0; i < count; ++i) {  // every tensor is checked before anything is launched
+        THGPUTensor *t = tensors[i];
+        if (!t) return fail("thgpu_fill_many: null tensor");
+        if (THGPUTensor_nElement(t) > 0 && (!THGPUTensor_isContiguous(t) || !tensor_backed(t)))
+            return fail("thgpu_fill_many: tensor %d is not contiguous or exceeds its storage", i);
+    }
+    for (int first = 0; first < count; first += kFillManyMax) {
+        FillMany f;
+        f.count = 0;
+        f.start[0] = 0;
+        for (int i = first; i < count && i < first + kFillManyMax; ++i) {
+            const long n = THGPUTensor_nElement(tensors[i]);
+            if (n == 0) continue;
+            f.p[f.count] = THGPUTensor_data(tensors[i]);
+            f.start[f.count + 1] = f.start[f.count] + n;
+            ++f.count;
+        }
+        const long total = f.start[f.count];
+        if (total == 0) continue;
+        long blocks = (total + 255) / 256;
+        if (blocks > 4096) blocks = 4096;
+        {
+            LaunchScope scope("fill", 0.0, 4.0 * total);
+            hipLaunchKernelGGL(fill_many_kernel, dim3((unsigned)blocks), dim3(256), 0, s, f, value);
+        }
+        if (check_launch("fill")) return 1;
+    }
+    return 0;
+}

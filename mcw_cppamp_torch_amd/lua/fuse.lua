@@ -9,9 +9,54 @@ gpunn = gpunn or {}
 local function isa(m, name) return torch.typename(m) == name end
 local function threshold(m) return isa(m, 'nn.Threshold') or isa(m, 'nn.ReLU') end
 
+-- The layer in front of a convolution that gathers from its padded input writes that padded image itself: before
+-- every forward pass its `output` is made a view into a zero-bordered buffer of the right size (the operators leave an
+-- output that already has the right sizes as it is), and the convolution is told so (inputInPaddedBuffer).
+local function output_sizes(m, input)
+   local n = input:dim()
+   local H, W = input:size(n - 1), input:size(n)
+   if isa(m, 'nn.SpatialConvolutionMM') then
+      local pW, pH = m.padW or m.padding, m.padH or m.padding
+      return m.nOutputPlane, math.floor((H + 2 * pH - m.kH) / m.dH) + 1, math.floor((W + 2 * pW - m.kW) / m.dW) + 1
+   end
+   return input:size(n - 2), math.floor((H - m.kH) / m.dH) + 1, math.floor((W - m.kW) / m.dW) + 1
+end
+
+local function link(producer, consumer)
+   local class_updateOutput = producer.updateOutput
+   producer.updateOutput = function(self, input)
+      local C, H, W = output_sizes(self, input)
+      local B = input:dim() == 4 and input:size(1) or 1
+      local pW, pH = consumer.padW or consumer.padding, consumer.padH or consumer.padding
+      local want = (pW > 0 or pH > 0) and H > 0 and W > 0 and thgpu.convGathers(B, C, H, W, consumer.nOutputPlane,
+                   consumer.kW, consumer.kH, consumer.dW, consumer.dH, pW, pH)
+      if want then
+         local b = self.paddedOutput
+         if not (b and b:dim() == input:dim() and b:size(b:dim()) == W + 2 * pW and b:size(b:dim() - 1) == H + 2 * pH
+                 and b:size(b:dim() - 2) == C and (input:dim() == 3 or b:size(1) == B)) then
+            b = input:dim() == 4 and input.new(B, C, H + 2 * pH, W + 2 * pW) or input.new(C, H + 2 * pH, W + 2 * pW)
+            b:zero()
+            self.paddedOutput = b
+            self.output = b:narrow(b:dim() - 1, pH + 1, H):narrow(b:dim(), pW + 1, W)
+         end
+         consumer.inputInPaddedBuffer = true
+      else
+         if self.paddedOutput then self.output = input.new(); self.paddedOutput = nil end
+         consumer.inputInPaddedBuffer = nil
+      end
+      return class_updateOutput(self, input)
+   end
+   producer.linkedConsumer = consumer
+end
+
 function gpunn.unfuse(net)
    for _, m in ipairs(net.modules) do
       if m.modules then gpunn.unfuse(m) end
+      if m.linkedConsumer then
+         m.linkedConsumer.inputInPaddedBuffer = nil
+         m.linkedConsumer, m.updateOutput = nil, nil
+         if m.paddedOutput then m.output = m.output.new(); m.paddedOutput = nil end
+      end
       if threshold(m) and (m.fusedForward or m.fusedBackward) then
          m.output = m.output.new()
          m.gradInput = m.gradInput.new()
@@ -39,6 +84,13 @@ function gpunn.fuse(net)
             m.fusedBackward = true
             m.updateGradInput = function(self, input, gradOutput) self.gradInput = gradOutput; return gradOutput end
          end
+      end
+   end
+   for i, m in ipairs(mods) do
+      if isa(m, 'nn.SpatialConvolutionMM') or isa(m, 'nn.SpatialMaxPooling') then
+         local j = i + 1
+         if mods[j] and threshold(mods[j]) and mods[j].fusedForward then j = j + 1 end
+         if mods[j] and isa(mods[j], 'nn.SpatialConvolutionMM') then link(m, mods[j]) end
       end
    end
    return net

@@ -15,6 +15,8 @@
 //                     applied as the output is stored
 //   inputThreshold    set by gpunn.fuse(net) on a convolution / max-pooling layer preceded by nn.Threshold: gradInput
 //                     is zeroed where the input is not above it
+//   inputInPaddedBuffer   set by gpunn.fuse(net) while the layer's input is a view into a zero-bordered buffer that
+//                     the layer in front writes (lua/fuse.lua): the gathered convolution reads it there
 extern "C" {
 #include <lua.h>
 #include <lauxlib.h>
@@ -72,10 +74,12 @@ PoolFields pool_fields(lua_State *L) {
 int conv_updateOutput(lua_State *L) {
     THGPUTensor *input = arg(L, 2);
     const ConvFields f = conv_fields(L);
-    if (has_field(L, "fusedThreshold"))
-        fail(L, thgpu_SpatialConvolutionMM_updateOutputThreshold(
+    const int flags = (has_field(L, "fusedThreshold") ? THGPU_FUSE_THRESHOLD : 0) |
+                      (has_field(L, "inputInPaddedBuffer") ? THGPU_INPUT_IN_PADDED_BUFFER : 0);
+    if (flags)
+        fail(L, thgpu_SpatialConvolutionMM_updateOutputFused(
                     input, field(L, "weight"), field(L, "bias"), field(L, "finput"), field(L, "fgradInput"),
-                    field(L, "output"), f.kW, f.kH, f.dW, f.dH, f.padW, f.padH,
+                    field(L, "output"), f.kW, f.kH, f.dW, f.dH, f.padW, f.padH, flags,
                     static_cast<float>(opt_number(L, "fusedThreshold", 0)), static_cast<float>(opt_number(L, "fusedValue", 0))));
     else
         fail(L, thgpu_SpatialConvolutionMM_updateOutput(input, field(L, "weight"), field(L, "bias"), field(L, "finput"),
@@ -87,9 +91,9 @@ int conv_updateGradInput(lua_State *L) {
     THGPUTensor *input = arg(L, 2), *gradOutput = arg(L, 3);
     const ConvFields f = conv_fields(L);
     if (has_field(L, "inputThreshold"))
-        fail(L, thgpu_SpatialConvolutionMM_updateGradInputMasked(
+        fail(L, thgpu_SpatialConvolutionMM_updateGradInputFused(
                     input, gradOutput, field(L, "weight"), field(L, "finput"), field(L, "fgradInput"),
-                    field(L, "gradInput"), f.kW, f.kH, f.dW, f.dH, f.padW, f.padH,
+                    field(L, "gradInput"), f.kW, f.kH, f.dW, f.dH, f.padW, f.padH, THGPU_FUSE_INPUT_MASK,
                     static_cast<float>(opt_number(L, "inputThreshold", 0))));
     else
         fail(L, thgpu_SpatialConvolutionMM_updateGradInput(input, gradOutput, field(L, "weight"), field(L, "finput"),
@@ -101,9 +105,10 @@ int conv_accGradParameters(lua_State *L) {
     THGPUTensor *input = arg(L, 2), *gradOutput = arg(L, 3);
     const float scale = static_cast<float>(luaL_optnumber(L, 4, 1));  // SpatialConvolutionMM.cpp:326
     const ConvFields f = conv_fields(L);
-    fail(L, thgpu_SpatialConvolutionMM_accGradParameters(input, gradOutput, field(L, "gradWeight"), field(L, "gradBias"),
-                                                         field(L, "finput"), field(L, "fgradInput"), f.kW, f.kH, f.dW,
-                                                         f.dH, f.padW, f.padH, scale));
+    fail(L, thgpu_SpatialConvolutionMM_accGradParametersFused(
+                input, gradOutput, field(L, "gradWeight"), field(L, "gradBias"), field(L, "finput"), field(L, "fgradInput"),
+                f.kW, f.kH, f.dW, f.dH, f.padW, f.padH, scale,
+                has_field(L, "inputInPaddedBuffer") ? THGPU_INPUT_IN_PADDED_BUFFER : 0));
     return 0;
 }
 
@@ -214,8 +219,16 @@ const struct luaL_Reg kOps[] = {
 int l_synchronize(lua_State *L) { return fail(L, thgpu_synchronize()); }
 int l_conv_mode(lua_State *L) { return fail(L, thgpu_conv_set_mode(static_cast<int>(luaL_checkinteger(L, 1)))); }
 int l_finput_reuse(lua_State *L) { return fail(L, thgpu_conv_set_finput_reuse(lua_toboolean(L, 1))); }
-const struct luaL_Reg kLib[] = {
-    {"synchronize", l_synchronize}, {"setConvMode", l_conv_mode}, {"setFinputReuse", l_finput_reuse}, {NULL, NULL}};
+int l_conv_gathers(lua_State *L) {  // (B, C, H, W, M, kW, kH, dW, dH, padW, padH)
+    int a[10];
+    for (int i = 0; i < 10; ++i) a[i] = static_cast<int>(luaL_checkinteger(L, i + 2));
+    lua_pushboolean(L, thgpu_conv_gathers(static_cast<long>(luaL_checkinteger(L, 1)), a[0], a[1], a[2], a[3], a[4], a[5],
+                                          a[6], a[7], a[8], a[9]));
+    return 1;
+}
+const struct luaL_Reg kLib[] = {{"synchronize", l_synchronize},    {"setConvMode", l_conv_mode},
+                                {"setFinputReuse", l_finput_reuse}, {"convGathers", l_conv_gathers},
+                                {NULL, NULL}};
 
 void lua_error_handler(const char *msg, void *data) { luaL_error(static_cast<lua_State *>(data), "%s", msg); }
 

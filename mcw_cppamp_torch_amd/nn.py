@@ -188,8 +188,20 @@ class Sequential(Module):
         self.modules[0].accUpdateGradParameters(input, cur, lr)
 
     def zeroGradParameters(self):
-        for m in self.modules:
-            m.zeroGradParameters()
+        # mcw_nn/Sequential.lua:85-89 zeroes module by module; the dense GPU gradients of all modules go in one launch
+        _, grads = self.parameters()
+        gpu = [g for g in grads or [] if isinstance(g, GPUTensor) and g.isContiguous()]
+        if len(gpu) > 1:
+            arr = (_lib.TensorP * len(gpu))(*[g._p for g in gpu])
+            _lib.check_status(lib.thgpu_fill_many(arr, len(gpu), 0.0))
+        else:
+            gpu = []
+        for g in grads or []:
+            if isinstance(g, GPUTensor):
+                if not any(g is h for h in gpu):
+                    g.zero()
+            else:
+                g[...] = 0
 
     def fuse(self):
         """Lets the neighbours of every nn.Threshold / nn.ReLU do its work while they store their own results: a
@@ -212,6 +224,16 @@ class Sequential(Module):
             if i + 1 < len(mods) and isinstance(mods[i + 1], (SpatialConvolutionMM, SpatialMaxPooling)):
                 mods[i + 1].inputThreshold = m.threshold
                 m.fusedBackward = True
+        # A convolution or pooling layer whose output reaches a convolution unchanged (directly, or through a
+        # Threshold the convolution in front applies itself) writes it into that convolution's padded image.
+        for i, m in enumerate(mods):
+            if not isinstance(m, (SpatialConvolutionMM, SpatialMaxPooling)):
+                continue
+            j = i + 1
+            if j < len(mods) and isinstance(mods[j], Threshold) and mods[j].fusedForward:
+                j += 1
+            if j < len(mods) and isinstance(mods[j], SpatialConvolutionMM):
+                m._consumer = mods[j]
         return self
 
     def unfuse(self):
@@ -226,6 +248,10 @@ class Sequential(Module):
                 m.fusedThreshold = m.inputThreshold = None
             elif isinstance(m, SpatialMaxPooling):
                 m.inputThreshold = None
+            if isinstance(m, (SpatialConvolutionMM, SpatialMaxPooling)):
+                m._consumer = None
+                if getattr(m.output, "_zero_border", None) is not None:
+                    m.output = type(m.output)()
         return self
 
     def updateParameters(self, learningRate):
@@ -256,6 +282,40 @@ class Sequential(Module):
     def reset(self, stdv=None):
         for m in self.modules:
             m.reset(stdv)
+
+
+def _padded_output(module, sizes):
+    """Gives `module.output` the `sizes` it is about to be resized to, as the interior of a zero-bordered buffer,
+    when the convolution that consumes it (module._consumer, set by Sequential.fuse) gathers from its padded input
+    at this size: the producer then writes the consumer's padded image itself and no copy of it is ever made.  The
+    view carries the border it sits in as `_zero_border`; consumers trust no tensor without that mark."""
+    consumer = getattr(module, "_consumer", None)
+    out = module.output
+    if consumer is not None and isinstance(out, GPUTensor):
+        B = sizes[0] if len(sizes) == 4 else 1
+        C, H, W = sizes[-3:]
+        pH, pW = consumer.padH, consumer.padW
+        if (pH or pW) and C == consumer.nInputPlane and lib.thgpu_conv_gathers(
+                B, C, H, W, consumer.nOutputPlane, consumer.kW, consumer.kH, consumer.dW, consumer.dH, pW, pH):
+            if getattr(out, "_zero_border", None) == (pH, pW) and tuple(out.size()) == tuple(sizes):
+                return
+            buf = GPUTensor(*(tuple(sizes[:-2]) + (H + 2 * pH, W + 2 * pW)))
+            buf.zero()
+            nd = len(sizes)
+            view = buf.narrow(nd - 2, pH, H).narrow(nd - 1, pW, W)
+            view._zero_border = (pH, pW)
+            view._padded_buffer = buf
+            module.output = view
+            return
+    if getattr(out, "_zero_border", None) is not None:
+        module.output = GPUTensor()      # back to a tensor of its own
+
+
+def _in_padded_buffer(input, padH, padW):
+    """Whether `input` may be handed to a convolution as lying in its own zero-bordered buffer."""
+    if (padH, padW) == (0, 0):
+        return isinstance(input, GPUTensor) and input.isContiguous()
+    return getattr(input, "_zero_border", None) == (padH, padW)
 
 
 class SpatialConvolutionMM(Module):
@@ -311,10 +371,19 @@ class SpatialConvolutionMM(Module):
 
     def updateOutput(self, input):
         _require_gpu(input, self.weight, self.bias, self.finput, self.fgradInput, self.output)
-        if self.fusedThreshold is not None:
-            _lib.check_status(lib.thgpu_SpatialConvolutionMM_updateOutputThreshold(
+        if getattr(self, "_consumer", None) is not None or getattr(self.output, "_zero_border", None) is not None:
+            sz = input.size()
+            if len(sz) in (3, 4):
+                Ho = (sz[-2] + 2 * self.padH - self.kH) // self.dH + 1
+                Wo = (sz[-1] + 2 * self.padW - self.kW) // self.dW + 1
+                if Ho > 0 and Wo > 0:
+                    _padded_output(self, tuple(sz[:-3]) + (self.nOutputPlane, Ho, Wo))
+        flags = (1 if self.fusedThreshold is not None else 0) | (2 if _in_padded_buffer(input, self.padH, self.padW) else 0)
+        if flags:
+            th, val = self.fusedThreshold if self.fusedThreshold is not None else (0.0, 0.0)
+            _lib.check_status(lib.thgpu_SpatialConvolutionMM_updateOutputFused(
                 input._p, self.weight._p, self.bias._p, self.finput._p, self.fgradInput._p, self.output._p,
-                *(self._geom() + (float(self.fusedThreshold[0]), float(self.fusedThreshold[1])))))
+                *(self._geom() + (flags, float(th), float(val)))))
             return self.output
         _lib.check_status(lib.thgpu_SpatialConvolutionMM_updateOutput(
             input._p, self.weight._p, self.bias._p, self.finput._p, self.fgradInput._p, self.output._p,
@@ -326,9 +395,9 @@ class SpatialConvolutionMM(Module):
             return None
         _require_gpu(input, gradOutput, self.weight, self.finput, self.fgradInput, self.gradInput)
         if self.inputThreshold is not None:
-            _lib.check_status(lib.thgpu_SpatialConvolutionMM_updateGradInputMasked(
+            _lib.check_status(lib.thgpu_SpatialConvolutionMM_updateGradInputFused(
                 input._p, gradOutput._p, self.weight._p, self.finput._p, self.fgradInput._p, self.gradInput._p,
-                *(self._geom() + (float(self.inputThreshold),))))
+                *(self._geom() + (1, float(self.inputThreshold)))))
             return self.gradInput
         _lib.check_status(lib.thgpu_SpatialConvolutionMM_updateGradInput(
             input._p, gradOutput._p, self.weight._p, self.finput._p, self.fgradInput._p, self.gradInput._p,
@@ -337,6 +406,11 @@ class SpatialConvolutionMM(Module):
 
     def accGradParameters(self, input, gradOutput, scale=1):
         _require_gpu(input, gradOutput, self.gradWeight, self.gradBias, self.finput, self.fgradInput)
+        if _in_padded_buffer(input, self.padH, self.padW):
+            _lib.check_status(lib.thgpu_SpatialConvolutionMM_accGradParametersFused(
+                input._p, gradOutput._p, self.gradWeight._p, self.gradBias._p, self.finput._p, self.fgradInput._p,
+                *(self._geom() + (float(scale), 2))))
+            return
         _lib.check_status(lib.thgpu_SpatialConvolutionMM_accGradParameters(
             input._p, gradOutput._p, self.gradWeight._p, self.gradBias._p, self.finput._p, self.fgradInput._p,
             *(self._geom() + (float(scale),))))
@@ -425,6 +499,12 @@ class SpatialMaxPooling(Module):
 
     def updateOutput(self, input):
         _require_gpu(input, self.output, self.indices)
+        if getattr(self, "_consumer", None) is not None or getattr(self.output, "_zero_border", None) is not None:
+            sz = input.size()
+            if len(sz) in (3, 4):
+                Ho, Wo = (sz[-2] - self.kH) // self.dH + 1, (sz[-1] - self.kW) // self.dW + 1
+                if Ho > 0 and Wo > 0:
+                    _padded_output(self, tuple(sz[:-2]) + (Ho, Wo))
         _lib.check_status(lib.thgpu_SpatialMaxPooling_updateOutput(
             input._p, self.output._p, self.indices._p, self.kW, self.kH, self.dW, self.dH))
         return self.output

@@ -83,6 +83,17 @@ def test_fused_stack_is_bit_identical_to_unfused(gt, mode):
         for (gw_u, gb_u), (gw_f, gb_f) in zip(grads_u, grads_f):
             assert np.array_equal(bits(gw_u), bits(gw_f)) and np.array_equal(bits(gb_u), bits(gb_f))
         assert (out_u == 0).mean() > 0.2                # the threshold did bite
+        # in gathered mode the layers in front of a padded convolution wrote that convolution's padded image themselves
+        marks = [getattr(m.output, "_zero_border", None) for m in net_f.modules]
+        if mode == 2:
+            assert marks[2] == (1, 1) and marks[3] == (1, 1) and marks[7] == (2, 2), marks   # pool1, conv2 (+ReLU), pool2
+            assert marks[4] is marks[3] or marks[4] == (1, 1)                                 # the fused ReLU passes it on
+            buf = net_f.modules[2].output._padded_buffer.float()
+            assert not buf[:, :, 0, :].any() and not buf[:, :, -1, :].any() and not buf[:, :, :, 0].any() \
+                and not buf[:, :, :, -1].any()                                                # the border is still zero
+            assert np.array_equal(bits(buf[:, :, 1:-1, 1:-1]), bits(outs_u[2]))
+        else:
+            assert marks == [None] * len(marks)
         # unfuse() restores the separate passes
         net_f.unfuse()
         assert not any(t.fusedForward or t.fusedBackward for t in thr)
@@ -171,3 +182,33 @@ def test_full_size_alexnet_fused_equals_unfused(gt):
     assert np.array_equal(bits(out_u), bits(out_f)) and np.array_equal(bits(gi_u), bits(gi_f))
     for (gw_u, gb_u), (gw_f, gb_f) in zip(gr_u, gr_f):
         assert np.array_equal(bits(gw_u), bits(gw_f)) and np.array_equal(bits(gb_u), bits(gb_f))
+
+
+def test_padded_buffer_claims_are_checked_and_a_column_route_producer_can_feed_a_gathering_consumer(gt):
+    lib, L = gt._lib.lib, gt._lib
+    nn = gt.nn
+    # the flag is refused for a tensor that does not lie in a buffer of the claimed geometry
+    conv = nn.SpatialConvolutionMM(64, 64, 3, 3, 1, 1, 1).gpu()
+    x = dev(gt, uniform(rng_for(96), (2, 64, 9, 9)))
+    rc = lib.thgpu_SpatialConvolutionMM_updateOutputFused(x._p, conv.weight._p, conv.bias._p, conv.finput._p,
+                                                          conv.fgradInput._p, conv.output._p, 3, 3, 1, 1, 1, 1, 2, 0.0, 0.0)
+    assert rc != 0 and b"not the interior" in lib.thgpu_last_error()
+    assert lib.thgpu_SpatialConvolutionMM_updateOutputFused(x._p, conv.weight._p, conv.bias._p, conv.finput._p,
+                                                            conv.fgradInput._p, conv.output._p, 3, 3, 1, 1, 1, 1, 8, 0.0, 0.0) != 0
+    assert lib.thgpu_conv_gathers(2, 64, 9, 9, 64, 3, 3, 1, 1, 1, 1) == (1 if lib.thgpu_conv_get_mode() != 0 else 0)
+    assert lib.thgpu_conv_gathers(2, 3, 9, 9, 64, 3, 3, 1, 1, 1, 1) == 0      # K = 27: no tile
+    # mode 1: a 600-plane producer stays on columns, its 64-plane consumer gathers from the producer's padded output
+    before = lib.thgpu_conv_get_mode()
+    assert lib.thgpu_conv_set_mode(1) == 0
+    try:
+        spec = [("conv", 16, 600, 3, 1, 1), ("relu",), ("conv", 600, 64, 3, 1, 1), ("relu",), ("pool", 2, 2)]
+        xx = uniform(rng_for(97), (2, 16, 12, 14))
+        net_u, out_u, gi_u, outs_u, grads_u, go = run(gt, spec, xx, 98, False)
+        net_f, out_f, gi_f, outs_f, grads_f, _ = run(gt, spec, xx, 98, True, go)
+        assert net_f.modules[0].finput.dim() == 3 and net_f.modules[0].output._zero_border == (1, 1)
+        assert net_f.modules[2].finput.nElement() == 0               # nothing copied
+        assert np.array_equal(bits(out_u), bits(out_f)) and np.array_equal(bits(gi_u), bits(gi_f))
+        for (gw_u, gb_u), (gw_f, gb_f) in zip(grads_u, grads_f):
+            assert np.array_equal(bits(gw_u), bits(gw_f)) and np.array_equal(bits(gb_u), bits(gb_f))
+    finally:
+        assert lib.thgpu_conv_set_mode(before) == 0

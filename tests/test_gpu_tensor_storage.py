@@ -295,3 +295,33 @@ def test_storage_write_read_binary_and_ascii_known_answers(gt):
         gt.gputorch.GPUStorage().read(io.BytesIO(struct.pack("<q", 4) + b"\0" * 8))
     with pytest.raises(gt._lib.THGPUError):
         gt.gputorch.GPUStorage().read(io.BytesIO(b"3\n1 2\n"), binary=False)
+
+
+def test_fill_many_fills_every_tensor_in_one_call_and_rejects_views(gt):
+    import ctypes
+    L = gt._lib
+    sizes = [(3, 5), (1,), (0,), (129, 7), (64, 363), (4097,)] + [(i + 1,) for i in range(40)]     # more than one launch's 32
+    tensors = [gt.GPUTensor(*s) if s != (0,) else gt.GPUTensor() for s in sizes]
+    for t in tensors:
+        t.fill(7.0)
+    guard = gt.GPUTensor(16)
+    guard.fill(3.0)
+    arr = (L.TensorP * len(tensors))(*[t._p for t in tensors])
+    L.check_status(L.lib.thgpu_fill_many(arr, len(tensors), -1.5))
+    for s, t in zip(sizes, tensors):
+        if s != (0,):
+            assert np.array_equal(t.float(), np.full(s, -1.5, np.float32)), s
+    assert np.array_equal(guard.float(), np.full(16, 3.0, np.float32))
+    view = tensors[3].narrow(1, 1, 3)                       # not contiguous: rejected before anything is written
+    arr2 = (L.TensorP * 2)(tensors[0]._p, view._p)
+    assert L.lib.thgpu_fill_many(arr2, 2, 9.0) != 0 and b"not contiguous" in L.lib.thgpu_last_error()
+    assert np.array_equal(tensors[0].float(), np.full((3, 5), -1.5, np.float32))
+    # nn.Sequential:zeroGradParameters goes through it
+    nn = gt.nn
+    net = nn.Sequential().add(nn.SpatialConvolutionMM(3, 4, 3, 3)).add(nn.ReLU()).add(nn.SpatialConvolutionMM(4, 5, 3, 3)).gpu()
+    for m in (net.get(0), net.get(2)):
+        m.gradWeight.fill(2.0)
+        m.gradBias.fill(2.0)
+    net.zeroGradParameters()
+    for m in (net.get(0), net.get(2)):
+        assert not m.gradWeight.float().any() and not m.gradBias.float().any()
