@@ -37,6 +37,7 @@ Other modes
   --workload ref_benchmark   the reference's own micro-benchmark (gpunn/test/benchmark.lua:7-91): seven single
                              layers, updateOutput / updateGradInput / accGradParameters timed separately and
                              reported with its GFLOP/s formula (:118).
+  --workload hbm_sweep       GB/s of the HBM-bound kernels at the stack's geometries as the launch size grows.
   --summarise kernel-trace|traffic|mfma ...   turns rocprofv3 CSV output into the text summaries kept under
                              profiles/ (see summarise()).
 """
@@ -209,6 +210,78 @@ def ref_benchmark(args, pkg):
         "layers": rows}))
 
 
+def hbm_sweep(args, pkg):
+    """GB/s of the HBM-bound kernels at the AlexNet-style stack's geometries as the batch, and with it the size of a
+    launch, grows from 32 to 2048 images: what a launch of 10-60 us loses to its ramp-up shows as the gap between
+    the batch-128 figure and the large-batch one.  HIP-event time per launch, algorithmic bytes as in `kernels`."""
+    import numpy as np
+
+    from mcw_cppamp_torch_amd import gputorch, nn
+
+    lib = pkg._lib.lib
+    rng = np.random.default_rng(0)
+
+    def dev(shape):
+        return pkg.FloatTensor(rng.uniform(-1, 1, shape).astype(np.float32)).gpu()
+
+    def timed(fn, n):
+        for _ in range(2):
+            fn()
+        gputorch.synchronize()
+        gputorch.prof_reset()
+        gputorch.prof_enable(True)
+        for _ in range(n):
+            fn()
+        gputorch.synchronize()
+        rep = gputorch.prof_report()
+        gputorch.prof_enable(False)
+        gputorch.prof_reset()
+        return {k: r for k, r in rep.items() if r["bytes"] > 0 and not k.startswith("gemm_conv")}
+
+    rows = []
+
+    def record(rep, geometry, batch):
+        for kn, r in sorted(rep.items()):
+            rows.append({"kernel": kn.split(" ")[0], "geometry": geometry, "batch": batch,
+                         "mb_per_launch": round(r["bytes"] / r["calls"] / 1e6, 1),
+                         "us": round(r["ms"] / r["calls"] * 1e3, 1), "gbs": round(r["bytes"] / r["ms"] / 1e6),
+                         "frac": round(r["bytes"] / r["ms"] / 1e6 / PEAK_HBM_GBS, 3)})
+
+    for C, H, k, s in ((64, 55, 3, 2), (192, 27, 3, 2), (256, 13, 3, 2)):
+        for B in (32, 128, 512, 2048):
+            x = dev((B, C, H, H))
+            m = nn.SpatialMaxPooling(k, k, s, s).gpu()
+            o = m.forward(x)
+            go = dev(o.size())
+            m.inputThreshold = 0.0       # the backward of a ReLU in front is applied as gradInput is stored
+            record(timed(lambda: (m.forward(x), m.updateGradInput(x, go)), args.steps),
+                   "%dx%dx%d k%d s%d" % (C, H, H, k, s), B)
+            del x, o, go, m
+    lib.thgpu_conv_set_mode(ROUTES["auto"])
+    for conv, shape, label in (((3, 64, 11, 11, 4, 4, 2), (3, 224, 224), "conv 3->64 224x224 k11 s4 p2"),
+                               ((256, 256, 3, 3, 1, 1, 1), (256, 13, 13), "conv 256->256 13x13 k3 p1")):
+        for B in (32, 128, 512):
+            m = nn.SpatialConvolutionMM(*conv).gpu()
+            x = dev((B,) + shape)
+            o = m.forward(x)
+            go = dev(o.size())
+            record(timed(lambda: (m.forward(x), m.updateGradInput(x, go), m.accGradParameters(x, go)),
+                         max(2, args.steps // 4)), label, B)
+            del m, x, o, go
+    print(json.dumps({
+        "metric": "GB/s of the HBM-bound kernels against launch size", "value": max(r["gbs"] for r in rows),
+        "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": 2, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "pooling forward / masked backward, pad, col2im, gradBias, split reduction at the "
+                               "AlexNet-style geometries, batch 32 .. 2048"}, "rows": rows}))
+    if args.table:
+        print("%-18s %-30s %6s %10s %9s %8s %6s" % ("kernel", "geometry", "batch", "MB/launch", "us", "GB/s", "frac"),
+              file=sys.stderr)
+        for r in rows:
+            print("%-18s %-30s %6d %10.1f %9.1f %8d %6.3f" % (r["kernel"], r["geometry"], r["batch"], r["mb_per_launch"],
+                                                             r["us"], r["gbs"], r["frac"]), file=sys.stderr)
+
+
 # ---- rocprofv3 output -> the text summaries under profiles/ ----------------------------------------------------------
 
 def _short(name):
@@ -330,7 +403,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="alexnet",
-                    choices=["alexnet", "overfeat", "vgg_a", "conv1_b16", "ref_benchmark"])
+                    choices=["alexnet", "overfeat", "vgg_a", "conv1_b16", "ref_benchmark", "hbm_sweep"])
+    ap.add_argument("--table", action="store_true", help="hbm_sweep: also print the rows as a table on stderr")
     ap.add_argument("--batch", type=int, default=None, help="override the workload's batch size")
     ap.add_argument("--cpu-sample-batch", type=int, default=128)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -364,6 +438,8 @@ def main():
     lib.thgpu_conv_set_finput_reuse(1 if args.reuse_finput else 0)
     if args.workload == "ref_benchmark":
         return ref_benchmark(args, pkg)
+    if args.workload == "hbm_sweep":
+        return hbm_sweep(args, pkg)
 
     name = args.workload
     B = args.batch or stacks.STACKS[name]["batch"]
