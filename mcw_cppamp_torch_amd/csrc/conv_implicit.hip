@@ -12,6 +12,17 @@
 // padded gradOutput with the flipped kernels.  The sums run over the same products as
 // gpunn-impl/SpatialConvolutionMM.cpp:110-429 (im2col + sgemm + col2im), in a different order for
 // gradInput.
+//
+// gradInput of a strided layer, by residue class of the pixel coordinates: write h + padH = dH*y + ph and
+// w + padW = dW*x + pw.  Pixel (h, w) only meets the taps kh = ph + dH*a, kw = pw + dW*b, through the output
+// positions (y - a, x - b), so each of the dH*dW classes is a unit-stride correlation of gradOutput with a
+// sub-sampled kernel of at most A x Bk = ceil(kH/dH) x ceil(kW/dW) taps:
+//   gradInput[b][c][h][w] = sum_{m,a,b} weight[m][c][ph + dH*a][pw + dW*b] * gradOutput[b][m][y - a][x - b].
+// One GEMM does all classes: row (c, ph, pw), reduction index (m, a, b) (taps beyond the kernel carry zero
+// weights), column (image, y, x), second operand gathered from gradOutput padded by (A-1, Bk-1), and a
+// scattered store (GemmProblem::scatter) that puts element ((c,ph,pw), (y,x)) at pixel (dH*y+ph-padH,
+// dW*x+pw-padW).  No zero-dilated gradOutput, no column buffer, no col2im; the work is that of the layer's
+// other products times (A*dH/kH)*(Bk*dW/kW) (taps rounded up to whole strides).
 #include "gemm_mfma.h"
 #include "kernels.h"
 
@@ -65,6 +76,25 @@ __global__ __launch_bounds__(256) void flip_weight_kernel(const float *__restric
     const unsigned m = cm % M, c = cm / M;
     const unsigned kh = tap / kW, kw = tap % kW;
     wt[idx] = w[((long)m * C + c) * kk + (kH - 1 - kh) * kW + (kW - 1 - kw)];
+}
+
+// wt[(c, ph, pw)][(m, a', b')] = w[m][c][ph + sH*(A-1-a')][pw + sW*(Bk-1-b')], zero where that tap lies outside the
+// kernel and in the rows beyond C*sH*sW (the product's rows are padded to a whole tile).
+__global__ __launch_bounds__(256) void phase_weight_kernel(const float *__restrict__ w, float *__restrict__ wt, int M,
+                                                           int C, int kH, int kW, int sH, int sW, int A, int Bk,
+                                                           int rows, int rows_pad) {
+    const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+    const unsigned R = (unsigned)(M * A * Bk);
+    if (idx >= (unsigned)rows_pad * R) return;
+    const unsigned row = idx / R, r = idx % R;
+    float v = 0.0f;
+    if (row < (unsigned)rows) {
+        const unsigned pw = row % sW, ph = (row / sW) % sH, c = row / (sW * sH);
+        const unsigned bb = r % Bk, aa = (r / Bk) % A, m = r / (Bk * A);
+        const unsigned kh = ph + sH * (A - 1 - aa), kw = pw + sW * (Bk - 1 - bb);
+        if (kh < (unsigned)kH && kw < (unsigned)kW) v = w[(((long)m * C + c) * kH + kh) * kW + kw];
+    }
+    wt[idx] = v;
 }
 
 // t[(c, kh, kw)] = c*plane + kh*pitch + kw
@@ -208,6 +238,56 @@ GemmProblem gradinput_problem(long B, int C, int H, int W, int M, int kH, int kW
     return p;
 }
 
+// Geometry of a strided layer's gradInput product (see the top of the file).
+struct PhaseGeom {
+    int A, Bk;     // taps per residue class: ceil(kH/sH), ceil(kW/sW)
+    int Yn, Xn;    // cells per image: y = (h + pH) / sH over the image rows, likewise x
+    int Hq, Wq;    // gradOutput padded by (A-1, Bk-1) in front and up to Yn + A - 1, Xn + Bk - 1 behind
+    int rows, rows_pad;
+};
+
+PhaseGeom phase_geom(int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW) {
+    PhaseGeom q;
+    q.A = (kH + sH - 1) / sH;
+    q.Bk = (kW + sW - 1) / sW;
+    q.Yn = (H - 1 + pH) / sH + 1;
+    q.Xn = (W - 1 + pW) / sW + 1;
+    q.Hq = q.Yn + q.A - 1;
+    q.Wq = q.Xn + q.Bk - 1;
+    q.rows = C * sH * sW;
+    q.rows_pad = q.rows < 64 ? 64 : q.rows;
+    return q;
+}
+
+GemmProblem gradinput_strided_problem(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH,
+                                      int sW) {
+    const PhaseGeom q = phase_geom(C, H, W, kH, kW, pH, pW, sH, sW);
+    const int Ho = (H + 2 * pH - kH) / sH + 1, Wo = (W + 2 * pW - kW) / sW + 1;
+    GemmProblem p;
+    p.a_rc = true;
+    p.sA = (long)M * q.A * q.Bk;
+    p.rowtab = p.coltab = &kNoTable;
+    p.bsB = (long)M * q.Hq * q.Wq;
+    p.b_extent = B * p.bsB;
+    p.bsC = (long)C * H * W;
+    p.M = q.rows_pad;
+    p.J = (int)(B * q.Yn * q.Xn);
+    p.N = q.Yn * q.Xn;
+    p.R = M * q.A * q.Bk;
+    p.c_w = q.Xn;
+    p.scatter = true;
+    p.scat_sH = sH;
+    p.scat_sW = sW;
+    p.scat_pH = pH;
+    p.scat_pW = pW;
+    p.scat_H = H;
+    p.scat_W = W;
+    p.scat_rows = q.rows;
+    p.flops = 2.0 * M * (double)Ho * Wo * C * kH * kW * B;
+    p.tag = "gemm_conv_gradinput";
+    return p;
+}
+
 }  // namespace
 
 int conv_mode() {
@@ -233,7 +313,16 @@ static bool forward_fits(long B, int C, int H, int W, int M, int kH, int kW, int
 }
 
 static bool gradinput_fits(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
-    if (sH != 1 || sW != 1 || kH - 1 - pH < 0 || kW - 1 - pW < 0) return false;
+    if (sH != 1 || sW != 1) {
+        // by residue class of the pixel coordinates: any padding, rows padded to a whole tile
+        const PhaseGeom q = phase_geom(C, H, W, kH, kW, pH, pW, sH, sW);
+        const long cols = B * (long)q.Yn * q.Xn;
+        if (!(cols >= 64 && cols < (1L << 31) && (long)M * q.A * q.Bk >= 16 && B * M * (long)q.Hq * q.Wq < kMaxExtent &&
+              (long)q.rows_pad * cols < (1L << 31)))
+            return false;
+        return gemm_tiled_fits(gradinput_strided_problem(B, C, H, W, M, kH, kW, pH, pW, sH, sW));
+    }
+    if (kH - 1 - pH < 0 || kW - 1 - pW < 0) return false;
     const long Hq = H + kH - 1, Wq = W + kW - 1;
     if (!(C >= 64 && B * H * W >= 64 && (long)M * kH * kW >= 16 && B * M * Hq * Wq < kMaxExtent &&
           B * (long)H * W < (1L << 31)))
@@ -256,30 +345,48 @@ bool conv_use_gathered(long B, int C, int H, int W, int M, int kH, int kW, int p
 bool conv_use_gathered_gradinput(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
     const int mode = conv_mode();
     if (mode == 0 || !gradinput_fits(B, C, H, W, M, kH, kW, pH, pW, sH, sW)) return false;
+    if (mode == 2) return true;
+    if (sH != 1 || sW != 1) {
+        // The product by residue class executes rows_pad*A*Bk*sH*sW / (C*kH*kW) times the layer's flops (rows
+        // padded to a tile, taps rounded up to whole strides) but saves the gradient columns, kH*kW/(sH*sW) times
+        // the input written and read back: it pays while that excess stays small.
+        const PhaseGeom q = phase_geom(C, H, W, kH, kW, pH, pW, sH, sW);
+        const double excess = (double)q.rows_pad * q.A * q.Bk / ((double)C * kH * kW);
+        return M < 512 && excess <= 2.0;
+    }
     const long rows = (C + 63L) / 64 * 64;
-    return mode == 2 || (M < 512 && rows * 8 <= C * 9L);
+    return M < 512 && rows * 8 <= C * 9L;
 }
 
-long conv_implicit_gradinput_scratch(long B, int C, int H, int W, int M, int kH, int kW) {
+long conv_implicit_gradinput_scratch(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH,
+                                     int sW) {
+    if (sH != 1 || sW != 1) {
+        const PhaseGeom q = phase_geom(C, H, W, kH, kW, pH, pW, sH, sW);
+        return B * M * (long)q.Hq * q.Wq + (long)q.rows_pad * M * q.A * q.Bk;
+    }
     return B * M * (H + kH - 1L) * (W + kW - 1L) + (long)C * M * kH * kW;
 }
 
-int pad_planes_launch(const float *in, long planes, int H, int W, int pH, int pW, float *out) {
+// out[plane][y][x] = in[plane][y - top][x - left], zero outside the H x W source; out planes are Hp x Wp.
+static int pad_planes_into(const float *in, long planes, int H, int W, int top, int left, long Hp, long Wp, float *out) {
     hipStream_t s = stream();
     if (!s) return 1;
-    const long Hp = H + 2L * pH, Wp = W + 2L * pW;
     const long total = planes * Hp * Wp;
     if (total <= 0) return 0;
     if (total >= (1L << 31)) return fail("pad: %ld elements exceed 32-bit indexing", total);
     {
-        const char *label = prof_enabled() ? prof_label("pad_planes planes=%ld %dx%d p=%dx%d", planes, H, W, pH, pW)
+        const char *label = prof_enabled() ? prof_label("pad_planes planes=%ld %dx%d p=%dx%d", planes, H, W, top, left)
                                            : "pad_planes";
         LaunchScope scope(label, 0.0, 4.0 * (total + planes * H * W));
         hipLaunchKernelGGL(pad_planes_kernel, dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0, s, in, out,
-                           (unsigned)total, H, W, pH, pW, (int)Hp, (int)Wp, FastDiv((uint32_t)Wp),
+                           (unsigned)total, H, W, top, left, (int)Hp, (int)Wp, FastDiv((uint32_t)Wp),
                            FastDiv((uint32_t)Hp), (reinterpret_cast<uintptr_t>(out) & 15) == 0);
     }
     return check_launch("pad_planes");
+}
+
+int pad_planes_launch(const float *in, long planes, int H, int W, int pH, int pW, float *out) {
+    return pad_planes_into(in, planes, H, W, pH, pW, H + 2L * pH, W + 2L * pW, out);
 }
 
 int conv_implicit_forward(const float *padded, const float *weight, const float *bias, float *output, long B, int C,
@@ -326,8 +433,45 @@ int conv_implicit_gradweight(const float *padded, const float *gradOutput, float
     return gemm_launch(p);
 }
 
+// gradInput of a strided layer as one product over the residue classes of the pixel coordinates.
+static int conv_implicit_gradinput_strided(const float *gradOutput, const float *weight, float *scratch,
+                                           float *gradInput, long B, int C, int H, int W, int M, int kH, int kW, int pH,
+                                           int pW, int sH, int sW, InputMask mask) {
+    hipStream_t s = stream();
+    if (!s) return 1;
+    if (mask.in && (mask.pitch > 0 || (mask.plane > 0 && mask.plane != (long)H * W)))
+        return fail("SpatialConvolutionMM: the strided gradInput product takes a densely packed mask only");
+    const PhaseGeom q = phase_geom(C, H, W, kH, kW, pH, pW, sH, sW);
+    const int Ho = (H + 2 * pH - kH) / sH + 1, Wo = (W + 2 * pW - kW) / sW + 1;
+    float *Q = scratch;
+    float *Wt = scratch + B * M * (long)q.Hq * q.Wq;
+    if (pad_planes_into(gradOutput, B * M, Ho, Wo, q.A - 1, q.Bk - 1, q.Hq, q.Wq, Q)) return 1;
+    const long nw = (long)q.rows_pad * M * q.A * q.Bk;
+    if (nw >= (1L << 31)) return fail("SpatialConvolutionMM: kernel bank too large for the strided gradInput product");
+    {
+        LaunchScope scope("flip_weight", 0.0, 4.0 * (nw + (long)M * C * kH * kW));
+        hipLaunchKernelGGL(phase_weight_kernel, dim3((unsigned)((nw + 255) / 256)), dim3(256), 0, s, weight, Wt, M, C, kH,
+                           kW, sH, sW, q.A, q.Bk, q.rows, q.rows_pad);
+    }
+    if (check_launch("flip_weight")) return 1;
+    if (trim_tables()) return 1;
+    GemmProblem p = gradinput_strided_problem(B, C, H, W, M, kH, kW, pH, pW, sH, sW);
+    p.A = Wt;
+    p.B = Q;
+    p.rowtab = tap_table(M, q.A, q.Bk, q.Hq * q.Wq, q.Wq);
+    p.coltab = pixel_table(q.Yn, q.Xn, q.Wq, 1);
+    if (!p.rowtab || !p.coltab) return 1;
+    p.C = gradInput;
+    p.mask = mask.in;
+    p.mask_threshold = mask.threshold;
+    return gemm_launch(p);
+}
+
 int conv_implicit_gradinput(const float *gradOutput, const float *weight, float *scratch, float *gradInput, long B,
-                            int C, int H, int W, int M, int kH, int kW, int pH, int pW, InputMask mask) {
+                            int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW, InputMask mask) {
+    if (sH != 1 || sW != 1)
+        return conv_implicit_gradinput_strided(gradOutput, weight, scratch, gradInput, B, C, H, W, M, kH, kW, pH, pW, sH,
+                                               sW, mask);
     hipStream_t s = stream();
     if (!s) return 1;
     const int Ho = H + 2 * pH - kH + 1, Wo = W + 2 * pW - kW + 1;

@@ -151,7 +151,8 @@ GemmPlan plan_gemm(const GemmProblem &p, int steps_total) {
         if (force && std::strcmp(force, c.name) != 0) continue;
         if (!force && c.below_rows > 0 && p.M >= c.below_rows) continue;
         const long tiles = cdiv(p.M, c.bm) * cdiv(p.J, c.bn);
-        const int max_split = (int)(steps_total / 8 > 0 ? (steps_total / 8 < 256 ? steps_total / 8 : 256) : 1);
+        int max_split = (int)(steps_total / 8 > 0 ? (steps_total / 8 < 256 ? steps_total / 8 : 256) : 1);
+        if (p.scatter) max_split = 1;  // the scattered store has no partial-sum form
         for (int ns = 1; ns <= max_split; ++ns) {
             if (fsplit > 0 && ns != (fsplit < max_split ? fsplit : max_split)) continue;
             if (tiles * ns > 8L * cus * c.resident && ns > 1 && fsplit <= 0) break;
@@ -227,6 +228,22 @@ int gemm_launch(const GemmProblem &p) {
     g.mask_sC = p.mask_sC ? p.mask_sC : p.sC;
     g.mask_bsC = p.mask_bsC ? p.mask_bsC : p.bsC;
     g.divCW = FastDiv((uint32_t)g.c_w);
+    if (p.scatter) {
+        if (!gather || red || p.bias || p.beta != 0.0f || p.c_pitch || p.mask_pitch || p.c_w <= 0 || g.N % p.c_w != 0 ||
+            p.scat_sH <= 0 || p.scat_sW <= 0 || p.scat_H <= 0 || p.scat_W <= 0 || p.scat_rows <= 0 || p.scat_rows > p.M ||
+            p.scat_pH < 0 || p.scat_pW < 0)
+            return fail("gemm: a scattered store needs a gathered B, column batching, no bias and beta = 0");
+        g.scatter = 1;
+        g.scat_sH = p.scat_sH;
+        g.scat_sW = p.scat_sW;
+        g.scat_pH = p.scat_pH;
+        g.scat_pW = p.scat_pW;
+        g.scat_H = p.scat_H;
+        g.scat_W = p.scat_W;
+        g.scat_rows = p.scat_rows;
+        g.divScatS = FastDiv((uint32_t)(p.scat_sH * p.scat_sW));
+        g.divScatW = FastDiv((uint32_t)p.scat_sW);
+    }
     g.steps_per_img = (p.R + GEMM_BK - 1) / GEMM_BK;
     g.steps_total = g.steps_per_img * (red ? p.nb : 1);
     g.divSpi = FastDiv((uint32_t)(g.steps_per_img > 0 ? g.steps_per_img : 1));

@@ -415,7 +415,55 @@ __global__ __launch_bounds__(WGM *WGN * 64)
             }
         }
     };
+    // The scattered store (see GemmProblem::scatter): rows are (plane, row phase, column phase) triples, columns
+    // cells of a per-image grid; an element lands at a strided position of the image or is dropped.
+    auto write_scatter = [&]() {
+        const bool masked = g.mask != nullptr;
+        long cbase[TN];  // float offset of the cell's phase-(0,0) pixel; may lie before the image (pH, pW)
+        int hy[TN], wx[TN];
+        bool own[TN];
+#pragma unroll
+        for (int b = 0; b < TN; ++b) {
+            const int jg = j0 + wn * (TN * 32) + b * 32 + l32;
+            own[b] = jg >= own_j0;
+            unsigned im, n, y, x;
+            g.divN.divmod((unsigned)jg, im, n);
+            g.divCW.divmod(n, y, x);
+            hy[b] = (int)y * g.scat_sH - g.scat_pH;
+            wx[b] = (int)x * g.scat_sW - g.scat_pW;
+            cbase[b] = (long)im * g.bsC + (long)hy[b] * g.scat_W + wx[b];
+        }
+        const long plane = (long)g.scat_H * g.scat_W;
+#pragma unroll
+        for (int a = 0; a < TM; ++a) {
+            const int iu = i0 + wm * (TM * 32) + a * 32;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = iu + 8 * (v / 4) + (v % 4) + 4 * half;
+                if (row < own_i0 || row >= g.scat_rows) continue;
+                unsigned c, rem, ph, pw;
+                g.divScatS.divmod((unsigned)row, c, rem);
+                g.divScatW.divmod(rem, ph, pw);
+                const long roff = (long)c * plane + (long)ph * g.scat_W + pw;
+#pragma unroll
+                for (int b = 0; b < TN; ++b) {
+                    const int h = hy[b] + (int)ph, w = wx[b] + (int)pw;
+                    if (!own[b] || h < 0 || h >= g.scat_H || w < 0 || w >= g.scat_W) continue;
+                    const long off = cbase[b] + roff;
+                    float val = acc[a][b][v] * g.alpha;
+                    if (masked) val = g.mask[off] > g.mask_threshold ? val : 0.0f;
+                    g.C[off] = val;
+                }
+            }
+        }
+    };
     using std::integral_constant;
+    if constexpr (LB == LD_XC_GATHER && !RED) {
+        if (g.scatter) {
+            write_scatter();
+            return;
+        }
+    }
     if (g.nsplit > 1) {
         if (edge_tile) write_out(integral_constant<int, 0>{}, integral_constant<bool, true>{});
         else write_out(integral_constant<int, 0>{}, integral_constant<bool, false>{});

@@ -57,6 +57,15 @@ struct GemmProblem {
     // (0: those of C).
     int c_w = 0, c_pitch = 0, mask_pitch = 0;
     long mask_sC = 0, mask_bsC = 0;
+    // Scattered store (column batching, no bias, beta = 0, never split): row i of the product is a (plane, row
+    // phase, column phase) triple, i = (c*scat_sH + ph)*scat_sW + pw, column n of an image a cell (y, x) of a grid
+    // c_w wide, and element (i, (image, y, x)) goes to
+    //     C[image*bsC + c*scat_H*scat_W + h*scat_W + w],   h = y*scat_sH + ph - scat_pH,  w = x*scat_sW + pw - scat_pW,
+    // when 0 <= h < scat_H, 0 <= w < scat_W and i < scat_rows; every other element is dropped.  This is how the
+    // gradInput of a strided convolution leaves its GEMM: one row per residue class of the pixel coordinates modulo
+    // the strides.  A mask is read at the same offsets (it is laid out exactly like C).  sC is unused.
+    bool scatter = false;
+    int scat_sH = 1, scat_sW = 1, scat_pH = 0, scat_pW = 0, scat_H = 0, scat_W = 0, scat_rows = 0;
     const char *tag = "gemm";     // name used by per-kernel timing
     // Flops the per-kernel timing credits the launch with; 0 means the product's own 2*M*J*R*nb.  A
     // convolution pass sets its algorithmic 2*M*N*K*B here, which a gathered gradInput product (one
@@ -104,6 +113,9 @@ struct GemmArgs {
     int c_w, c_pitch, mask_pitch;
     long mask_sC, mask_bsC;
     FastDiv divCW;
+    int scatter;  // see GemmProblem
+    int scat_sH, scat_sW, scat_pH, scat_pW, scat_H, scat_W, scat_rows;
+    FastDiv divScatS, divScatW;  // a row index by sH*sW and its remainder by sW
 };
 
 // Workgroups are handed to the 8 XCDs round-robin by linear id.  Remap so that

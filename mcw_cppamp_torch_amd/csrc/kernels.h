@@ -46,7 +46,8 @@ int conv_mode();
 void conv_set_mode(int mode);
 bool conv_use_gathered(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW);
 bool conv_use_gathered_gradinput(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW);
-long conv_implicit_gradinput_scratch(long B, int C, int H, int W, int M, int kH, int kW);
+long conv_implicit_gradinput_scratch(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH,
+                                     int sW);
 int pad_planes_launch(const float *in, long planes, int H, int W, int pH, int pW, float *out);
 // `act` applies nn.Threshold (threshold, value) to the output as it is stored; `mask` zeroes gradInput where the
 // convolution's input does not exceed a threshold (the backward of a Threshold in front of the convolution).
@@ -60,7 +61,8 @@ int conv_implicit_forward(const float *padded, const float *weight, const float 
 int conv_implicit_gradweight(const float *padded, const float *gradOutput, float *gradWeight, long B, int C, int H,
                              int W, int M, int kH, int kW, int pH, int pW, int sH, int sW, float scale);
 int conv_implicit_gradinput(const float *gradOutput, const float *weight, float *scratch, float *gradInput, long B,
-                            int C, int H, int W, int M, int kH, int kW, int pH, int pW, InputMask mask = InputMask());
+                            int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW,
+                            InputMask mask = InputMask());
 
 // Host-only checks of the launch planners (no GPU needed); each returns the number of violations.
 long im2col_plan_selftest();

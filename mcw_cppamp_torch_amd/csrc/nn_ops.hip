@@ -230,7 +230,8 @@ int conv_update_grad_input(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTen
     THGPUTensor *in = nullptr;
     InputMask mask;
     if (mask_on) {
-        if (gathered && plane_layout(input, mask_layout)) {
+        // (the strided layers' scattered store reads a dense mask only)
+        if (gathered && plane_layout(input, mask_layout) && ((dH == 1 && dW == 1) || mask_layout.dense)) {
             mask.in = dptr(input);
         } else {
             in = THGPUTensor_newContiguous(input);
@@ -255,7 +256,7 @@ int conv_update_grad_input(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTen
 
     if (gathered) {
         // fgradInput holds the padded gradOutput and the flipped kernels instead of the gradient columns
-        const long need = conv_implicit_gradinput_scratch(s.B, s.C, s.H, s.W, s.M, kH, kW);
+        const long need = conv_implicit_gradinput_scratch(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW);
         if (s.batched)
             THGPUTensor_resize4d(gradInput, s.B, s.C, s.H, s.W);
         else
@@ -266,7 +267,7 @@ int conv_update_grad_input(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTen
         if (!(tensor_backed(go) && tensor_backed(weight)))
             return fail("SpatialConvolutionMM: a tensor's shape exceeds its storage");
         return conv_implicit_gradinput(dptr(go), dptr(weight), dptr(fgradInput), dptr(gradInput), s.B, s.C, s.H, s.W,
-                                       s.M, kH, kW, padH, padW, mask);
+                                       s.M, kH, kW, padH, padW, dH, dW, mask);
     }
     if (s.batched) {
         THGPUTensor_resize4d(gradInput, s.B, s.C, s.H, s.W);

@@ -387,3 +387,79 @@ def test_accgradparameters_depends_on_its_arguments_alone(gt, mode):
     finally:
         assert lib.thgpu_conv_set_finput_reuse(0) == 0
         assert lib.thgpu_conv_set_mode(before) == 0
+
+
+STRIDED = [
+    # B, C, H, W, M, kH, kW, pH, pW, sH, sW
+    (2, 3, 40, 37, 64, 11, 11, 2, 2, 4, 4),     # the first-layer geometry: 48 rows padded to a 64-row tile
+    (3, 5, 23, 19, 16, 2, 2, 0, 0, 3, 3),       # kernel smaller than the stride: some pixels receive nothing
+    (2, 8, 17, 30, 24, 5, 3, 4, 2, 2, 3),       # padding above the stride, anisotropic everything
+    (1, 20, 64, 64, 32, 3, 3, 1, 1, 2, 2),      # 80 rows: an edge tile shifted back
+    (2, 70, 12, 10, 80, 3, 3, 1, 1, 2, 1),      # strided along one axis only
+    (4, 3, 101, 77, 37, 5, 5, 0, 0, 3, 3),      # odd sizes of the edge sweep
+    (32, 64, 128, 96, 128, 7, 3, 3, 1, 2, 1),   # the non-square case of the edge sweep at its stated size
+]
+
+
+@pytest.mark.parametrize("cfg", STRIDED)
+def test_strided_gradinput_by_residue_class(gt, gathered_route, cfg):
+    """gradInput of a strided layer as one product over the residue classes of the pixel coordinates (scattered
+    store, no column buffer), against the oracle's GEMM + col2im; the timing label shows that this product ran:
+    its reduction is M*ceil(kH/sH)*ceil(kW/sW) long and it has one column per cell of the strided grid."""
+    B, C, H, W, M, kH, kW, pH, pW, sH, sW = cfg
+    geo = (kH, kW, pH, pW, sH, sW)
+    K = C * kH * kW
+    rng = rng_for(51)
+    s = 1.0 / np.sqrt(K)
+    x = uniform(rng, (B, C, H, W))
+    w, b = uniform(rng, (M, K), -s, s), uniform(rng, (M,), -s, s)
+    Ho, Wo = (H + 2 * pH - kH) // sH + 1, (W + 2 * pW - kW) // sW + 1
+    go = uniform(rng, (B, M, Ho, Wo))
+    gi_ref, _ = oracle.conv_updateGradInput(go, w, x.shape, *geo)
+    m = gt.nn.SpatialConvolutionMM(C, M, kW, kH, sW, sH, 0, padW=pW, padH=pH)
+    m._assign("weight", w)
+    m._assign("bias", b)
+    m.gpu()
+    dx, dgo = dev(gt, x), dev(gt, go)
+    gt.gputorch.synchronize()
+    gt.gputorch.prof_reset()
+    gt.gputorch.prof_enable(True)
+    try:
+        gi = m.updateGradInput(dx, dgo).float()
+        gi2 = m.updateGradInput(dx, dgo).float()
+        gt.gputorch.synchronize()
+        labels = [k for k in gt.gputorch.prof_report() if k.startswith("gemm_conv_gradinput")]
+    finally:
+        gt.gputorch.prof_enable(False)
+        gt.gputorch.prof_reset()
+    A, Bk = -(-kH // sH), -(-kW // sW)
+    Yn, Xn = (H - 1 + pH) // sH + 1, (W - 1 + pW) // sW + 1
+    assert len(labels) == 1 and " J=%d R=%d " % (B * Yn * Xn, M * A * Bk) in labels[0], labels
+    assert np.array_equal(bits(gi), bits(gi2))
+    check_close("conv b%d %d->%d %dx%d k%dx%d p%dx%d s%dx%d gradInput by residue class" %
+                (B, C, M, H, W, kH, kW, pH, pW, sH, sW), gi, gi_ref, M * kH * kW)
+
+
+def test_strided_gradinput_integer_exact_and_untouched_neighbours(gt, gathered_route):
+    """Small integers make every sum exact: the scattered store must then reproduce the oracle bit for bit, and it
+    must write nothing outside gradInput (checked with a guard band around a view of a larger buffer)."""
+    B, C, H, W, M, kH, kW, pH, pW, sH, sW = 3, 6, 21, 26, 40, 5, 4, 2, 1, 3, 2
+    geo = (kH, kW, pH, pW, sH, sW)
+    rng = rng_for(52)
+    ints = lambda lo, hi, shape: rng.integers(lo, hi + 1, size=shape).astype(np.float32)
+    x, w = ints(-2, 2, (B, C, H, W)), ints(-2, 2, (M, C * kH * kW))
+    Ho, Wo = (H + 2 * pH - kH) // sH + 1, (W + 2 * pW - kW) // sW + 1
+    go = ints(-2, 2, (B, M, Ho, Wo))
+    gi_ref, _ = oracle.conv_updateGradInput(go, w, x.shape, *geo)
+    m = gt.nn.SpatialConvolutionMM(C, M, kW, kH, sW, sH, 0, padW=pW, padH=pH)
+    m._assign("weight", w)
+    m.gpu()
+    n = B * C * H * W
+    guard = 4096
+    big = dev(gt, np.full(n + 2 * guard, 7.5, np.float32))
+    m.gradInput = big.narrow(0, guard, n).view(B, C, H, W)
+    gi = m.updateGradInput(dev(gt, x), dev(gt, go)).float()
+    assert np.array_equal(gi, gi_ref)
+    host = big.float()
+    assert np.all(host[:guard] == 7.5) and np.all(host[guard + n:] == 7.5)
+    assert np.array_equal(host[guard:guard + n].reshape(B, C, H, W), gi_ref)

@@ -124,6 +124,8 @@ CASES = [
     ({"gemm_split": "3"}, ("conv", 64, 64, 3, 1, 1), 2),     # ... through the split reduction's final pass
     ({"gemm_tile": "64x64"}, ("conv", 64, 128, 3, 1, 1), 2),
     ({"gemm_tile": "128x128", "gemm_split": "2"}, ("conv", 128, 128, 3, 1, 1), 2),
+    ({}, ("conv", 16, 64, 7, 3, 2), 2),                      # strided gathered gradInput: the scattered store
+    ({"gemm_tile": "64x64"}, ("conv", 8, 64, 4, 2, 1), 2),   # ... with its rows padded to a tile
 ]
 
 
