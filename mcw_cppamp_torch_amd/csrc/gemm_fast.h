@@ -174,7 +174,10 @@ __global__ __launch_bounds__(WGM *WGN * 64)
             for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
 
     float ra[NA], rb[NB];
-    int roff[LB == LD_XC_GATHER ? NB : 1];  // gathered B: float offsets of the step's rows (uniform)
+    // Gathered B: float offsets of the rows of the step being loaded (uniform), and of the step after it.  The
+    // latter are fetched (scalar loads) in the middle of a step, a whole step before they turn into addresses,
+    // so that no step starts by waiting for its row offsets.
+    int roff[LB == LD_XC_GATHER ? NB : 1], roff_nx[LB == LD_XC_GATHER ? NB : 1];
 
     // Load number u of an operand for the step whose uniform base is `base`.
     auto load_unit = [&](auto kind_tag, const char *base, long stride, unsigned voff, float *dst, int u) {
@@ -206,11 +209,31 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         ga = tileA + ((RED ? (long)ld_img * g.rbA : 0L) + (LA == LD_XC_SCALAR ? (long)r0 * g.sA : (long)r0)) * 4;
         if (LB == LD_XC_GATHER) {
             gb = tileB + (RED ? (long)ld_img * g.rbB : 0L) * 4;
-            const int *rt = g.rowtab + r0 + b_r;
 #pragma unroll
-            for (int u = 0; u < NB; ++u) roff[u] = rt[u];
+            for (int u = 0; u < NB; ++u) roff[u] = roff_nx[u];
         } else {
             gb = tileB + ((RED ? (long)ld_img * g.rbB : 0L) + (LB == LD_XC_SCALAR ? (long)r0 * g.sB : (long)r0)) * 4;
+        }
+    };
+    // Row offsets of the step whose reduction window starts at `pos` (moved back like the step itself).
+    auto fetch_rows = [&](int pos) {
+        if (LB == LD_XC_GATHER) {
+            const int r0 = pos + BK <= g.R ? pos : g.R - BK;
+            const int *rt = g.rowtab + r0 + b_r;
+#pragma unroll
+            for (int u = 0; u < NB; ++u) roff_nx[u] = rt[u];
+        }
+    };
+    // Takes delivery of them (an empty statement that names the values keeps the compiler from postponing the
+    // loads to the point of first use).
+    auto pin_rows = [&]() {
+        if (LB == LD_XC_GATHER) {
+#pragma unroll
+            for (int u = 0; u < NB; ++u) {
+                int t = __builtin_amdgcn_readfirstlane(roff_nx[u]);
+                asm("" : "+s"(t));
+                roff_nx[u] = t;
+            }
         }
     };
     auto advance = [&]() {
@@ -270,6 +293,7 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     const char *ga = tileA, *gb = tileB;
     int shift = 0;
     if (nsteps > 0) {
+        fetch_rows(ld_r0);
         step_bases(ga, gb, shift);
 #pragma unroll
         for (int u = 0; u < UA; ++u) load_unit(std::integral_constant<int, KA>{}, ga, g.sA, voffA, ra, u);
@@ -277,6 +301,7 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         for (int u = 0; u < UB; ++u) load_unit(std::integral_constant<int, LB>{}, gb, g.sB, voffB, rb, u);
         stash(0, shift);
         advance();
+        fetch_rows(ld_r0);
     }
     __syncthreads();
 
@@ -327,6 +352,15 @@ __global__ __launch_bounds__(WGM *WGN * 64)
 #pragma unroll
                 for (int u = 0; u < UB; ++u)
                     if (u * SLICES / UB == slice) load_unit(std::integral_constant<int, LB>{}, gb, g.sB, voffB, rb, u);
+                // Offsets of the step after the one being loaded: requested once every LDS operand of this step
+                // has arrived (the scalar loads then share the wait counter with no outstanding LDS read), taken
+                // delivery of two slices later, still under this step's MFMAs.
+                if (slice == 5) {
+                    int pos = ld_r0 + BK;
+                    if (RED && pos >= g.R) pos = 0;
+                    fetch_rows(pos);
+                }
+                if (!RED && slice == 7) pin_rows();
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
