@@ -179,23 +179,34 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     // so that no step starts by waiting for its row offsets.
     int roff[LB == LD_XC_GATHER ? NB : 1], roff_nx[LB == LD_XC_GATHER ? NB : 1];
 
-    // Load number u of an operand for the step whose uniform base is `base`.
+    // Load number u of an operand for the step whose uniform base is `base`.  Buffer loads: the address is a
+    // descriptor in scalar registers (the step's base) plus a scalar offset (which load) plus the lane's constant
+    // 32-bit offset, so the loop spends no vector ALU instruction on addressing.  That matters more than its
+    // instruction count suggests: fp32 MFMAs and ordinary vector instructions share the SIMD's ALU (a v_add
+    // between two MFMAs costs 6 to 13 cycles of matrix-pipe time, measured), while scalar instructions and the
+    // issue of memory instructions run beside the matrix pipe.
+    typedef float float4v __attribute__((ext_vector_type(4)));
+    auto descriptor = [](const char *base) {
+        // raw buffer, no bounds (every offset below 2^32 passes), dword format
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(base), 0, -1, 0x00020000);
+    };
     auto load_unit = [&](auto kind_tag, const char *base, long stride, unsigned voff, float *dst, int u) {
         constexpr int KIND = decltype(kind_tag)::value;
+        const __amdgpu_buffer_rsrc_t rsrc = descriptor(base);
+        const int st = (int)stride * 4;
         if (KIND == LD_RC_VEC) {
-            const float4u v = *reinterpret_cast<const float4u *>(base + (long)(u * (NT / 4)) * stride * 4 + voff);
+            const float4v v = __builtin_bit_cast(
+                float4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff, u * (NT / 4) * st, 0));
             dst[u * 4 + 0] = v.x;
             dst[u * 4 + 1] = v.y;
             dst[u * 4 + 2] = v.z;
             dst[u * 4 + 3] = v.w;
-        } else if (KIND == LD_RC_SCALAR) {
-            dst[u] = *reinterpret_cast<const float *>(base + (long)(u * (NT / 16)) * stride * 4 + voff);
-        } else if (KIND == LD_XC_BLOCK) {
-            dst[u] = *reinterpret_cast<const float *>(base + (long)(u & 3) * stride * 4 + (u >> 2) * 256 + voff);
-        } else if (KIND == LD_XC_GATHER) {
-            dst[u] = *reinterpret_cast<const float *>(base + (long)roff[u] * 4 + voff);
         } else {
-            dst[u] = *reinterpret_cast<const float *>(base + (long)u * stride * 4 + voff);
+            const int so = KIND == LD_RC_SCALAR  ? u * (NT / 16) * st
+                           : KIND == LD_XC_BLOCK ? (u & 3) * st + (u >> 2) * 256
+                           : KIND == LD_XC_GATHER ? roff[u] * 4
+                                                  : u * st;
+            dst[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)voff, so, 0));
         }
     };
 
