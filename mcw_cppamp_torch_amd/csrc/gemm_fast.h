@@ -321,8 +321,10 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     // in slices between its MFMAs (a steady trickle of requests; a burst at the
     // head of the step would hold the wavefront, and with it its MFMAs, in the
     // memory pipeline's queue) and written to the other buffer afterwards.
-    for (int s = 0; s < nsteps; ++s) {
-        const int buf = s & 1;
+    // Two steps per trip, one per LDS buffer, so that the buffer is a compile-time constant and folds into the
+    // offset field of every LDS instruction instead of costing vector adds per step.
+    auto one_step = [&](auto buf_tag, int s) {
+        constexpr int buf = decltype(buf_tag)::value;
         const bool more = s + 1 < nsteps;
         // The last step has nothing to fetch; it re-reads the previous addresses
         // (valid, cached) rather than branching around the loads.
@@ -380,6 +382,10 @@ __global__ __launch_bounds__(WGM *WGN * 64)
             advance();
         }
         __syncthreads();
+    };
+    for (int s = 0; s < nsteps; s += 2) {
+        one_step(std::integral_constant<int, 0>{}, s);
+        if (s + 1 < nsteps) one_step(std::integral_constant<int, 1>{}, s + 1);
     }
 
     // ---- epilogue ----------------------------------------------------------------------
