@@ -315,6 +315,18 @@ void THGPUTensor_addr(THGPUTensor *self, float beta, THGPUTensor *t, float alpha
 
 /* ---- BLAS ------------------------------------------------------------------ */
 
+/* Level-1 / level-2 BLAS on device pointers with strided vectors: the generic TH signatures
+ * (mcw_torch7_core/lib/TH/generic/THBlas.h) in place of the array_view + offset ones of
+ * gputorch/lib/THC/THCBlas.h:29-48 (called from THCTensorMath.cpp:122,671-688,835-852 and
+ * gpunn-impl/SpatialConvolutionMM.cpp:413).  Column-major, semantics and degenerate-dimension fix-ups of
+ * TH/generic/THBlas.c:68-100,182-264; gemv 'n', ger and axpy add in TH's own order (bit-identical to its
+ * fallback loops), gemv 't' sums each column with a fixed-shape tree.  THGPUTensor_addmv / addr keep riding
+ * the GEMM. */
+void THGPUBlas_axpy(long n, float a, float *x, long incx, float *y, long incy);
+void THGPUBlas_ger(long m, long n, float alpha, float *x, long incx, float *y, long incy, float *a, long lda);
+void THGPUBlas_gemv(char trans, long m, long n, float alpha, float *a, long lda, float *x, long incx, float beta,
+                    float *y, long incy);
+
 /* Column-major C = beta*C + alpha*op(A)*op(B) on DEVICE pointers: the generic
  * THBlas signature (TH/generic/THBlas.h:17 instantiated by gputorch/lib/THC/
  * THCBlas.h:6-14); replaces the array_view overload THCBlas.h:35-39 and its

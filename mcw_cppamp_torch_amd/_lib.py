@@ -178,6 +178,9 @@ _SIGNATURES = {
     "THGPUTensor_addr": (None, [TensorP, c_float, TensorP, c_float, TensorP, TensorP]),
     "THGPUBlas_gemm": (None, [c_char, c_char, c_long, c_long, c_long, c_float, f32p, c_long, f32p, c_long,
                               c_float, f32p, c_long]),
+    "THGPUBlas_axpy": (None, [c_long, c_float, f32p, c_long, f32p, c_long]),
+    "THGPUBlas_ger": (None, [c_long, c_long, c_float, f32p, c_long, f32p, c_long, f32p, c_long]),
+    "THGPUBlas_gemv": (None, [c_char, c_long, c_long, c_float, f32p, c_long, f32p, c_long, c_float, f32p, c_long]),
     "thgpu_gemm_noalloc": (c_int, [c_char, c_char, c_long, c_long, c_long, c_float, f32p, c_long, f32p, c_long,
                                    c_float, f32p, c_long]),
     "thgpu_gemm_strided_batched": (c_int, [c_char, c_char, c_long, c_long, c_long, c_float, f32p, c_long, c_long, f32p,

@@ -47,9 +47,109 @@ void unary_scalar(THGPUTensor *self_, THGPUTensor *src_, float value, int op, co
     THGPUTensor_freeCopyTo(self, self_);
 }
 
+// ---- level-1 / level-2 BLAS with strided vectors, in the loop order of TH's own routines ---------------------
+
+// y[i*incy] += a * x[i*incx]   (TH/generic/THBlas.c:96-99)
+__global__ __launch_bounds__(256) void axpy_kernel(long n, float a, const float *__restrict__ x, long incx,
+                                                   float *__restrict__ y, long incy) {
+    const long stride = (long)gridDim.x * blockDim.x;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        y[i * incy] = __fadd_rn(y[i * incy], __fmul_rn(a, x[i * incx]));
+}
+
+// a[i + j*lda] += (alpha * y[j*incy]) * x[i*incx]   (TH/generic/THBlas.c:254-262)
+__global__ __launch_bounds__(256) void ger_kernel(long m, long n, float alpha, const float *__restrict__ x, long incx,
+                                                  const float *__restrict__ y, long incy, float *__restrict__ a,
+                                                  long lda) {
+    const long total = m * n;
+    const long stride = (long)gridDim.x * blockDim.x;
+    for (long e = (long)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += stride) {
+        const long j = e / m, i = e - j * m;
+        const float z = __fmul_rn(alpha, y[j * incy]);
+        a[i + j * lda] = __fadd_rn(a[i + j * lda], __fmul_rn(z, x[i * incx]));
+    }
+}
+
+// 'n': y[i] = beta*y[i], then += (alpha*x[j]) * a[i + j*lda] for j ascending: one lane per row i, rows coalesced
+// (TH/generic/THBlas.c:229-240; beta == 1 leaves y as it is, any other beta scales it first, as scal does).
+__global__ __launch_bounds__(256) void gemv_n_kernel(long m, long n, float alpha, const float *__restrict__ a, long lda,
+                                                     const float *__restrict__ x, long incx, float beta,
+                                                     float *__restrict__ y, long incy) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= m) return;
+    float acc = beta == 1.0f ? y[i * incy] : __fmul_rn(beta, y[i * incy]);
+    for (long j = 0; j < n; ++j) acc = __fadd_rn(acc, __fmul_rn(__fmul_rn(alpha, x[j * incx]), a[i + j * lda]));
+    y[i * incy] = acc;
+}
+
+// 't': y[i] = beta*y[i] + alpha * sum_j x[j] * a[j + i*lda]: one wavefront per output, lanes along the column, then a
+// fixed-shape tree over the 64 lane sums (TH/generic/THBlas.c:216-226 adds j ascending: tolerance parity, not bit parity).
+__global__ __launch_bounds__(256) void gemv_t_kernel(long m, long n, float alpha, const float *__restrict__ a, long lda,
+                                                     const float *__restrict__ x, long incx, float beta,
+                                                     float *__restrict__ y, long incy) {
+    const long i = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (i >= n) return;
+    const float *col = a + i * lda;
+    float sum = 0.0f;
+    for (long j = lane; j < m; j += 64) sum += x[j * incx] * col[j];
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off, 64);
+    if (lane == 0) y[i * incy] = beta * y[i * incy] + alpha * sum;
+}
+
+int launch_grid(long work) {
+    long blocks = (work + 255) / 256;
+    const long cap = 8L * 4 * num_cus();
+    return (int)(blocks > cap ? cap : blocks < 1 ? 1 : blocks);
+}
+
 }  // namespace
 
 extern "C" {
+
+void THGPUBlas_axpy(long n, float a, float *x, long incx, float *y, long incy) {
+    hipStream_t s = stream();
+    if (!s) return raise("%s", thgpu_last_error());
+    if (n <= 0) return;
+    if (n == 1) incx = incy = 1;  // TH/generic/THBlas.c:72-76
+    {
+        LaunchScope scope("blas_axpy", 2.0 * n, 12.0 * n);
+        hipLaunchKernelGGL(axpy_kernel, dim3(launch_grid(n)), dim3(256), 0, s, n, a, x, incx, y, incy);
+    }
+    if (check_launch("blas_axpy")) raise("%s", thgpu_last_error());
+}
+
+void THGPUBlas_ger(long m, long n, float alpha, float *x, long incx, float *y, long incy, float *a, long lda) {
+    hipStream_t s = stream();
+    if (!s) return raise("%s", thgpu_last_error());
+    if (m <= 0 || n <= 0) return;
+    if (n == 1) lda = m;  // TH/generic/THBlas.c:232-233
+    {
+        LaunchScope scope("blas_ger", 2.0 * m * n, 8.0 * m * n);
+        hipLaunchKernelGGL(ger_kernel, dim3(launch_grid(m * n)), dim3(256), 0, s, m, n, alpha, x, incx, y, incy, a, lda);
+    }
+    if (check_launch("blas_ger")) raise("%s", thgpu_last_error());
+}
+
+void THGPUBlas_gemv(char trans, long m, long n, float alpha, float *a, long lda, float *x, long incx, float beta,
+                    float *y, long incy) {
+    hipStream_t s = stream();
+    if (!s) return raise("%s", thgpu_last_error());
+    if (n == 1) lda = m;  // TH/generic/THBlas.c:184-185
+    const bool t = trans == 't' || trans == 'T';
+    const long outs = t ? n : m;
+    if (outs <= 0) return;
+    {
+        LaunchScope scope("blas_gemv", 2.0 * m * n, 4.0 * m * n);
+        if (t)
+            hipLaunchKernelGGL(gemv_t_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, s, m, n, alpha, a, lda, x, incx,
+                               beta, y, incy);
+        else
+            hipLaunchKernelGGL(gemv_n_kernel, dim3((unsigned)((m + 255) / 256)), dim3(256), 0, s, m, n, alpha, a, lda, x,
+                               incx, beta, y, incy);
+    }
+    if (check_launch("blas_gemv")) raise("%s", thgpu_last_error());
+}
 
 void THGPUTensor_add(THGPUTensor *self, THGPUTensor *src, float value) { unary_scalar(self, src, value, 0, "tensor_add"); }
 void THGPUTensor_mul(THGPUTensor *self, THGPUTensor *src, float value) { unary_scalar(self, src, value, 1, "tensor_mul"); }

@@ -503,6 +503,26 @@ def gemm(transa, transb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc):
     _lib.check()
 
 
+def gemv(trans, m, n, alpha, a, lda, x, incx, beta, y, incy):
+    """THGPUBlas_gemv on GPUTensor operands (column-major, strided vectors)."""
+    lib.THGPUBlas_gemv(trans.encode(), m, n, alpha, lib.THGPUTensor_data(a._p), lda, lib.THGPUTensor_data(x._p), incx,
+                       beta, lib.THGPUTensor_data(y._p), incy)
+    _lib.check()
+
+
+def ger(m, n, alpha, x, incx, y, incy, a, lda):
+    """THGPUBlas_ger: a += alpha * x y^T on a column-major m x n matrix."""
+    lib.THGPUBlas_ger(m, n, alpha, lib.THGPUTensor_data(x._p), incx, lib.THGPUTensor_data(y._p), incy,
+                      lib.THGPUTensor_data(a._p), lda)
+    _lib.check()
+
+
+def axpy(n, a, x, incx, y, incy):
+    """THGPUBlas_axpy: y += a * x."""
+    lib.THGPUBlas_axpy(n, a, lib.THGPUTensor_data(x._p), incx, lib.THGPUTensor_data(y._p), incy)
+    _lib.check()
+
+
 class Event(object):
     """HIP event on the library stream."""
 

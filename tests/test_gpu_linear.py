@@ -254,3 +254,72 @@ def test_gemm_strided_batched(gt, ta, tb, shared_b):
         Bi = B[0 if shared_b else i]
         opB = Bi.T if tb == "n" else Bi                                # k x n
         assert np.array_equal(got[i].T, 3 * C[i].T + 2 * (opA @ opB)), i
+
+
+def _ref_gemv(trans, m, n, alpha, a, lda, x, incx, beta, y, incy):
+    """TH's fallback loops (TH/generic/THBlas.c:216-240) in float32, for the bit-for-bit comparisons."""
+    a, x, y = a.copy(), x.copy(), y.copy()
+    f = np.float32
+    if trans == "t":
+        for i in range(n):
+            s = f(0)
+            for j in range(m):
+                s = f(s + f(x[j * incx] * a[j + i * lda]))
+            y[i * incy] = f(f(beta * y[i * incy]) + f(alpha * s))
+    else:
+        if beta != 1:
+            for i in range(m):
+                y[i * incy] = f(beta * y[i * incy])
+        for j in range(n):
+            z = f(f(alpha) * x[j * incx])
+            for i in range(m):
+                y[i * incy] = f(y[i * incy] + f(z * a[i + j * lda]))
+    return y
+
+
+@pytest.mark.parametrize("trans", ["n", "t"])
+@pytest.mark.parametrize("shape", [(1, 1), (5, 3), (70, 130), (257, 64), (3, 1), (1, 9)])
+def test_blas_gemv_strided(gt, trans, shape):
+    """THGPUBlas_gemv with padded leading dimension and strided vectors: 'n' bit for bit with TH's loop order,
+    't' within 1e-4*sqrt(m) (its column sums are trees), both exact on integers."""
+    m, n = shape
+    rng = rng_for(71)
+    lda, incx, incy = m + 3, 2, 3
+    nx, ny = (n, m) if trans == "n" else (m, n)
+    for integers in (False, True):
+        draw = (lambda shp: rng.integers(-3, 4, size=shp).astype(np.float32)) if integers else (lambda shp: uniform(rng, shp))
+        a, x, y = draw((lda * n,)), draw((nx * incx,)), draw((ny * incy,))
+        alpha, beta = (2.0, -1.0) if integers else (0.75, 0.5)
+        da, dx, dy = dev(gt, a), dev(gt, x), dev(gt, y)
+        gt.gputorch.gemv(trans, m, n, alpha, da, lda, dx, incx, beta, dy, incy)
+        got = dy.float()
+        ref = _ref_gemv(trans, m, n, np.float32(alpha), a, lda if n != 1 else m, x, incx, np.float32(beta), y, incy)
+        if trans == "n" or integers:
+            assert np.array_equal(got, ref)
+        else:
+            assert np.max(np.abs(got - ref)) <= 1e-4 * np.sqrt(m) * max(1.0, np.max(np.abs(ref)))
+        # elements between the strided ones are untouched
+        mask = np.ones(ny * incy, bool)
+        mask[::incy] = False
+        assert np.array_equal(got[mask], y[mask])
+
+
+def test_blas_ger_and_axpy(gt):
+    rng = rng_for(72)
+    m, n, lda, incx, incy = 37, 21, 40, 2, 3
+    a, x, y = uniform(rng, (lda * n,)), uniform(rng, (m * incx,)), uniform(rng, (n * incy,))
+    da = dev(gt, a)
+    gt.gputorch.ger(m, n, 0.5, dev(gt, x), incx, dev(gt, y), incy, da, lda)
+    ref = a.copy()
+    f = np.float32
+    for j in range(n):
+        z = f(f(0.5) * y[j * incy])
+        ref[j * lda:j * lda + m] = ref[j * lda:j * lda + m] + z * x[:m * incx:incx]
+    assert np.array_equal(da.float(), ref)
+    k = 1000
+    u, v = uniform(rng, (k * 2,)), uniform(rng, (k * 3,))
+    dv = dev(gt, v)
+    gt.gputorch.axpy(k, 1.5, dev(gt, u), 2, dv, 3)
+    ref = v.copy()
+    ref[::3] = ref[::3] + f(1.5) * u[::2]
+    assert np.array_equal(dv.float(), ref)
