@@ -307,6 +307,7 @@ def summarise(args):
     """bench.py --summarise kernel-trace STATS.csv BENCH.json STEPS   (rocprofv3 --kernel-trace --stats ... _kernel_stats.csv)
     bench.py --summarise traffic FETCH.csv WRITE.csv BENCH.json STEPS  (two --pmc runs' _counter_collection.csv)
     bench.py --summarise mfma COUNTERS.csv                             (one --pmc run with the SQ_* counters)
+    bench.py --summarise hbm-pmc COUNTERS.csv KERNEL_TRACE.csv         (one --pmc run around --workload hbm_sweep)
     BENCH.json is the line an ordinary run of the same configuration printed; STEPS the steps the profiled runs made
     (warm-up included).  Writes the summary to stdout; `header` lines (the commands) come from --summary-header."""
     kind, files = args.summarise[0], args.summarise[1:]
@@ -392,8 +393,41 @@ def summarise(args):
                 100 * c["SQ_WAIT_INST_LDS"] / wave, 100 * c["SQ_LDS_BANK_CONFLICT"] / max(c["SQ_ACTIVE_INST_LDS"], 1)))
         out.append("mfma_busy = SQ_VALU_MFMA_BUSY_CYCLES / (4 * SQ_BUSY_CU_CYCLES); wait_* = SQ_WAIT_INST_* / SQ_WAVE_CYCLES; "
                    "lds_confl = SQ_LDS_BANK_CONFLICT / SQ_ACTIVE_INST_LDS.")
+    elif kind == "hbm-pmc":
+        # COUNTERS.csv of `rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_WAIT_ANY SQ_WAIT_INST_ANY
+        # SQ_INSTS_VALU SQ_INSTS_LDS SQ_INSTS_VMEM --kernel-trace` around `bench.py --workload hbm_sweep`, and the
+        # kernel trace of the same run (durations): what a wavefront of each HBM-bound kernel spends its life on.
+        dur = {}
+        for r in csv.DictReader(open(files[1])):
+            dur[int(r["Dispatch_Id"])] = int(r["End_Timestamp"]) - int(r["Start_Timestamp"])
+        agg = collections.OrderedDict()
+        for r in csv.DictReader(open(files[0])):
+            fam = _family(r["Kernel_Name"])
+            if fam is None or fam == "gemm":
+                continue
+            key = (fam, int(r["Grid_Size"]))
+            a = agg.setdefault(key, collections.defaultdict(float))
+            a[r["Counter_Name"]] += float(r["Counter_Value"])
+            if r["Counter_Name"] == "SQ_WAVES":
+                a["_launches"] += 1
+                a["_ns"] += dur.get(int(r["Dispatch_Id"]), 0)
+        out.append("%-18s %11s %8s %9s %10s %8s %8s %7s %6s %6s %6s" % (
+            "kernel", "threads", "launches", "us/launch", "waves/SIMD", "life us", "waiting", "on mem", "VALU", "LDS", "VMEM"))
+        for (fam, grid), c in agg.items():
+            n = max(c["_launches"], 1)
+            waves = max(c["SQ_WAVES"], 1)
+            us = c["_ns"] / n / 1e3
+            wave_cycles = c["SQ_WAVE_CYCLES"] * 4          # the counter ticks once per four cycles
+            clocks = c["_ns"] * 2.4                          # 2.4 GHz shader clock
+            out.append("%-18s %11d %8d %9.1f %10.2f %8.1f %7.0f%% %6.0f%% %6.0f %6.0f %6.0f" % (
+                fam, grid, n, us, wave_cycles / max(clocks, 1) / 1024, wave_cycles / waves / 2400.0,
+                100 * c["SQ_WAIT_ANY"] / max(c["SQ_WAVE_CYCLES"], 1), 100 * c["SQ_WAIT_INST_ANY"] / max(c["SQ_WAVE_CYCLES"], 1),
+                c["SQ_INSTS_VALU"] / waves, c["SQ_INSTS_LDS"] / waves, c["SQ_INSTS_VMEM"] / waves))
+        out.append("waves/SIMD = 4 * SQ_WAVE_CYCLES / (launch duration * 2.4 GHz * 1024 SIMDs), at most 8; life = mean residence of "
+                   "a wavefront; waiting = SQ_WAIT_ANY / SQ_WAVE_CYCLES (any wait, barriers included); on mem = SQ_WAIT_INST_ANY / "
+                   "SQ_WAVE_CYCLES; VALU / LDS / VMEM = instructions per wavefront.")
     else:
-        sys.exit("--summarise kernel-trace | traffic | mfma")
+        sys.exit("--summarise kernel-trace | traffic | mfma | hbm-pmc")
     print("\n".join(out))
 
 

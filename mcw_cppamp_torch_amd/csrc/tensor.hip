@@ -579,7 +579,11 @@ void THGPUTensor_copy(THGPUTensor *self, THGPUTensor *src) {
             return;
         }
     }
-    THGPU_ARGCHECK(self->nDimension <= THGPU_MAX_DIMS, 1, "too many dimensions", );
+    if (self->nDimension > THGPU_MAX_DIMS) {
+        if (s != src) THGPUTensor_free(s);
+        raise("bad argument #1: too many dimensions");
+        return;
+    }
     StridedDesc d;
     d.nd = self->nDimension;
     long dense = 1;
@@ -591,6 +595,7 @@ void THGPUTensor_copy(THGPUTensor *self, THGPUTensor *src) {
     }
     hipStream_t st = stream();
     if (!st) {
+        if (s != src) THGPUTensor_free(s);
         raise("%s", thgpu_last_error());
         return;
     }
