@@ -117,6 +117,13 @@ int thgpu_debug_set(const char *name, const char *value);
 /* Real stream synchronisation, replacing the no-op gputorch.synchronize
  * (gputorch/init.cpp:10-14). */
 int thgpu_synchronize(void);
+/* Storage buffers that are released (free, resize) are kept and handed out again to the next request of the
+ * same size instead of going through hipFree / hipMalloc and a stream drain (everything runs on the library's
+ * one in-order stream, so reuse is ordered).  thgpu_empty_cache returns the kept blocks to the device (it
+ * drains the stream first); thgpu_cached_bytes says how much is kept.  The cache empties itself above 8 GiB
+ * and when an allocation fails.  No counterpart in the reference, whose array_views freed eagerly. */
+int thgpu_empty_cache(void);
+long thgpu_cached_bytes(void);
 
 /* Device name / compute-unit count / total memory, replacing the stubbed
  * getDeviceProperties (gputorch/init.cpp:40-66). */

@@ -324,7 +324,7 @@ using namespace thgpu;
 namespace {
 
 // Column-major BLAS arguments as a GemmProblem.  Returns 1 for the quick returns of the reference
-// dispatcher (nothing to do), -1 for a dimension the kernels cannot index, 0 otherwise.
+// dispatcher (nothing to do), -1 for a dimension the kernels cannot index, -2 for a null operand, 0 otherwise.
 int blas_problem(GemmProblem &p, char transa, char transb, long m, long n, long k, float alpha, const float *a,
                  long lda, const float *b, long ldb, float beta, float *c, long ldc) {
     const bool ta = (transa == 't' || transa == 'T');
@@ -344,6 +344,8 @@ int blas_problem(GemmProblem &p, char transa, char transb, long m, long n, long 
         if (n == 1) ldb = k;
     }
     if (m < 0 || n < 0 || k < 0 || m >= (1L << 31) || n >= (1L << 31) || k >= (1L << 31)) return -1;
+    // a product that will touch memory needs its operands: a null pointer here would fault on the GPU
+    if (!c || (alpha != 0 && k > 0 && (!a || !b))) return -2;
     // Column-major C(m x n) is the row-major n x m matrix C'(i', j') =
     // c[j' + i'*ldc]; C' = op(B)' * op(A)' with
     //   A'(i', r) = op(B)(r, i'),  B'(r, j') = op(A)(j', r).
@@ -373,7 +375,7 @@ extern "C" void THGPUBlas_gemm(char transa, char transb, long m, long n, long k,
     const int rc = blas_problem(p, transa, transb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
     if (rc > 0) return;
     if (rc < 0) {
-        raise("THGPUBlas_gemm: dimension exceeds 2^31");
+        raise(rc == -2 ? "THGPUBlas_gemm: null operand" : "THGPUBlas_gemm: dimension exceeds 2^31");
         return;
     }
     if (gemm_launch(p)) raise("%s", thgpu_last_error());
@@ -392,7 +394,7 @@ extern "C" int thgpu_gemm_noalloc(char transa, char transb, long m, long n, long
     GemmProblem p;
     const int rc = blas_problem(p, transa, transb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
     if (rc > 0) return 0;
-    if (rc < 0) return fail("thgpu_gemm_noalloc: dimension exceeds 2^31");
+    if (rc < 0) return fail(rc == -2 ? "thgpu_gemm_noalloc: null operand" : "thgpu_gemm_noalloc: dimension exceeds 2^31");
     p.ws_fixed = ws;
     p.ws_fixed_floats = (long)cap;
     p.tag = "gemm_blas_noalloc";
@@ -407,6 +409,7 @@ extern "C" int thgpu_gemm_strided_batched(char transa, char transb, long m, long
     if (batch <= 0 || !m || !n) return 0;
     if (m >= (1L << 31) || n >= (1L << 31) || k >= (1L << 31)) return fail("gemm_strided_batched: dimension exceeds 2^31");
     if (stride_c == 0 && batch > 1) return fail("gemm_strided_batched: the results of a batch must not overlap");
+    if (!c || (alpha != 0 && k > 0 && (!a || !b))) return fail("gemm_strided_batched: null operand");
     // One launch for the whole batch when op(B) is shared, op(A) = A and the batch's columns fit the
     // kernel's 32-bit tile indexing: the batch index then simply extends the columns of the (row-major,
     // transposed) product, as in the convolution's forward and gradInput GEMMs.

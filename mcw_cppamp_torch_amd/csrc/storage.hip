@@ -6,6 +6,7 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <unordered_map>
 #include <vector>
 
 using namespace thgpu;
@@ -92,13 +93,68 @@ int copy_d2d(float *dst, const float *src, long n) {
 
 }  // namespace thgpu
 
-static void release_buffer(THGPUStorage *self) {
-    if (self->data) {
-        // Work enqueued earlier may still use the buffer.
-        hipStream_t s = stream();
-        if (s) (void)hipStreamSynchronize(s);
-        (void)hipFree(self->data);
+// ---- device blocks ------------------------------------------------------------------------------------
+// A released block goes to a free list keyed by its size and is handed out again to the next request of that
+// size, without draining the stream and without hipFree / hipMalloc: everything the library enqueues runs on
+// its one in-order stream, so whatever still uses the block was enqueued before its release and whatever the
+// next owner enqueues runs after it.  Shapes recur in this workload (the same modules resize the same buffers
+// every step), so exact-size reuse hits.  The cache is dropped (after a stream drain) when it holds more than
+// kCacheLimit bytes or when hipMalloc fails.
+namespace {
+
+constexpr size_t kCacheLimit = size_t(8) << 30;
+std::unordered_map<size_t, std::vector<float *>> g_free_blocks;
+size_t g_cached_bytes = 0;
+
+void drop_cached_blocks() {
+    if (g_free_blocks.empty()) return;
+    hipStream_t s = thgpu::stream();
+    if (s) (void)hipStreamSynchronize(s);
+    for (auto &kv : g_free_blocks)
+        for (float *p : kv.second) (void)hipFree(p);
+    g_free_blocks.clear();
+    g_cached_bytes = 0;
+}
+
+// hipSuccess and a block of `floats` floats, or the error of the failed hipMalloc (cleared from the runtime's
+// sticky state: the failure is reported by the caller, later launch checks must not see it again).
+hipError_t acquire_block(long floats, float **out) {
+    const size_t bytes = sizeof(float) * (size_t)floats;
+    auto it = g_free_blocks.find(bytes);
+    if (it != g_free_blocks.end() && !it->second.empty()) {
+        *out = it->second.back();
+        it->second.pop_back();
+        g_cached_bytes -= bytes;
+        return hipSuccess;
     }
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(out), bytes);
+    if (e != hipSuccess && !g_free_blocks.empty()) {
+        (void)hipGetLastError();
+        drop_cached_blocks();
+        e = hipMalloc(reinterpret_cast<void **>(out), bytes);
+    }
+    if (e != hipSuccess) (void)hipGetLastError();
+    return e;
+}
+
+void release_block(float *p, long floats) {
+    if (!p) return;
+    const size_t bytes = sizeof(float) * (size_t)floats;
+    if (floats <= 0 || g_cached_bytes + bytes > kCacheLimit) {
+        hipStream_t s = thgpu::stream();
+        if (s) (void)hipStreamSynchronize(s);  // work enqueued earlier may still use the buffer
+        (void)hipFree(p);
+        if (g_cached_bytes + bytes > kCacheLimit) drop_cached_blocks();
+        return;
+    }
+    g_free_blocks[bytes].push_back(p);
+    g_cached_bytes += bytes;
+}
+
+}  // namespace
+
+static void release_buffer(THGPUStorage *self) {
+    release_block(self->data, self->size);
     self->data = nullptr;
     self->size = 0;
 }
@@ -140,10 +196,9 @@ THGPUStorage *THGPUStorage_newWithSize(long size) {
         raise("%s", thgpu_last_error());
         return nullptr;
     }
-    hipError_t e = hipMalloc(reinterpret_cast<void **>(&s->data), sizeof(float) * (size_t)size);
+    hipError_t e = acquire_block(size, &s->data);
     if (e != hipSuccess) {
         std::free(s);
-        (void)hipGetLastError();  // the failure is reported here; later launch checks must not see it again
         raise("hipMalloc of %ld floats failed: %s", size, hipGetErrorString(e));
         return nullptr;
     }
@@ -216,9 +271,8 @@ void THGPUStorage_resize(THGPUStorage *self, long size) {
         raise("%s", thgpu_last_error());
         return;
     }
-    hipError_t e = hipMalloc(reinterpret_cast<void **>(&fresh), sizeof(float) * (size_t)size);
+    hipError_t e = acquire_block(size, &fresh);
     if (e != hipSuccess) {
-        (void)hipGetLastError();
         raise("hipMalloc of %ld floats failed: %s", size, hipGetErrorString(e));
         return;
     }
@@ -277,6 +331,13 @@ THGPU_STORAGE_COPY_VIA_FLOAT(Short, short)
 THGPU_STORAGE_COPY_VIA_FLOAT(Int, int)
 THGPU_STORAGE_COPY_VIA_FLOAT(Long, long)
 THGPU_STORAGE_COPY_VIA_FLOAT(Double, double)
+
+int thgpu_empty_cache(void) {
+    drop_cached_blocks();
+    return 0;
+}
+
+long thgpu_cached_bytes(void) { return (long)g_cached_bytes; }
 
 }  // extern "C"
 

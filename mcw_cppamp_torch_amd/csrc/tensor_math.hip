@@ -111,6 +111,7 @@ void THGPUBlas_axpy(long n, float a, float *x, long incx, float *y, long incy) {
     hipStream_t s = stream();
     if (!s) return raise("%s", thgpu_last_error());
     if (n <= 0) return;
+    if (!x || !y) return raise("THGPUBlas_axpy: null operand");
     if (n == 1) incx = incy = 1;  // TH/generic/THBlas.c:72-76
     {
         LaunchScope scope("blas_axpy", 2.0 * n, 12.0 * n);
@@ -123,6 +124,7 @@ void THGPUBlas_ger(long m, long n, float alpha, float *x, long incx, float *y, l
     hipStream_t s = stream();
     if (!s) return raise("%s", thgpu_last_error());
     if (m <= 0 || n <= 0) return;
+    if (!x || !y || !a) return raise("THGPUBlas_ger: null operand");
     if (n == 1) lda = m;  // TH/generic/THBlas.c:232-233
     {
         LaunchScope scope("blas_ger", 2.0 * m * n, 8.0 * m * n);
@@ -139,6 +141,7 @@ void THGPUBlas_gemv(char trans, long m, long n, float alpha, float *a, long lda,
     const bool t = trans == 't' || trans == 'T';
     const long outs = t ? n : m;
     if (outs <= 0) return;
+    if (!a || !x || !y) return raise("THGPUBlas_gemv: null operand");
     {
         LaunchScope scope("blas_gemv", 2.0 * m * n, 4.0 * m * n);
         if (t)

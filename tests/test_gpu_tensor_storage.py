@@ -325,3 +325,32 @@ def test_fill_many_fills_every_tensor_in_one_call_and_rejects_views(gt):
     net.zeroGradParameters()
     for m in (net.get(0), net.get(2)):
         assert not m.gradWeight.float().any() and not m.gradBias.float().any()
+
+
+def test_released_blocks_are_reused_without_a_device_free(gt):
+    """A released storage buffer is handed to the next request of the same size (same device address, contents of
+    the new owner intact although the old owner's work was still queued), other sizes get other blocks, and
+    thgpu_empty_cache returns everything to the device."""
+    lib = gt._lib.lib
+    assert lib.thgpu_empty_cache() == 0 and lib.thgpu_cached_bytes() == 0
+    n = 1 << 20
+    a = gt.GPUTensor(n).fill(1.5)
+    addr = lib.THGPUTensor_data(a._p)
+    addr = ctypes_addr(addr)
+    del a
+    import gc
+    gc.collect()
+    assert lib.thgpu_cached_bytes() == 4 * n
+    b = gt.GPUTensor(n // 2).fill(2.5)          # another size: a fresh block
+    assert ctypes_addr(lib.THGPUTensor_data(b._p)) != addr
+    c = gt.GPUTensor(n).fill(3.5)               # the same size: the kept block, ordered after the old owner's fill
+    assert ctypes_addr(lib.THGPUTensor_data(c._p)) == addr and lib.thgpu_cached_bytes() == 0
+    assert np.all(c.float() == 3.5) and np.all(b.float() == 2.5)
+    c.resize(n + 7)                             # a resize keeps the prefix and releases the old block
+    assert np.all(c.float()[:n] == 3.5) and lib.thgpu_cached_bytes() == 4 * n
+    assert lib.thgpu_empty_cache() == 0 and lib.thgpu_cached_bytes() == 0
+
+
+def ctypes_addr(p):
+    import ctypes
+    return ctypes.cast(p, ctypes.c_void_p).value
