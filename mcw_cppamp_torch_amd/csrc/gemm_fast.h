@@ -22,9 +22,17 @@
 //     lanes = consecutive rows) has rows of 16 + 4 floats; a tile written a row
 //     at a time (four lanes per row) has rows of 16 floats whose four 16-byte
 //     quarters are stored at quarter (r/4) xor ((x/4) mod 4).
-//   * LDS is double buffered; the next tile's global loads are issued before
+//   * LDS is double buffered; the next tile's global loads are issued between
 //     the current tile's MFMAs and written to the other buffer afterwards: one
 //     barrier per reduction step.
+//   * Between the MFMAs of a step there are memory and scalar instructions only.
+//     fp32 MFMAs and ordinary vector instructions share the SIMD's ALU (a v_add
+//     between two MFMAs costs 6 to 13 cycles of matrix time, measured), and a
+//     wavefront with MFMAs to issue keeps the other wavefronts of its SIMD from
+//     issuing anything, so nothing the loop does is hidden by another wavefront:
+//     operands are fetched with buffer loads (descriptor and offsets in scalar
+//     registers, a constant lane offset), and the loop is unrolled by two so
+//     that the LDS buffer folds into the offset field of the LDS instructions.
 #pragma once
 
 #include <type_traits>
