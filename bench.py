@@ -176,6 +176,8 @@ def ref_benchmark(args, pkg):
 
     rng = np.random.Generator(np.random.PCG64(77))
     rows, tot_fl, tot_t = [], 0.0, 0.0
+    if pkg._lib.lib.thgpu_conv_set_mode(ROUTES[args.conv_route]) != 0:
+        sys.exit("bench.py: " + pkg._lib.lib.thgpu_last_error().decode())
     for ni, no, kw, kh, iw, ih, bs, dw, dh in REF_BENCHMARK_RUNS:
         m = nn.SpatialConvolutionMM(ni, no, kw, kh, dw, dh, rng=rng).gpu()
         x = pkg.FloatTensor(rng.standard_normal((bs, ni, ih, iw)).astype(np.float32)).gpu()
@@ -206,7 +208,7 @@ def ref_benchmark(args, pkg):
         "warmup": args.warmup, "ms_per_step": round(tot_t * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "seven single layers, three passes each timed on its own; value = all flops / all time",
-                   "device": gputorch.getDeviceProperties()["name"]},
+                   "conv_route": args.conv_route, "device": gputorch.getDeviceProperties()["name"]},
         "layers": rows}))
 
 

@@ -355,7 +355,15 @@ bool conv_use_gathered_gradinput(long B, int C, int H, int W, int M, int kH, int
         return M < 512 && excess <= 2.0;
     }
     const long rows = (C + 63L) / 64 * 64;
-    return M < 512 && rows * 8 <= C * 9L;
+    // An unpadded (or lightly padded) layer has fewer output positions than input pixels, and the gathered
+    // product computes one column per input pixel: it executes H*W / (Ho*Wo) times the layer's flops, where the
+    // column route pays the algorithmic flops plus the gradient columns' trip through memory (8*K*N bytes per
+    // image).  At the measured rates (120 TFLOP/s, 4.5 TB/s) the columns win once (H*W/(Ho*Wo) - 1) * M exceeds
+    // about 100; measured on the reference benchmark's unpadded layers, the switch-over lies between 100 (gathered
+    // still 9 % ahead) and 150 (columns 19 % ahead).
+    const long Ho = H + 2L * pH - kH + 1, Wo = W + 2L * pW - kW + 1;
+    const bool inflation_ok = ((long)H * W - Ho * Wo) * M <= 110 * Ho * Wo;
+    return M < 512 && rows * 8 <= C * 9L && inflation_ok;
 }
 
 long conv_implicit_gradinput_scratch(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH,
