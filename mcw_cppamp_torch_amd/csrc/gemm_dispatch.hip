@@ -67,6 +67,9 @@ struct TileCfg {
     // the row count from which the tile is no longer considered (0: no limit).
     const double *occ;
     int below_rows;
+    // Short-row variant: the rows of the tile its wavefronts multiply (0: all of them).  It takes scattered products
+    // of exactly one tile of rows, of which no more than this many are in use.
+    int rows_used;
 };
 
 // The 64 x 128 tile's wavefronts own 64 x 32 outputs, half the MFMAs per reduction step of the large tiles: it needs all
@@ -76,13 +79,15 @@ struct TileCfg {
 const double kOccNarrow[5] = {0.0, 0.50, 0.75, 0.88, 1.0};
 
 const TileCfg kCfgs[] = {
-    {"128x128", 128, 128, 4, {0.90, 0.90, 0.88, 0.86, 0.90}, gemm_fast_128x128, nullptr, 0},
-    {"192x128", 192, 128, 3, {0.90, 0.90, 0.90, 0.86, 0.90}, gemm_fast_192x128, nullptr, 0},
-    {"64x256", 64, 256, 3, {0.76, 0.74, 0.90, 0.74, 0.70}, gemm_fast_64x256, nullptr, 0},
-    {"128x256", 128, 256, 2, {0.85, 0.87, 0.95, 0.85, 0.85}, gemm_fast_128x256, nullptr, 0},
-    {"256x128", 256, 128, 2, {0.90, 0.75, 0.95, 0.75, 0.90}, gemm_fast_256x128, nullptr, 0},
-    {"64x64", 64, 64, 4, {0.68, 0.60, 0.74, 0.60, 0.72}, gemm_fast_64x64, nullptr, 0},
-    {"64x128", 64, 128, 4, {0.84, 0.78, 0.84, 0.78, 0.86}, gemm_fast_64x128, kOccNarrow, 128},
+    {"128x128", 128, 128, 4, {0.90, 0.90, 0.88, 0.86, 0.90}, gemm_fast_128x128, nullptr, 0, 0},
+    {"192x128", 192, 128, 3, {0.90, 0.90, 0.90, 0.86, 0.90}, gemm_fast_192x128, nullptr, 0, 0},
+    {"64x256", 64, 256, 3, {0.76, 0.74, 0.90, 0.74, 0.70}, gemm_fast_64x256, nullptr, 0, 0},
+    {"128x256", 128, 256, 2, {0.85, 0.87, 0.95, 0.85, 0.85}, gemm_fast_128x256, nullptr, 0, 0},
+    {"256x128", 256, 128, 2, {0.90, 0.75, 0.95, 0.75, 0.90}, gemm_fast_256x128, nullptr, 0, 0},
+    {"64x64", 64, 64, 4, {0.68, 0.60, 0.74, 0.60, 0.72}, gemm_fast_64x64, nullptr, 0, 0},
+    {"64x128", 64, 128, 4, {0.84, 0.78, 0.84, 0.78, 0.86}, gemm_fast_64x128, kOccNarrow, 128, 0},
+    {"48x128", 64, 128, 4, {0, 0, 0, 0, 0.84}, gemm_fast_48x128, kOccNarrow, 128, 48},
+    {"48x256", 64, 256, 3, {0, 0, 0, 0, 0.70}, gemm_fast_48x256, nullptr, 0, 48},
 };
 
 inline long cdiv(long a, long b) { return (a + b - 1) / b; }
@@ -101,7 +106,7 @@ double model_cycles(const TileCfg &c, int layout, long M, long J, long steps_tot
     const long tiles = cdiv(M, c.bm) * cdiv(J, c.bn);
     const long wgs = tiles * nsplit;
     const long steps = cdiv(steps_total, nsplit);
-    const double per_step = 2.0 * c.bm * c.bn * GEMM_BK / 256.0 / c.eff[layout];
+    const double per_step = 2.0 * (c.rows_used ? c.rows_used : c.bm) * c.bn * GEMM_BK / 256.0 / c.eff[layout];
     const double ovh = 3000.0 + 6.0 * c.bm * c.bn / 64.0;
     const long slots = (long)cus * c.resident;
     const long full = wgs / slots, rest = wgs - full * slots;
@@ -150,6 +155,7 @@ GemmPlan plan_gemm(const GemmProblem &p, int steps_total) {
         if (!fast_ok || p.M < c.bm || p.J < c.bn || !offsets_fit(c.bm, c.bn)) continue;
         if (force && std::strcmp(force, c.name) != 0) continue;
         if (!force && c.below_rows > 0 && p.M >= c.below_rows) continue;
+        if (c.rows_used > 0 && !(p.scatter && layout == 4 && p.M == c.bm && p.scat_rows <= c.rows_used)) continue;
         const long tiles = cdiv(p.M, c.bm) * cdiv(p.J, c.bn);
         int max_split = (int)(steps_total / 8 > 0 ? (steps_total / 8 < 256 ? steps_total / 8 : 256) : 1);
         if (p.scatter) max_split = 1;  // the scattered store has no partial-sum form

@@ -70,12 +70,19 @@ constexpr int gemm_min_waves() {
     return (BM / WGM) * (BN / WGN) / 64 >= 96 ? 2 : 3;
 }
 
-template <int BM, int BN, int WGM, int WGN, int LA, int LB, bool RED>
+// ROWS16 > 0 selects the short-row variant: the workgroup still loads BM = 64 rows of the first operand, but its
+// wavefronts multiply only the first 16*ROWS16 of them, in 16x16 blocks (v_mfma_f32_16x16x4_f32, four registers per
+// lane and block).  It exists for scattered products whose row count is 48 (three planes at stride 4 x 4), which
+// would otherwise spend a quarter of their MFMAs on padding; it has the scattered store only.
+template <int BM, int BN, int WGM, int WGN, int LA, int LB, bool RED, int ROWS16 = 0>
 __global__ __launch_bounds__(WGM *WGN * 64)
     __attribute__((amdgpu_waves_per_eu(gemm_min_waves<BM, BN, WGM, WGN>()))) void gemm_fast_kernel(const GemmArgs g) {
     constexpr int NT = WGM * WGN * 64;
     constexpr int BK = GEMM_BK;
-    constexpr int TM = BM / WGM / 32, TN = BN / WGN / 32;
+    constexpr bool SMALL = ROWS16 > 0;
+    constexpr int TM = SMALL ? ROWS16 : BM / WGM / 32, TN = SMALL ? BN / WGN / 16 : BN / WGN / 32;
+    static_assert(!SMALL || (WGM == 1 && BM == 64 && ROWS16 <= 4 && LB == LD_XC_GATHER && !RED && TN % 2 == 0),
+                  "the short-row variant: one row of wavefronts over a 64-row tile, gathered B, scattered store");
     constexpr int NA = BM * BK / NT, NB = BN * BK / NT;
     static_assert(BM % (WGM * 32) == 0 && BN % (WGN * 32) == 0, "wave tile must be whole 32x32 blocks");
     static_assert(NT % 16 == 0 && NA >= 4 && NB >= 4 && NA % 4 == 0 && NB % 4 == 0, "loader shape");
@@ -173,13 +180,16 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     constexpr int UA = LA == LD_RC_VEC ? NA / 4 : NA;  // load instructions per step and operand
     constexpr int UB = LB == LD_RC_VEC ? NB / 4 : NB;
 
-    floatx16 acc[TM][TN];
+    // One accumulator per block: 16 registers (32x32 blocks) or 4 (16x16 blocks of the short-row variant).
+    using Acc = std::conditional_t<SMALL, floatx4, floatx16>;
+    constexpr int ACCV = SMALL ? 4 : 16;
+    Acc acc[TM][TN];
 #pragma unroll
     for (int a = 0; a < TM; ++a)
 #pragma unroll
         for (int b = 0; b < TN; ++b)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
+            for (int v = 0; v < ACCV; ++v) acc[a][b][v] = 0.0f;
 
     float ra[NA], rb[NB];
     // Gathered B: float offsets of the rows of the step being loaded (uniform), and of the step after it.  The
@@ -338,52 +348,93 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         // (valid, cached) rather than branching around the loads.
         if (more) step_bases(ga, gb, shift);
 
-        // MFMA operands: 8 reduction indices per lane and block, two 128-bit reads.
-        float4 av[TM][2], bv[TN][2];
+        // What every slice of a step does besides its MFMAs: its share of the next step's loads, and the row
+        // offsets of the step after that (requested once every LDS operand of this step has arrived, so that the
+        // scalar loads share the wait counter with no outstanding LDS read; taken delivery of two slices later,
+        // still under this step's MFMAs).
+        constexpr int SLICES = 8;
+        auto slice_tail = [&](auto slice_tag) {
+            constexpr int slice = decltype(slice_tag)::value;
 #pragma unroll
-        for (int h2 = 0; h2 < 2; ++h2) {
+            for (int u = 0; u < UA; ++u)
+                if (u * SLICES / UA == slice) load_unit(std::integral_constant<int, KA>{}, ga, g.sA, voffA, ra, u);
+#pragma unroll
+            for (int u = 0; u < UB; ++u)
+                if (u * SLICES / UB == slice) load_unit(std::integral_constant<int, LB>{}, gb, g.sB, voffB, rb, u);
+            if (slice == 5) {
+                int pos = ld_r0 + BK;
+                if (RED && pos >= g.R) pos = 0;
+                fetch_rows(pos);
+            }
+            if (!RED && slice == 7) pin_rows();
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        auto component = [](const float4 &v, int e) { return e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w; };
+
+        if constexpr (SMALL) {
+            // 16x16 blocks: lane (x, q) reads r = 4q .. 4q+3 of its row and column with one 128-bit read each, and
+            // MFMA e takes r = 4q + e from quarter-wave q.
+            const int q4 = lane >> 4, l16 = lane & 15;
+            float4 av[TM], bv[TN];
 #pragma unroll
             for (int a = 0; a < TM; ++a)
-                av[a][h2] = *reinterpret_cast<const float4 *>(
-                    &As[buf][wm * (TM * 32) + a * 32 + l32][RowA::col(l32, 8 * half + 4 * h2)]);
+                av[a] = *reinterpret_cast<const float4 *>(&As[buf][a * 16 + l16][RowA::col(l16, 4 * q4)]);
 #pragma unroll
             for (int b = 0; b < TN; ++b)
-                bv[b][h2] = *reinterpret_cast<const float4 *>(
-                    &Bs[buf][wn * (TN * 32) + b * 32 + l32][RowB::col(l32, 8 * half + 4 * h2)]);
-        }
+                bv[b] = *reinterpret_cast<const float4 *>(&Bs[buf][wn * (TN * 16) + b * 16 + l16][RowB::col(l16, 4 * q4)]);
+            auto half_slice = [&](auto e_tag, auto bh_tag) {
+                constexpr int e = decltype(e_tag)::value, bh = decltype(bh_tag)::value;
 #pragma unroll
-        for (int h2 = 0; h2 < 2; ++h2) {
+                for (int a = 0; a < TM; ++a)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                constexpr int SLICES = 8;
-                const int slice = h2 * 4 + e;
+                    for (int b = bh * (TN / 2); b < (bh + 1) * (TN / 2); ++b)
+                        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(component(av[a], e), component(bv[b], e),
+                                                                         acc[a][b], 0, 0, 0);
+                slice_tail(std::integral_constant<int, e * 2 + bh>{});
+            };
+            using std::integral_constant;
+            half_slice(integral_constant<int, 0>{}, integral_constant<int, 0>{});
+            half_slice(integral_constant<int, 0>{}, integral_constant<int, 1>{});
+            half_slice(integral_constant<int, 1>{}, integral_constant<int, 0>{});
+            half_slice(integral_constant<int, 1>{}, integral_constant<int, 1>{});
+            half_slice(integral_constant<int, 2>{}, integral_constant<int, 0>{});
+            half_slice(integral_constant<int, 2>{}, integral_constant<int, 1>{});
+            half_slice(integral_constant<int, 3>{}, integral_constant<int, 0>{});
+            half_slice(integral_constant<int, 3>{}, integral_constant<int, 1>{});
+        } else {
+            // MFMA operands: 8 reduction indices per lane and block, two 128-bit reads.
+            float4 av[TM][2], bv[TN][2];
 #pragma unroll
-                for (int a = 0; a < TM; ++a) {
-                    const float x = e == 0 ? av[a][h2].x : e == 1 ? av[a][h2].y : e == 2 ? av[a][h2].z : av[a][h2].w;
+            for (int h2 = 0; h2 < 2; ++h2) {
 #pragma unroll
-                    for (int b = 0; b < TN; ++b) {
-                        const float y =
-                            e == 0 ? bv[b][h2].x : e == 1 ? bv[b][h2].y : e == 2 ? bv[b][h2].z : bv[b][h2].w;
-                        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, acc[a][b], 0, 0, 0);
-                    }
-                }
+                for (int a = 0; a < TM; ++a)
+                    av[a][h2] = *reinterpret_cast<const float4 *>(
+                        &As[buf][wm * (TM * 32) + a * 32 + l32][RowA::col(l32, 8 * half + 4 * h2)]);
 #pragma unroll
-                for (int u = 0; u < UA; ++u)
-                    if (u * SLICES / UA == slice) load_unit(std::integral_constant<int, KA>{}, ga, g.sA, voffA, ra, u);
-#pragma unroll
-                for (int u = 0; u < UB; ++u)
-                    if (u * SLICES / UB == slice) load_unit(std::integral_constant<int, LB>{}, gb, g.sB, voffB, rb, u);
-                // Offsets of the step after the one being loaded: requested once every LDS operand of this step
-                // has arrived (the scalar loads then share the wait counter with no outstanding LDS read), taken
-                // delivery of two slices later, still under this step's MFMAs.
-                if (slice == 5) {
-                    int pos = ld_r0 + BK;
-                    if (RED && pos >= g.R) pos = 0;
-                    fetch_rows(pos);
-                }
-                if (!RED && slice == 7) pin_rows();
-                __builtin_amdgcn_sched_barrier(0);
+                for (int b = 0; b < TN; ++b)
+                    bv[b][h2] = *reinterpret_cast<const float4 *>(
+                        &Bs[buf][wn * (TN * 32) + b * 32 + l32][RowB::col(l32, 8 * half + 4 * h2)]);
             }
+            auto slice_of = [&](auto slice_tag) {
+                constexpr int slice = decltype(slice_tag)::value;
+                constexpr int h2 = slice / 4, e = slice % 4;
+#pragma unroll
+                for (int a = 0; a < TM; ++a)
+#pragma unroll
+                    for (int b = 0; b < TN; ++b)
+                        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(component(av[a][h2], e), component(bv[b][h2], e),
+                                                                         acc[a][b], 0, 0, 0);
+                slice_tail(slice_tag);
+            };
+            using std::integral_constant;
+            slice_of(integral_constant<int, 0>{});
+            slice_of(integral_constant<int, 1>{});
+            slice_of(integral_constant<int, 2>{});
+            slice_of(integral_constant<int, 3>{});
+            slice_of(integral_constant<int, 4>{});
+            slice_of(integral_constant<int, 5>{});
+            slice_of(integral_constant<int, 6>{});
+            slice_of(integral_constant<int, 7>{});
         }
         if (more) {
             stash(buf ^ 1, shift);
@@ -476,14 +527,18 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     };
     // The scattered store (see GemmProblem::scatter): rows are (plane, row phase, column phase) triples, columns
     // cells of a per-image grid; an element lands at a strided position of the image or is dropped.
+    // Block geometry of the accumulators: 32x32 blocks keep D[8*(v/4) + 4*(l/32) + v%4][l%32] in register v of lane
+    // l, 16x16 blocks D[4*(l/16) + v][l%16].
+    constexpr int BLK = SMALL ? 16 : 32;
     auto write_scatter = [&]() {
         const bool masked = g.mask != nullptr;
+        const int lcol = lane & (BLK - 1);
         long cbase[TN];  // float offset of the cell's phase-(0,0) pixel; may lie before the image (pH, pW)
         int hy[TN], wx[TN];
         bool own[TN];
 #pragma unroll
         for (int b = 0; b < TN; ++b) {
-            const int jg = j0 + wn * (TN * 32) + b * 32 + l32;
+            const int jg = j0 + wn * (TN * BLK) + b * BLK + lcol;
             own[b] = jg >= own_j0;
             unsigned im, n, y, x;
             g.divN.divmod((unsigned)jg, im, n);
@@ -495,10 +550,10 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         const long plane = (long)g.scat_H * g.scat_W;
 #pragma unroll
         for (int a = 0; a < TM; ++a) {
-            const int iu = i0 + wm * (TM * 32) + a * 32;
+            const int iu = i0 + wm * (TM * BLK) + a * BLK;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = iu + 8 * (v / 4) + (v % 4) + 4 * half;
+            for (int v = 0; v < ACCV; ++v) {
+                const int row = SMALL ? iu + 4 * (lane >> 4) + v : iu + 8 * (v / 4) + (v % 4) + 4 * half;
                 if (row < own_i0 || row >= g.scat_rows) continue;
                 unsigned c, rem, ph, pw;
                 g.divScatS.divmod((unsigned)row, c, rem);
@@ -518,20 +573,33 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     };
     using std::integral_constant;
     if constexpr (LB == LD_XC_GATHER && !RED) {
-        if (g.scatter) {
+        if (SMALL || g.scatter) {
             write_scatter();
             return;
         }
     }
-    if (g.nsplit > 1) {
-        if (edge_tile) write_out(integral_constant<int, 0>{}, integral_constant<bool, true>{});
-        else write_out(integral_constant<int, 0>{}, integral_constant<bool, false>{});
-    } else if (g.beta == 0.0f) {
-        if (edge_tile) write_out(integral_constant<int, 1>{}, integral_constant<bool, true>{});
-        else write_out(integral_constant<int, 1>{}, integral_constant<bool, false>{});
-    } else {
-        write_out(integral_constant<int, 2>{}, integral_constant<bool, true>{});
+    if constexpr (!SMALL) {
+        if (g.nsplit > 1) {
+            if (edge_tile) write_out(integral_constant<int, 0>{}, integral_constant<bool, true>{});
+            else write_out(integral_constant<int, 0>{}, integral_constant<bool, false>{});
+        } else if (g.beta == 0.0f) {
+            if (edge_tile) write_out(integral_constant<int, 1>{}, integral_constant<bool, true>{});
+            else write_out(integral_constant<int, 1>{}, integral_constant<bool, false>{});
+        } else {
+            write_out(integral_constant<int, 2>{}, integral_constant<bool, true>{});
+        }
     }
+}
+
+// The short-row variant (see the kernel's ROWS16): first operand along r, gathered B, scattered store, unsplit.
+template <int BN, int WGN, int ROWS16>
+int gemm_fast_short_rows_go(const GemmArgs &g, hipStream_t s) {
+    if (!g.scatter || g.nsplit != 1 || g.M != 64 || g.scat_rows > 16 * ROWS16)
+        return fail("gemm: the short-row kernel takes an unsplit scattered product of 64 padded rows, at most %d used",
+                    16 * ROWS16);
+    hipLaunchKernelGGL((gemm_fast_kernel<64, BN, 1, WGN, LD_RC_VEC, LD_XC_GATHER, false, ROWS16>), dim3(g.total),
+                       dim3(WGN * 64), 0, s, g);
+    return 0;
 }
 
 template <int BM, int BN, int WGM, int WGN, int LA, int LB, bool RED>

@@ -130,6 +130,7 @@ __device__ inline unsigned xcd_remap(unsigned id, unsigned total) {
 }
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 // How an operand tile travels from global memory to LDS.
 enum Loader {
@@ -149,6 +150,9 @@ int gemm_fast_256x128(const GemmArgs &g, int la, int lb, bool red, hipStream_t s
 int gemm_fast_64x64(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
 int gemm_fast_64x256(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
 int gemm_fast_64x128(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
+// Short-row variants: 48 of the tile's 64 rows multiplied (scattered products of a gathered B only).
+int gemm_fast_48x128(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
+int gemm_fast_48x256(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
 // The bounds-checked kernel for shapes smaller than a tile (gemm_generic.hip).
 int gemm_generic_64x64(const GemmArgs &g, bool a_rc, bool b_rc, bool red, hipStream_t s);
 

@@ -463,3 +463,58 @@ def test_strided_gradinput_integer_exact_and_untouched_neighbours(gt, gathered_r
     host = big.float()
     assert np.all(host[:guard] == 7.5) and np.all(host[guard + n:] == 7.5)
     assert np.array_equal(host[guard:guard + n].reshape(B, C, H, W), gi_ref)
+
+
+SHORT_ROWS = [
+    # B, C, H, W, kH, kW, pH, pW, sH, sW: C*sH*sW <= 48 rows in use of the product's single 64-row tile
+    (3, 3, 45, 38, 11, 11, 2, 2, 4, 4),    # 48 rows: the first-layer geometry
+    (3, 12, 21, 30, 3, 5, 1, 2, 2, 2),     # 48 rows from twelve planes
+    (3, 2, 50, 41, 7, 6, 3, 0, 5, 4),      # 40 rows, strides that differ
+    (2, 11, 33, 35, 4, 4, 1, 1, 3, 1),     # 33 rows: one row of the third block of sixteen
+    (4, 1, 64, 49, 9, 9, 4, 4, 4, 4),      # 16 rows
+]
+
+
+@pytest.mark.parametrize("tile", ["48x128", "48x256"])
+@pytest.mark.parametrize("masked", [False, True])
+@pytest.mark.parametrize("cfg", SHORT_ROWS)
+def test_strided_gradinput_short_row_kernel_integer_exact(gt, gathered_route, switches, cfg, masked, tile):
+    """The scattered product whose rows fit 48 of its 64-row tile runs on the kernel that multiplies 48 rows in
+    16x16 blocks.  Small integers make every sum exact, so the result must equal the oracle's bit for bit, with and
+    without the fused nn.Threshold mask, and nothing outside gradInput may be written."""
+    B, C, H, W, kH, kW, pH, pW, sH, sW = cfg
+    M = 24
+    geo = (kH, kW, pH, pW, sH, sW)
+    rng = rng_for(53)
+    ints = lambda lo, hi, shape: rng.integers(lo, hi + 1, size=shape).astype(np.float32)
+    x, w = ints(-2, 2, (B, C, H, W)), ints(-2, 2, (M, C * kH * kW))
+    Ho, Wo = (H + 2 * pH - kH) // sH + 1, (W + 2 * pW - kW) // sW + 1
+    go = ints(-2, 2, (B, M, Ho, Wo))
+    gi_ref, _ = oracle.conv_updateGradInput(go, w, x.shape, *geo)
+    if masked:
+        gi_ref = np.where(x > 0.0, gi_ref, np.float32(0.0))
+    m = gt.nn.SpatialConvolutionMM(C, M, kW, kH, sW, sH, 0, padW=pW, padH=pH)
+    m._assign("weight", w)
+    m.gpu()
+    n = B * C * H * W
+    guard = 4096
+    big = dev(gt, np.full(n + 2 * guard, 7.5, np.float32))
+    m.gradInput = big.narrow(0, guard, n).view(B, C, H, W)
+    switches("gemm_tile", tile)
+    dx, dgo = dev(gt, x), dev(gt, go)
+    gt.gputorch.synchronize()
+    gt.gputorch.prof_reset()
+    gt.gputorch.prof_enable(True)
+    try:
+        if masked:
+            m.inputThreshold = 0.0  # what Sequential.fuse() sets on a convolution that follows an nn.Threshold
+        gi = m.updateGradInput(dx, dgo).float()
+        gt.gputorch.synchronize()
+        labels = [k for k in gt.gputorch.prof_report() if k.startswith("gemm_conv_gradinput")]
+    finally:
+        gt.gputorch.prof_enable(False)
+        gt.gputorch.prof_reset()
+    assert len(labels) == 1 and "tile=%s " % tile in labels[0], labels
+    assert np.array_equal(gi, gi_ref)
+    host = big.float()
+    assert np.all(host[:guard] == 7.5) and np.all(host[guard + n:] == 7.5)
