@@ -70,6 +70,8 @@ struct TileCfg {
     // Short-row variant: the rows of the tile its wavefronts multiply (0: all of them).  It takes scattered products
     // of exactly one tile of rows, of which no more than this many are in use.
     int rows_used;
+    // The tile has no loader for a first operand contiguous along its rows.
+    bool a_rc_only;
 };
 
 // The 64 x 128 tile's wavefronts own 64 x 32 outputs, half the MFMAs per reduction step of the large tiles: it needs all
@@ -79,15 +81,16 @@ struct TileCfg {
 const double kOccNarrow[5] = {0.0, 0.50, 0.75, 0.88, 1.0};
 
 const TileCfg kCfgs[] = {
-    {"128x128", 128, 128, 4, {0.90, 0.90, 0.88, 0.86, 0.90}, gemm_fast_128x128, nullptr, 0, 0},
-    {"192x128", 192, 128, 3, {0.90, 0.90, 0.90, 0.86, 0.90}, gemm_fast_192x128, nullptr, 0, 0},
-    {"64x256", 64, 256, 3, {0.76, 0.74, 0.90, 0.74, 0.70}, gemm_fast_64x256, nullptr, 0, 0},
-    {"128x256", 128, 256, 2, {0.85, 0.87, 0.95, 0.85, 0.85}, gemm_fast_128x256, nullptr, 0, 0},
-    {"256x128", 256, 128, 2, {0.90, 0.75, 0.95, 0.75, 0.90}, gemm_fast_256x128, nullptr, 0, 0},
-    {"64x64", 64, 64, 4, {0.68, 0.60, 0.74, 0.60, 0.72}, gemm_fast_64x64, nullptr, 0, 0},
-    {"64x128", 64, 128, 4, {0.84, 0.78, 0.84, 0.78, 0.86}, gemm_fast_64x128, kOccNarrow, 128, 0},
-    {"48x128", 64, 128, 4, {0, 0, 0, 0, 0.84}, gemm_fast_48x128, kOccNarrow, 128, 48},
-    {"48x256", 64, 256, 3, {0, 0, 0, 0, 0.70}, gemm_fast_48x256, nullptr, 0, 48},
+    {"128x128", 128, 128, 4, {0.90, 0.90, 0.88, 0.86, 0.90}, gemm_fast_128x128, nullptr, 0, 0, false},
+    {"192x128", 192, 128, 3, {0.90, 0.90, 0.90, 0.86, 0.90}, gemm_fast_192x128, nullptr, 0, 0, false},
+    {"64x256", 64, 256, 3, {0.76, 0.74, 0.90, 0.74, 0.70}, gemm_fast_64x256, nullptr, 0, 0, false},
+    {"128x256", 128, 256, 2, {0.85, 0.87, 0.95, 0.85, 0.85}, gemm_fast_128x256, nullptr, 0, 0, false},
+    {"256x128", 256, 128, 2, {0.90, 0.75, 0.95, 0.75, 0.90}, gemm_fast_256x128, nullptr, 0, 0, false},
+    {"64x64", 64, 64, 4, {0.68, 0.60, 0.74, 0.60, 0.72}, gemm_fast_64x64, nullptr, 0, 0, false},
+    {"64x128", 64, 128, 4, {0.84, 0.78, 0.84, 0.78, 0.86}, gemm_fast_64x128, kOccNarrow, 128, 0, false},
+    {"48x128", 64, 128, 4, {0, 0, 0, 0, 0.84}, gemm_fast_48x128, kOccNarrow, 128, 48, false},
+    {"48x256", 64, 256, 3, {0, 0, 0, 0, 0.70}, gemm_fast_48x256, nullptr, 0, 48, false},
+    {"96x128", 96, 128, 4, {0.84, 0, 0.84, 0, 0.86}, gemm_fast_96x128, kOccNarrow, 128, 0, true},
 };
 
 inline long cdiv(long a, long b) { return (a + b - 1) / b; }
@@ -155,6 +158,7 @@ GemmPlan plan_gemm(const GemmProblem &p, int steps_total) {
         if (!fast_ok || p.M < c.bm || p.J < c.bn || !offsets_fit(c.bm, c.bn)) continue;
         if (force && std::strcmp(force, c.name) != 0) continue;
         if (!force && c.below_rows > 0 && p.M >= c.below_rows) continue;
+        if (c.a_rc_only && !p.a_rc) continue;
         if (c.rows_used > 0 && !(p.scatter && layout == 4 && p.M == c.bm && p.scat_rows <= c.rows_used)) continue;
         const long tiles = cdiv(p.M, c.bm) * cdiv(p.J, c.bn);
         int max_split = (int)(steps_total / 8 > 0 ? (steps_total / 8 < 256 ? steps_total / 8 : 256) : 1);

@@ -83,7 +83,12 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     constexpr int TM = SMALL ? ROWS16 : BM / WGM / 32, TN = SMALL ? BN / WGN / 16 : BN / WGN / 32;
     static_assert(!SMALL || (WGM == 1 && BM == 64 && ROWS16 <= 4 && LB == LD_XC_GATHER && !RED && TN % 2 == 0),
                   "the short-row variant: one row of wavefronts over a 64-row tile, gathered B, scattered store");
-    constexpr int NA = BM * BK / NT, NB = BN * BK / NT;
+    // A first operand along r whose 128-bit loads the threads do not divide (96 rows: 384 loads, 256 threads): the
+    // last round of loads is made by the leading wavefronts only (a uniform branch; wavefront w loads rows
+    // 16w .. 16w+15 of every 64).
+    constexpr bool PART_A = LA == LD_RC_VEC && (BM * BK) % (NT * 4) != 0;
+    constexpr int NA = PART_A ? (BM * BK + NT * 4 - 1) / (NT * 4) * 4 : BM * BK / NT, NB = BN * BK / NT;
+    static_assert(!PART_A || (NT == 256 && BM % 16 == 0), "partial loader shape");
     static_assert(BM % (WGM * 32) == 0 && BN % (WGN * 32) == 0, "wave tile must be whole 32x32 blocks");
     static_assert(NT % 16 == 0 && NA >= 4 && NB >= 4 && NA % 4 == 0 && NB % 4 == 0, "loader shape");
     // The kind the A loader really uses: x-contiguous with 192 rows goes block-wise.
@@ -192,6 +197,12 @@ __global__ __launch_bounds__(WGM *WGN * 64)
             for (int v = 0; v < ACCV; ++v) acc[a][b][v] = 0.0f;
 
     float ra[NA], rb[NB];
+    auto a_unit_live = [&](int u) { return !PART_A || u * (NT / 4) + 16 * wave < BM; };
+    auto always_live = [](int) { return true; };
+    if (PART_A) {
+#pragma unroll
+        for (int q = 0; q < NA; ++q) ra[q] = 0.0f;
+    }
     // Gathered B: float offsets of the rows of the step being loaded (uniform), and of the step after it.  The
     // latter are fetched (scalar loads) in the middle of a step, a whole step before they turn into addresses,
     // so that no step starts by waiting for its row offsets.
@@ -285,15 +296,16 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         }
     };
 
-    auto stash_one = [&](auto kind_tag, auto tile, int t_x, int t_r, const float *src, auto count_tag) {
+    auto stash_one = [&](auto kind_tag, auto tile, int t_x, int t_r, const float *src, auto count_tag, auto live) {
         constexpr int KIND = decltype(kind_tag)::value;
         using Row = LdsRow<KIND>;
         constexpr int CNT = decltype(count_tag)::value;
         if (KIND == LD_RC_VEC) {
 #pragma unroll
             for (int q = 0; q < CNT / 4; ++q)
-                *reinterpret_cast<float4 *>(&tile[t_x + q * (NT / 4)][Row::col(t_x + q * (NT / 4), t_r)]) =
-                    make_float4(src[q * 4], src[q * 4 + 1], src[q * 4 + 2], src[q * 4 + 3]);
+                if (live(q))
+                    *reinterpret_cast<float4 *>(&tile[t_x + q * (NT / 4)][Row::col(t_x + q * (NT / 4), t_r)]) =
+                        make_float4(src[q * 4], src[q * 4 + 1], src[q * 4 + 2], src[q * 4 + 3]);
         } else if (KIND == LD_RC_SCALAR) {
 #pragma unroll
             for (int q = 0; q < CNT; ++q) tile[t_x + q * (NT / 16)][Row::col(t_x + q * (NT / 16), t_r)] = src[q];
@@ -314,8 +326,8 @@ __global__ __launch_bounds__(WGM *WGN * 64)
             mask_one(std::integral_constant<int, KA>{}, a_r, ra, std::integral_constant<int, NA>{}, shift);
             mask_one(std::integral_constant<int, LB>{}, b_r, rb, std::integral_constant<int, NB>{}, shift);
         }
-        stash_one(std::integral_constant<int, KA>{}, As[buf], a_x, a_r, ra, std::integral_constant<int, NA>{});
-        stash_one(std::integral_constant<int, LB>{}, Bs[buf], b_x, b_r, rb, std::integral_constant<int, NB>{});
+        stash_one(std::integral_constant<int, KA>{}, As[buf], a_x, a_r, ra, std::integral_constant<int, NA>{}, a_unit_live);
+        stash_one(std::integral_constant<int, LB>{}, Bs[buf], b_x, b_r, rb, std::integral_constant<int, NB>{}, always_live);
     };
 
     // ---- prologue: first step ---------------------------------------------------------
@@ -325,7 +337,8 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         fetch_rows(ld_r0);
         step_bases(ga, gb, shift);
 #pragma unroll
-        for (int u = 0; u < UA; ++u) load_unit(std::integral_constant<int, KA>{}, ga, g.sA, voffA, ra, u);
+        for (int u = 0; u < UA; ++u)
+            if (a_unit_live(u)) load_unit(std::integral_constant<int, KA>{}, ga, g.sA, voffA, ra, u);
 #pragma unroll
         for (int u = 0; u < UB; ++u) load_unit(std::integral_constant<int, LB>{}, gb, g.sB, voffB, rb, u);
         stash(0, shift);
@@ -357,7 +370,8 @@ __global__ __launch_bounds__(WGM *WGN * 64)
             constexpr int slice = decltype(slice_tag)::value;
 #pragma unroll
             for (int u = 0; u < UA; ++u)
-                if (u * SLICES / UA == slice) load_unit(std::integral_constant<int, KA>{}, ga, g.sA, voffA, ra, u);
+                if (u * SLICES / UA == slice && a_unit_live(u))
+                    load_unit(std::integral_constant<int, KA>{}, ga, g.sA, voffA, ra, u);
 #pragma unroll
             for (int u = 0; u < UB; ++u)
                 if (u * SLICES / UB == slice) load_unit(std::integral_constant<int, LB>{}, gb, g.sB, voffB, rb, u);

@@ -150,6 +150,7 @@ int gemm_fast_256x128(const GemmArgs &g, int la, int lb, bool red, hipStream_t s
 int gemm_fast_64x64(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
 int gemm_fast_64x256(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
 int gemm_fast_64x128(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
+int gemm_fast_96x128(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);  // first operand along r only
 // Short-row variants: 48 of the tile's 64 rows multiplied (scattered products of a gathered B only).
 int gemm_fast_48x128(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);
 int gemm_fast_48x256(const GemmArgs &g, int la, int lb, bool red, hipStream_t s);

@@ -204,7 +204,7 @@ def test_gathered_conv_random_geometry(gt, gathered_route, cfg):
 
 
 @pytest.mark.parametrize("split", [1, 3])
-@pytest.mark.parametrize("tile", ["128x128", "192x128", "64x256", "128x256", "256x128", "64x64", "64x128"])
+@pytest.mark.parametrize("tile", ["128x128", "192x128", "64x256", "128x256", "256x128", "64x64", "64x128", "96x128"])
 def test_gathered_conv_every_tile_configuration(gt, gathered_route, tile, split, switches):
     """Every tile of the GEMM has its own gathering kernels (plain and reduction-batched); the library's choice
     would leave most of them to the large benchmark shapes, so each is forced here on a shape all of them fit."""

@@ -14,14 +14,14 @@ import zlib
 import numpy as np
 import pytest
 
-from helpers import rng_for
+from helpers import rng_for, uniform
 
 pytestmark = pytest.mark.gpu
 
 import oracle  # noqa: E402
 
 TILES = {"128x128": (128, 128), "192x128": (192, 128), "64x256": (64, 256), "128x256": (128, 256),
-         "256x128": (256, 128), "64x64": (64, 64), "64x128": (64, 128)}
+         "256x128": (256, 128), "64x64": (64, 64), "64x128": (64, 128), "96x128": (96, 128)}
 
 SHAPES = {
     # name: B, C, H, W, M, kH, kW, pH, pW, sH, sW
@@ -31,6 +31,8 @@ SHAPES = {
     "ragged_M200_K630_N195": (3, 70, 15, 13, 200, 3, 3, 1, 1, 1, 1),  # nothing a multiple of any tile
     "ragged_M130_K1188_N100": (7, 132, 12, 12, 130, 3, 3, 0, 0, 1, 1),
     "strided_M257_K588_N221": (2, 12, 40, 51, 257, 7, 7, 3, 3, 3, 3),
+    "first_layer_M96_N225": (3, 3, 70, 70, 96, 11, 11, 0, 0, 4, 4),    # 96 rows: the tile of 96 to 127 rows
+    "ragged_M110_K225_N144": (2, 25, 14, 14, 110, 3, 3, 0, 0, 1, 1),   # ... with an edge tile shifted back
 }
 
 
@@ -150,3 +152,35 @@ def test_integer_conv_exact_every_tile_and_split(gt, name, mode, tile, split, sw
     max_split = max(1, min(256, B * ((N + 15) // 16) // 8))
     ran = int(gw_label.split("split=")[1])
     assert ran == min(split, max_split), labels
+
+
+@pytest.mark.parametrize("mode", [0, 2], ids=["columns", "gathered"])
+def test_products_of_96_rows_take_the_96_row_tile(gt, mode):
+    """Products of 96 to 127 rows whose first operand lies along the reduction (forward and gradWeight on either
+    route) run on the 96 x 128 tile rather than on two 64-row tiles with a third of the work repeated: the
+    library's choice at the size of the reference benchmark's first layer (gpunn/test/benchmark.lua:73-80; the
+    results of this tile are checked on the small shapes above)."""
+    B, C, H, W, M, k = 16, 3, 128, 128, 96, 11
+    lib = gt._lib.lib
+    before = lib.thgpu_conv_get_mode()
+    assert lib.thgpu_conv_set_mode(mode) == 0
+    try:
+        m = gt.nn.SpatialConvolutionMM(C, M, k, k).gpu()
+        rng = rng_for(85)
+        dx = dev(gt, uniform(rng, (B, C, H, W)))
+        dgo = dev(gt, uniform(rng, (B, M, H - k + 1, W - k + 1)))
+        gt.gputorch.synchronize()
+        gt.gputorch.prof_reset()
+        gt.gputorch.prof_enable(True)
+        try:
+            m.forward(dx)
+            m.accGradParameters(dx, dgo, 1.0)
+            gt.gputorch.synchronize()
+            labels = {k2.split(" ")[0]: k2 for k2 in gt.gputorch.prof_report() if k2.startswith("gemm_conv")}
+        finally:
+            gt.gputorch.prof_enable(False)
+            gt.gputorch.prof_reset()
+    finally:
+        assert lib.thgpu_conv_set_mode(before) == 0
+    assert "tile=96x128 " in labels["gemm_conv_fwd"], labels
+    assert "tile=96x128 " in labels["gemm_conv_gradweight"], labels

@@ -250,7 +250,7 @@ def test_blas_gemm_integer_exact_beta0_ignores_nan_and_quick_returns(gt):
     assert np.array_equal(dc.float(), before * 3.0)
 
 
-GEMM_TILES = ["128x128", "192x128", "64x256", "128x256", "256x128", "64x64", "64x128"]
+GEMM_TILES = ["128x128", "192x128", "64x256", "128x256", "256x128", "64x64", "64x128", "96x128"]
 
 
 @pytest.mark.parametrize("split", [1, 3])
@@ -290,7 +290,9 @@ def test_blas_gemm_every_tile_configuration_exact(gt, tile, ta, tb, split, switc
     assert np.array_equal(dc.float().reshape(n, ldc), ref)
     assert len(labels) == 1
     ran = labels[0].split("tile=")[1].split(" ")[0]
-    assert ran == tile, labels
+    # the 96-row tile loads its first operand along the reduction only: op(B) = B, in BLAS terms
+    expect = "generic" if tile == "96x128" and tb == "t" else tile
+    assert ran == expect, labels
     assert ("split=%d" % split) in labels[0] or ran == "generic", labels
 
 
