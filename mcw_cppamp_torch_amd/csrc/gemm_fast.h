@@ -25,6 +25,8 @@
 //   * LDS is double buffered; the next tile's global loads are issued between
 //     the current tile's MFMAs and written to the other buffer afterwards: one
 //     barrier per reduction step.
+//   * Two variants for row counts the 32-row blocks fit badly: ROWS16 (16x16 blocks over the first 48 rows of a
+//     64-row tile, scattered products only) and the 96-row tile, whose first-operand loads the threads do not divide.
 //   * Between the MFMAs of a step there are memory and scalar instructions only.
 //     fp32 MFMAs and ordinary vector instructions share the SIMD's ALU (a v_add
 //     between two MFMAs costs 6 to 13 cycles of matrix time, measured), and a
