@@ -49,12 +49,27 @@ namespace thgpu {
 constexpr int LD_XC_BLOCK = 3;
 
 // LDS row layout by loader kind: pitch in floats, and the column at which element r of row x is stored.
-template <int KIND>
+//
+// Measured on this hardware with eight wavefronts issuing nothing else: a conflict-free ds_read_b128 takes 4 cycles
+// per wavefront and is served sixteen lanes at a time, where the sixteen are lanes 0-3, 12-15, 20-23, 24-27, then
+// 4-7, 8-11, 16-19, 28-31 (likewise in the upper half-wave), over 64 banks; a ds_write_b128 is served eight
+// consecutive lanes at a time, whose 16-byte units must differ modulo 128 bytes.  Hence:
+//   * 32x32 blocks (lane l reads row l%32, quarter pair l/32): rows written a column at a time (consecutive lanes =
+//     consecutive rows) are padded to 20 floats; rows written four lanes to a row keep 16 floats, quarter q of row x
+//     stored at q xor (x/4)%4.  Reads and writes of both are conflict-free (the conflict counter reads zero).
+//   * 16x16 blocks (SMALL16: lane l reads row l%16, quarter l/16): the row-written tile stores quarter q of row x
+//     at p(q) xor (x/4)%4 with p = (0, 3, 1, 2), conflict-free both ways (the plain xor puts rows 0-3 and rows 4-7
+//     of two lane quarters on the same banks).  The column-written tile keeps its 20-float rows: its writes need
+//     an odd pitch in 16-byte units, and no placement of four quarters in such a row also frees these reads of
+//     conflicts; they take 8 cycles instead of 4, two of a step's five operand reads.
+template <int KIND, bool SMALL16 = false>
 struct LdsRow {
     static constexpr bool kSwizzled = KIND == LD_RC_VEC;
     static constexpr int kPitch = kSwizzled ? GEMM_BK : GEMM_BK + 4;
     __device__ static __forceinline__ int col(int x, int r) {
-        return kSwizzled ? ((r & 3) | ((((r >> 2) ^ (x >> 2)) & 3) << 2)) : r;
+        if (!kSwizzled) return r;
+        const int q = SMALL16 ? (0x9C >> (2 * (r >> 2))) & 3 : r >> 2;
+        return (r & 3) | (((q ^ (x >> 2)) & 3) << 2);
     }
 };
 
@@ -103,8 +118,8 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     static_assert(!RED || (LA != LD_XC_SCALAR && LB != LD_XC_SCALAR),
                   "reduction batching needs r-contiguous or gathered operands");
 
-    using RowA = LdsRow<KA>;
-    using RowB = LdsRow<LB>;
+    using RowA = LdsRow<KA, SMALL>;
+    using RowB = LdsRow<LB, SMALL>;
     __shared__ __attribute__((aligned(16))) float As[2][BM][RowA::kPitch];
     __shared__ __attribute__((aligned(16))) float Bs[2][BN][RowB::kPitch];
 
@@ -300,7 +315,7 @@ __global__ __launch_bounds__(WGM *WGN * 64)
 
     auto stash_one = [&](auto kind_tag, auto tile, int t_x, int t_r, const float *src, auto count_tag, auto live) {
         constexpr int KIND = decltype(kind_tag)::value;
-        using Row = LdsRow<KIND>;
+        using Row = LdsRow<KIND, SMALL>;
         constexpr int CNT = decltype(count_tag)::value;
         if (KIND == LD_RC_VEC) {
 #pragma unroll
