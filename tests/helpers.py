@@ -170,7 +170,7 @@ MARGIN_LOG = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file
 
 def check_close(tag, got, ref, k_red):
     """Asserts the norm-wise bound 1e-4*sqrt(k_red) and puts the observed norm-wise and element-wise errors on
-    record (printed, and appended to gpurun_out/parity_margins.jsonl) so the margin under the bound is known."""
+    record (printed, and appended to the file MARGIN_LOG names) so the margin under the bound is known."""
     norm, elem, bound = rel_err(got, ref), elem_rel_err(got, ref), gemm_tol(k_red)
     rec = {"case": tag, "k_red": int(k_red), "bound": bound, "norm_rel_err": norm, "elem_rel_err": elem,
            "bound_used": norm / bound}
