@@ -295,7 +295,7 @@ FAMILIES = [("gemm_fast", "gemm"), ("gemm_generic", "gemm"), ("im2col", "im2col"
             ("maxpool_bwd", "maxpool_bwd"), ("maxpool_fwd", "maxpool_fwd"), ("threshold_fwd", "threshold_fwd"),
             ("threshold_bwd", "threshold_bwd"), ("split_reduce", "gemm_split_reduce"),
             ("gradbias_partial", "gradbias"), ("gradbias_final", "gradbias_final"), ("fill_kernel", "fill"),
-            ("pad_planes", "pad_planes"), ("flip_weight", "flip_weight"), ("phase_weight", "flip_weight")]
+            ("pad_planes", "pad_planes")]
 
 
 def _family(kernel_name):

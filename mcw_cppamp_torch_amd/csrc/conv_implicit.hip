@@ -37,64 +37,84 @@ namespace {
 
 // out[plane][y][x] = in[plane][y - pH][x - pW], zero outside.  A lane produces four consecutive
 // output elements (one 128-bit store; single stores at the end of an odd-sized buffer or into an unaligned one).
-__global__ __launch_bounds__(256) void pad_planes_kernel(const float *__restrict__ in, float *__restrict__ out,
-                                                         unsigned total, int H, int W, int pH, int pW, int Hp, int Wp,
-                                                         FastDiv divWp, FastDiv divHp, bool aligned) {
-    const unsigned idx = (blockIdx.x * 256u + threadIdx.x) * 4u;
-    if (idx >= total) return;
+struct PadJob {
+    const float *in;
+    float *out;
+    unsigned total;
+    int H, W, pH, pW, Hp, Wp;
+    FastDiv divWp, divHp;
+    bool aligned;
+};
+
+__device__ __forceinline__ void pad_four(const PadJob &j, unsigned block) {
+    const unsigned idx = (block * 256u + threadIdx.x) * 4u;
+    if (idx >= j.total) return;
     unsigned rest, x, plane, y;
-    divWp.divmod(idx, rest, x);
-    divHp.divmod(rest, plane, y);
+    j.divWp.divmod(idx, rest, x);
+    j.divHp.divmod(rest, plane, y);
     float v[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-        const int h = (int)y - pH, w = (int)x - pW;
+        const int h = (int)y - j.pH, w = (int)x - j.pW;
         v[q] = 0.0f;
-        if (h >= 0 && h < H && w >= 0 && w < W && idx + q < total) v[q] = in[((long)plane * H + h) * W + w];
-        if (++x == (unsigned)Wp) {
+        if (h >= 0 && h < j.H && w >= 0 && w < j.W && idx + q < j.total) v[q] = j.in[((long)plane * j.H + h) * j.W + w];
+        if (++x == (unsigned)j.Wp) {
             x = 0;
-            if (++y == (unsigned)Hp) {
+            if (++y == (unsigned)j.Hp) {
                 y = 0;
                 ++plane;
             }
         }
     }
-    if (aligned && idx + 4 <= total) {
-        *reinterpret_cast<float4 *>(out + idx) = make_float4(v[0], v[1], v[2], v[3]);
+    if (j.aligned && idx + 4 <= j.total) {
+        *reinterpret_cast<float4 *>(j.out + idx) = make_float4(v[0], v[1], v[2], v[3]);
     } else {
-        for (unsigned q = 0; idx + q < total; ++q) out[idx + q] = v[q];
+        for (unsigned q = 0; idx + q < j.total; ++q) j.out[idx + q] = v[q];
     }
 }
 
-// wt[c][m][kh][kw] = w[m][c][kH-1-kh][kW-1-kw]
-__global__ __launch_bounds__(256) void flip_weight_kernel(const float *__restrict__ w, float *__restrict__ wt, int M,
-                                                          int C, int kH, int kW) {
-    const unsigned idx = blockIdx.x * 256u + threadIdx.x;
-    const unsigned kk = (unsigned)(kH * kW);
-    if (idx >= (unsigned)M * C * kk) return;
-    const unsigned tap = idx % kk, cm = idx / kk;
-    const unsigned m = cm % M, c = cm / M;
-    const unsigned kh = tap / kW, kw = tap % kW;
-    wt[idx] = w[((long)m * C + c) * kk + (kH - 1 - kh) * kW + (kW - 1 - kw)];
-}
+__global__ __launch_bounds__(256) void pad_planes_kernel(const PadJob j) { pad_four(j, blockIdx.x); }
 
-// wt[(c, ph, pw)][(m, a', b')] = w[m][c][ph + sH*(A-1-a')][pw + sW*(Bk-1-b')], zero where that tap lies outside the
-// kernel and in the rows beyond C*sH*sW (the product's rows are padded to a whole tile).
-__global__ __launch_bounds__(256) void phase_weight_kernel(const float *__restrict__ w, float *__restrict__ wt, int M,
-                                                           int C, int kH, int kW, int sH, int sW, int A, int Bk,
-                                                           int rows, int rows_pad) {
-    const unsigned idx = blockIdx.x * 256u + threadIdx.x;
-    const unsigned R = (unsigned)(M * A * Bk);
-    if (idx >= (unsigned)rows_pad * R) return;
+// The kernel bank as the first operand of a gradInput product, one element per lane:
+//   unit stride:  wt[c][m][kh][kw] = w[m][c][kH-1-kh][kW-1-kw]
+//   strided:      wt[(c, ph, pw)][(m, a', b')] = w[m][c][ph + sH*(A-1-a')][pw + sW*(Bk-1-b')], zero where that tap lies
+//                 outside the kernel and in the rows beyond C*sH*sW (the product's rows are padded to a whole tile).
+struct WeightJob {
+    const float *w;
+    float *wt;
+    int M, C, kH, kW;
+    int sH, sW, A, Bk, rows, rows_pad;  // strided form only (sH = 0: unit stride)
+    unsigned count;                     // elements of wt
+};
+
+__device__ __forceinline__ void reorder_weight(const WeightJob &j, unsigned idx) {
+    if (idx >= j.count) return;
+    if (j.sH == 0) {
+        const unsigned kk = (unsigned)(j.kH * j.kW);
+        const unsigned tap = idx % kk, cm = idx / kk;
+        const unsigned m = cm % j.M, c = cm / j.M;
+        const unsigned kh = tap / j.kW, kw = tap % j.kW;
+        j.wt[idx] = j.w[((long)m * j.C + c) * kk + (j.kH - 1 - kh) * j.kW + (j.kW - 1 - kw)];
+        return;
+    }
+    const unsigned R = (unsigned)(j.M * j.A * j.Bk);
     const unsigned row = idx / R, r = idx % R;
     float v = 0.0f;
-    if (row < (unsigned)rows) {
-        const unsigned pw = row % sW, ph = (row / sW) % sH, c = row / (sW * sH);
-        const unsigned bb = r % Bk, aa = (r / Bk) % A, m = r / (Bk * A);
-        const unsigned kh = ph + sH * (A - 1 - aa), kw = pw + sW * (Bk - 1 - bb);
-        if (kh < (unsigned)kH && kw < (unsigned)kW) v = w[(((long)m * C + c) * kH + kh) * kW + kw];
+    if (row < (unsigned)j.rows) {
+        const unsigned pw = row % j.sW, ph = (row / j.sW) % j.sH, c = row / (j.sW * j.sH);
+        const unsigned bb = r % j.Bk, aa = (r / j.Bk) % j.A, m = r / (j.Bk * j.A);
+        const unsigned kh = ph + j.sH * (j.A - 1 - aa), kw = pw + j.sW * (j.Bk - 1 - bb);
+        if (kh < (unsigned)j.kH && kw < (unsigned)j.kW) v = j.w[(((long)m * j.C + c) * j.kH + kh) * j.kW + kw];
     }
-    wt[idx] = v;
+    j.wt[idx] = v;
+}
+
+// Both preparations of a gradInput product in one launch (they are independent, and the kernel bank alone is a
+// launch of a few microseconds of work): the first pad_blocks workgroups pad gradOutput, the rest re-order the bank.
+__global__ __launch_bounds__(256) void pad_planes_and_weights_kernel(const PadJob pad, unsigned pad_blocks,
+                                                                      const WeightJob wj) {
+    if (blockIdx.x < pad_blocks) pad_four(pad, blockIdx.x);
+    else reorder_weight(wj, (blockIdx.x - pad_blocks) * 256u + threadIdx.x);
 }
 
 // t[(c, kh, kw)] = c*plane + kh*pitch + kw
@@ -375,20 +395,41 @@ long conv_implicit_gradinput_scratch(long B, int C, int H, int W, int M, int kH,
     return B * M * (H + kH - 1L) * (W + kW - 1L) + (long)C * M * kH * kW;
 }
 
-// out[plane][y][x] = in[plane][y - top][x - left], zero outside the H x W source; out planes are Hp x Wp.
-static int pad_planes_into(const float *in, long planes, int H, int W, int top, int left, long Hp, long Wp, float *out) {
+// out[plane][y][x] = in[plane][y - top][x - left], zero outside the H x W source; out planes are Hp x Wp.  With a
+// weight job the same launch also re-orders the kernel bank.
+static int pad_planes_into(const float *in, long planes, int H, int W, int top, int left, long Hp, long Wp, float *out,
+                           const WeightJob *wj = nullptr) {
     hipStream_t s = stream();
     if (!s) return 1;
     const long total = planes * Hp * Wp;
-    if (total <= 0) return 0;
+    if (total <= 0 && !wj) return 0;
     if (total >= (1L << 31)) return fail("pad: %ld elements exceed 32-bit indexing", total);
     {
         const char *label = prof_enabled() ? prof_label("pad_planes planes=%ld %dx%d p=%dx%d", planes, H, W, top, left)
                                            : "pad_planes";
-        LaunchScope scope(label, 0.0, 4.0 * (total + planes * H * W));
-        hipLaunchKernelGGL(pad_planes_kernel, dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0, s, in, out,
-                           (unsigned)total, H, W, top, left, (int)Hp, (int)Wp, FastDiv((uint32_t)Wp),
-                           FastDiv((uint32_t)Hp), (reinterpret_cast<uintptr_t>(out) & 15) == 0);
+        const double wbytes = wj ? 4.0 * (wj->count + (double)wj->M * wj->C * wj->kH * wj->kW) : 0.0;
+        LaunchScope scope(label, 0.0, 4.0 * (total + planes * H * W) + wbytes);
+        PadJob pj;
+        pj.in = in;
+        pj.out = out;
+        pj.total = (unsigned)total;
+        pj.H = H;
+        pj.W = W;
+        pj.pH = top;
+        pj.pW = left;
+        pj.Hp = (int)Hp;
+        pj.Wp = (int)Wp;
+        pj.divWp = FastDiv((uint32_t)Wp);
+        pj.divHp = FastDiv((uint32_t)Hp);
+        pj.aligned = (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+        const unsigned pad_blocks = (unsigned)((total + 1023) / 1024);
+        if (wj) {
+            const unsigned wblocks = (wj->count + 255u) / 256u;
+            hipLaunchKernelGGL(pad_planes_and_weights_kernel, dim3(pad_blocks + wblocks), dim3(256), 0, s, pj, pad_blocks,
+                               *wj);
+        } else {
+            hipLaunchKernelGGL(pad_planes_kernel, dim3(pad_blocks), dim3(256), 0, s, pj);
+        }
     }
     return check_launch("pad_planes");
 }
@@ -453,15 +494,23 @@ static int conv_implicit_gradinput_strided(const float *gradOutput, const float 
     const int Ho = (H + 2 * pH - kH) / sH + 1, Wo = (W + 2 * pW - kW) / sW + 1;
     float *Q = scratch;
     float *Wt = scratch + B * M * (long)q.Hq * q.Wq;
-    if (pad_planes_into(gradOutput, B * M, Ho, Wo, q.A - 1, q.Bk - 1, q.Hq, q.Wq, Q)) return 1;
     const long nw = (long)q.rows_pad * M * q.A * q.Bk;
     if (nw >= (1L << 31)) return fail("SpatialConvolutionMM: kernel bank too large for the strided gradInput product");
-    {
-        LaunchScope scope("flip_weight", 0.0, 4.0 * (nw + (long)M * C * kH * kW));
-        hipLaunchKernelGGL(phase_weight_kernel, dim3((unsigned)((nw + 255) / 256)), dim3(256), 0, s, weight, Wt, M, C, kH,
-                           kW, sH, sW, q.A, q.Bk, q.rows, q.rows_pad);
-    }
-    if (check_launch("flip_weight")) return 1;
+    WeightJob wj;
+    wj.w = weight;
+    wj.wt = Wt;
+    wj.M = M;
+    wj.C = C;
+    wj.kH = kH;
+    wj.kW = kW;
+    wj.sH = sH;
+    wj.sW = sW;
+    wj.A = q.A;
+    wj.Bk = q.Bk;
+    wj.rows = q.rows;
+    wj.rows_pad = q.rows_pad;
+    wj.count = (unsigned)nw;
+    if (pad_planes_into(gradOutput, B * M, Ho, Wo, q.A - 1, q.Bk - 1, q.Hq, q.Wq, Q, &wj)) return 1;
     if (trim_tables()) return 1;
     GemmProblem p = gradinput_strided_problem(B, C, H, W, M, kH, kW, pH, pW, sH, sW);
     p.A = Wt;
@@ -487,14 +536,18 @@ int conv_implicit_gradinput(const float *gradOutput, const float *weight, float 
     const int Hq = Ho + 2 * qH, Wq = Wo + 2 * qW;  // = H + kH - 1, W + kW - 1
     float *Q = scratch;
     float *Wt = scratch + B * M * (long)Hq * Wq;
-    if (pad_planes_launch(gradOutput, B * M, Ho, Wo, qH, qW, Q)) return 1;
     const long nw = (long)M * C * kH * kW;
-    {
-        LaunchScope scope("flip_weight", 0.0, 8.0 * nw);
-        hipLaunchKernelGGL(flip_weight_kernel, dim3((unsigned)((nw + 255) / 256)), dim3(256), 0, s, weight, Wt, M, C, kH,
-                           kW);
-    }
-    if (check_launch("flip_weight")) return 1;
+    if (nw >= (1L << 31)) return fail("SpatialConvolutionMM: kernel bank too large for the gradInput product");
+    WeightJob wj;
+    wj.w = weight;
+    wj.wt = Wt;
+    wj.M = M;
+    wj.C = C;
+    wj.kH = kH;
+    wj.kW = kW;
+    wj.sH = wj.sW = wj.A = wj.Bk = wj.rows = wj.rows_pad = 0;
+    wj.count = (unsigned)nw;
+    if (pad_planes_into(gradOutput, B * M, Ho, Wo, qH, qW, Hq, Wq, Q, &wj)) return 1;
     if (trim_tables()) return 1;
     GemmProblem p = gradinput_problem(B, C, H, W, M, kH, kW, pH, pW);
     p.A = Wt;
