@@ -37,6 +37,8 @@ Other modes
   --workload ref_benchmark   the reference's own micro-benchmark (gpunn/test/benchmark.lua:7-91): seven single
                              layers, updateOutput / updateGradInput / accGradParameters timed separately and
                              reported with its GFLOP/s formula (:118).
+  --workload plan_check      the library's GEMM tile/split choice against every forced configuration, per layer and
+                             pass of the three stacks and the reference benchmark set (a few minutes).
   --workload hbm_sweep       GB/s of the HBM-bound kernels at the stack's geometries as the launch size grows.
   --summarise kernel-trace|traffic|mfma ...   turns rocprofv3 CSV output into the text summaries kept under
                              profiles/ (see summarise()).
@@ -210,6 +212,119 @@ def ref_benchmark(args, pkg):
         "config": {"workload": "seven single layers, three passes each timed on its own; value = all flops / all time",
                    "conv_route": args.conv_route, "device": gputorch.getDeviceProperties()["name"]},
         "layers": rows}))
+
+
+PLAN_TILES = ["128x128", "192x128", "64x256", "128x256", "256x128", "64x64", "64x128", "96x128", "48x128", "48x256"]
+PLAN_SPLITS = [1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16, 20, 24, 28, 32, 40, 48, 59, 64, 96, 128, 170, 256]
+
+
+def plan_check(args, pkg):
+    """How good is the library's own (tile, split) choice?  For every convolution of the AlexNet-, OverFeat- and
+    VGG-A-style stacks and of the reference's benchmark set, and every pass, the pass is timed with the library's
+    choice and with every tile configuration and reduction split forced in turn (the switches of thgpu_debug_set);
+    a row gives the choice, the fastest forced configuration, and the ratio of their times (pad copies, split
+    reduction and bias gradient of the pass included on both sides)."""
+    import numpy as np
+
+    from mcw_cppamp_torch_amd import gputorch, nn, stacks
+
+    lib = pkg._lib.lib
+    rng = np.random.Generator(np.random.PCG64(78))
+    shapes = []  # (tag, B, C, H, W, M, kH, kW, sH, sW, pH, pW)
+    for name in ("alexnet", "overfeat", "vgg_a"):
+        cfg = stacks.STACKS[name]
+        for l, (C, H, W), _ in stacks.trace_shapes(cfg["layers"], cfg["input"]):
+            if l[0] == "conv":
+                shapes.append((name, cfg["batch"], C, H, W, l[2], l[4], l[3], l[6], l[5], l[8], l[7]))
+    for ni, no, kw, kh, iw, ih, bs, dw, dh in REF_BENCHMARK_RUNS:
+        shapes.append(("ref_benchmark", bs, ni, ih, iw, no, kh, kw, dh, dw, 0, 0))
+    only = set(args.plan_stacks.split(",")) if args.plan_stacks else None
+    seen, rows = set(), []
+
+    def set_plan(tile, split):
+        lib.thgpu_debug_set(b"gemm_tile", tile.encode() if tile else None)
+        lib.thgpu_debug_set(b"gemm_split", str(split).encode() if split else None)
+
+    for tag, B, C, H, W, M, kH, kW, sH, sW, pH, pW in shapes:
+        key = (B, C, H, W, M, kH, kW, sH, sW, pH, pW)
+        if key in seen or (only and tag not in only):
+            continue
+        seen.add(key)
+        m = nn.SpatialConvolutionMM(C, M, kW, kH, sW, sH, 0, padW=pW, padH=pH, rng=rng).gpu()
+        x = pkg.FloatTensor(rng.standard_normal((B, C, H, W)).astype(np.float32)).gpu()
+        o = m.forward(x)
+        passes = (("updateOutput", "gemm_conv_fwd", lambda: m.updateOutput(x)),
+                  ("updateGradInput", "gemm_conv_gradinput", lambda: m.updateGradInput(x, o)),
+                  ("accGradParameters", "gemm_conv_gradweight", lambda: m.accGradParameters(x, o)))
+
+        def timed(call, label_key, reps):
+            """(ms per call, the GEMM's tile and split) for the plan currently set, or None when it cannot run."""
+            try:
+                call()
+                gputorch.synchronize()
+                gputorch.prof_reset()
+                gputorch.prof_enable(True)
+                call()
+                gputorch.synchronize()
+                labels = [k for k in gputorch.prof_report() if k.startswith(label_key)]
+                gputorch.prof_enable(False)
+                gputorch.prof_reset()
+                t0 = time.perf_counter()
+                for _ in range(reps):
+                    call()
+                gputorch.synchronize()
+                ms = (time.perf_counter() - t0) / reps * 1e3
+            except pkg.THGPUError:
+                gputorch.prof_enable(False)
+                gputorch.prof_reset()
+                return None
+            cfg = labels[0].split("tile=")[1] if labels else "?"
+            return ms, cfg
+
+        for pname, label_key, call in passes:
+            set_plan(None, None)
+            for _ in range(3):
+                call()
+            auto = min(timed(call, label_key, args.steps) for _ in range(2))
+            best = None
+            tried = set()
+            for tile in PLAN_TILES:
+                for split in PLAN_SPLITS:
+                    set_plan(tile, split)
+                    r = timed(call, label_key, max(2, args.steps // 4))
+                    if r is None or r[1] in tried or not r[1].startswith(tile + " "):
+                        continue
+                    tried.add(r[1])
+                    if best is None or r[0] < best[0]:
+                        best = r
+            set_plan(None, None)
+            if best is not None:  # the winner again, at the library choice's repetition count
+                tile, split = best[1].split(" split=")
+                set_plan(tile, int(split))
+                best = min(timed(call, label_key, args.steps) for _ in range(2))
+                set_plan(None, None)
+                again = min(timed(call, label_key, args.steps) for _ in range(2))
+                auto = min(auto, again)
+            row = {"stack": tag, "layer": "b%d %d->%d %dx%d k%dx%d s%d p%d" % (B, C, M, H, W, kH, kW, sH, pH),
+                   "pass": pname, "choice": auto[1], "choice_ms": round(auto[0], 4),
+                   "best_forced": best[1] if best else None, "best_forced_ms": round(best[0], 4) if best else None,
+                   "choice_over_best": round(auto[0] / best[0], 4) if best else None}
+            rows.append(row)
+            print("plan_check %(stack)s %(layer)s %(pass)s: choice %(choice)s %(choice_ms).4f ms, best forced "
+                  "%(best_forced)s %(best_forced_ms)s ms, ratio %(choice_over_best)s" % row, file=sys.stderr, flush=True)
+        del m, x, o
+    ratios = [r["choice_over_best"] for r in rows if r["choice_over_best"]]
+    tot_c = sum(r["choice_ms"] for r in rows if r["choice_over_best"])
+    tot_b = sum(r["best_forced_ms"] for r in rows if r["choice_over_best"])
+    print(json.dumps({
+        "metric": "time of the library's own GEMM tile/split choice over the fastest forced configuration, summed "
+                  "over all passes of all layers", "value": round(tot_c / tot_b, 4), "unit": "ratio", "n_gpus": 1,
+        "steps": args.steps, "warmup": 3, "ms_per_step": round(tot_c, 4), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "every convolution of the alexnet, overfeat, vgg_a stacks and the reference benchmark "
+                               "set, three passes each", "worst_ratio": max(ratios) if ratios else None,
+                   "device": gputorch.getDeviceProperties()["name"]},
+        "rows": rows}))
 
 
 def hbm_sweep(args, pkg):
@@ -439,7 +554,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="alexnet",
-                    choices=["alexnet", "overfeat", "vgg_a", "conv1_b16", "ref_benchmark", "hbm_sweep"])
+                    choices=["alexnet", "overfeat", "vgg_a", "conv1_b16", "ref_benchmark", "hbm_sweep", "plan_check"])
+    ap.add_argument("--plan-stacks", default=None,
+                    help="plan_check: comma-separated subset of alexnet,overfeat,vgg_a,ref_benchmark")
     ap.add_argument("--table", action="store_true", help="hbm_sweep: also print the rows as a table on stderr")
     ap.add_argument("--batch", type=int, default=None, help="override the workload's batch size")
     ap.add_argument("--cpu-sample-batch", type=int, default=128)
@@ -476,6 +593,8 @@ def main():
         return ref_benchmark(args, pkg)
     if args.workload == "hbm_sweep":
         return hbm_sweep(args, pkg)
+    if args.workload == "plan_check":
+        return plan_check(args, pkg)
 
     name = args.workload
     B = args.batch or stacks.STACKS[name]["batch"]
