@@ -126,6 +126,8 @@ CASES = [
     ({"gemm_tile": "128x128", "gemm_split": "2"}, ("conv", 128, 128, 3, 1, 1), 2),
     ({}, ("conv", 16, 64, 7, 3, 2), 2),                      # strided gathered gradInput: the scattered store
     ({"gemm_tile": "64x64"}, ("conv", 8, 64, 4, 2, 1), 2),   # ... with its rows padded to a tile
+    ({"gemm_tile": "96x128"}, ("conv", 96, 100, 3, 1, 1), 2),  # the 96-row tile: thresholded output, masked gradInput
+    ({"gemm_tile": "48x128"}, ("conv", 12, 64, 4, 2, 1), 2),   # the short-row kernel's masked scattered store
 ]
 
 
