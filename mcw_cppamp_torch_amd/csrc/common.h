@@ -70,6 +70,7 @@ struct Tuning {
     bool col2im_generic = false;
     bool pool_fwd_wave = false;   // the wavefront-level tile kernel instead of the direct forward kernel
     bool pool_bwd_direct = false;
+    bool gradbias_separate = false;  // the two-stage bias-gradient sum even where the gradWeight product could do it
 };
 const Tuning &tuning();
 

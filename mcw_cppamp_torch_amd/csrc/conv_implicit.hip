@@ -467,7 +467,8 @@ int conv_implicit_forward(const float *padded, const float *weight, const float 
 }
 
 int conv_implicit_gradweight(const float *padded, const float *gradOutput, float *gradWeight, long B, int C, int H,
-                             int W, int M, int kH, int kW, int pH, int pW, int sH, int sW, float scale) {
+                             int W, int M, int kH, int kW, int pH, int pW, int sH, int sW, float scale, float *gradBias,
+                             bool *bias_done) {
     const int Hp = H + 2 * pH, Wp = W + 2 * pW;
     const int Ho = (Hp - kH) / sH + 1, Wo = (Wp - kW) / sW + 1;
     if (trim_tables()) return 1;
@@ -479,6 +480,8 @@ int conv_implicit_gradweight(const float *padded, const float *gradOutput, float
     if (!p.rowtab || !p.coltab) return 1;
     p.C = gradWeight;
     p.alpha = scale;
+    p.rowsum = gradBias;  // gradBias[m] += scale * sum of gradOutput[.][m][.]: the row sums of this product's A
+    p.rowsum_done = bias_done;
     return gemm_launch(p);
 }
 

@@ -12,13 +12,40 @@ namespace {
 
 // C(i, j) = beta*C + alpha * sum_s ws[s][i][j] (+ bias[i]), s ascending; j is
 // mapped through (image, n) when the output is column batched.
-__global__ __launch_bounds__(256) void split_reduce_kernel(const float *__restrict__ ws, float *__restrict__ C,
+// The second job of a reduction launch: out[i] += alpha * sum over slots of ws[i][slot].  One wavefront per row:
+// lane l adds slots l, l + 64, ... in ascending order, then the lanes are added pairwise in a fixed tree, so the
+// result is reproducible.
+struct RowSumJob {
+    const float *ws;
+    float *out;
+    int M, slots;
+    float alpha;
+    unsigned first_block;  // workgroups from this one on work on the row sums, four rows each
+};
+
+__device__ __forceinline__ void rowsum_reduce(const RowSumJob &j, unsigned block) {
+    const int lane = threadIdx.x & 63;
+    const int row = (int)block * 4 + (int)(threadIdx.x >> 6);
+    if (row >= j.M) return;  // a whole wavefront
+    const float *src = j.ws + (long)row * j.slots;
+    float sum = 0.0f;
+    for (int s = lane; s < j.slots; s += 64) sum += src[s];
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) sum += __shfl_down(sum, d);
+    if (lane == 0) j.out[row] += j.alpha * sum;
+}
+
+__global__ __launch_bounds__(256) void split_reduce_kernel(const RowSumJob rs, const float *__restrict__ ws, float *__restrict__ C,
                                                            const float *__restrict__ bias, int M, int J, int N,
                                                            long sC, long bsC, FastDiv divJ, FastDiv divN, int nsplit,
                                                            float alpha, float beta, int act, float act_threshold,
                                                            float act_value, const float *__restrict__ mask,
                                                            float mask_threshold, int c_pitch, int mask_pitch,
                                                            long mask_sC, long mask_bsC, FastDiv divCW) {
+    if (rs.out && blockIdx.x >= rs.first_block) {
+        rowsum_reduce(rs, blockIdx.x - rs.first_block);
+        return;
+    }
     unsigned idx = blockIdx.x * blockDim.x + threadIdx.x;
     const unsigned total = (unsigned)M * (unsigned)J;
     if (idx >= total) return;
@@ -285,8 +312,13 @@ int gemm_launch(const GemmProblem &p) {
     const long total = (long)g.tilesM * g.tilesJ * g.nsplit;
     if (total <= 0 || total >= (1L << 31)) return fail("gemm: tile count %ld out of range", total);
     g.total = (unsigned)total;
-    if (g.nsplit > 1) {
-        const size_t need = (size_t)g.nsplit * p.M * p.J;
+    // Row sums of A ride along with a tiled reduction-batched product (never with the fixed workspace of the
+    // entry point that may not allocate: nothing there asks for them).
+    const bool rowsum = p.rowsum && best && red && !p.ws_fixed;
+    if (p.rowsum_done) *p.rowsum_done = rowsum;
+    const size_t rowsum_floats = rowsum ? (size_t)g.nsplit * g.tilesJ * p.M : 0;
+    if (g.nsplit > 1 || rowsum) {
+        const size_t need = (g.nsplit > 1 ? (size_t)g.nsplit * p.M * p.J : 0) + rowsum_floats;
         if (p.ws_fixed) {
             if ((long)need > p.ws_fixed_floats)
                 return fail("gemm: %zu floats of partial sums exceed the fixed workspace of %ld", need, p.ws_fixed_floats);
@@ -295,6 +327,7 @@ int gemm_launch(const GemmProblem &p) {
             g.ws = workspace(sizeof(float) * need);
         }
         if (!g.ws) return 1;
+        if (rowsum) g.rowsum_ws = g.ws + (need - rowsum_floats);
     }
 
     // ---- loaders: r-contiguous operands use 128-bit loads (4-byte alignment suffices) --------
@@ -313,11 +346,23 @@ int gemm_launch(const GemmProblem &p) {
     }
     if (rc) return rc;
     if (check_launch(p.tag)) return 1;
-    if (g.nsplit > 1) {
-        const long n = (long)p.M * p.J;
+    if (g.nsplit > 1 || rowsum) {
+        const long n = g.nsplit > 1 ? (long)p.M * p.J : 0;  // an unsplit product has stored its own result
+        RowSumJob rs;
+        std::memset(&rs, 0, sizeof(rs));
+        unsigned blocks = (unsigned)cdiv(n, 256);
+        if (rowsum) {
+            rs.ws = g.rowsum_ws;
+            rs.out = p.rowsum;
+            rs.M = p.M;
+            rs.slots = (int)(g.nsplit * g.tilesJ);
+            rs.alpha = p.alpha;
+            rs.first_block = blocks;
+            blocks += (unsigned)cdiv(p.M, 4);
+        }
         {
-            LaunchScope scope("gemm_split_reduce", 0.0, 4.0 * n * (g.nsplit + 2));
-            hipLaunchKernelGGL(split_reduce_kernel, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, s, g.ws, p.C, p.bias,
+            LaunchScope scope("gemm_split_reduce", 0.0, 4.0 * n * (g.nsplit + 2) + 4.0 * rowsum_floats);
+            hipLaunchKernelGGL(split_reduce_kernel, dim3(blocks), dim3(256), 0, s, rs, g.ws, p.C, p.bias,
                                p.M, p.J, g.N, p.sC, p.bsC, FastDiv((uint32_t)p.J), g.divN, g.nsplit, p.alpha,
                                p.beta, g.act, g.act_threshold, g.act_value, g.mask, g.mask_threshold, g.c_pitch,
                                g.mask_pitch, g.mask_sC, g.mask_bsC, g.divCW);

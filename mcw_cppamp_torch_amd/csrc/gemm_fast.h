@@ -213,6 +213,18 @@ __global__ __launch_bounds__(WGM *WGN * 64)
 #pragma unroll
             for (int v = 0; v < ACCV; ++v) acc[a][b][v] = 0.0f;
 
+    // Row sums of the first operand (GemmProblem::rowsum), reduction batching only.  The column tiles of a row of
+    // tiles all load the same first-operand tiles, so they share the work: the workgroup of column tile tj sums the
+    // steps whose index is tj modulo the number of column tiles, from the MFMA operands its first column of
+    // wavefronts holds in registers anyway (lane (x, h) holds r = 8h .. 8h+7 of row x).  A handful of vector adds
+    // every tilesJ-th step; the partial sums go to rowsum_ws[row][split * tilesJ + tj].
+    float bsum[TM];
+#pragma unroll
+    for (int a = 0; a < TM; ++a) bsum[a] = 0.0f;
+    const bool rs_on = RED && !SMALL && g.rowsum_ws != nullptr && wn == 0;
+    int rs_next = 0;
+    if (rs_on) rs_next = (int)(((unsigned)tj + g.tilesJ - (unsigned)step % g.tilesJ) % g.tilesJ);
+
     float ra[NA], rb[NB];
     auto a_unit_live = [&](int u) { return !PART_A || u * (NT / 4) + 16 * wave < BM; };
     auto always_live = [](int) { return true; };
@@ -374,6 +386,8 @@ __global__ __launch_bounds__(WGM *WGN * 64)
     auto one_step = [&](auto buf_tag, int s) {
         constexpr int buf = decltype(buf_tag)::value;
         const bool more = s + 1 < nsteps;
+        const bool rs_hit = rs_on && s == rs_next;  // uniform
+        if (rs_hit) rs_next += (int)g.tilesJ;
         // The last step has nothing to fetch; it re-reads the previous addresses
         // (valid, cached) rather than branching around the loads.
         if (more) step_bases(ga, gb, shift);
@@ -455,6 +469,13 @@ __global__ __launch_bounds__(WGM *WGN * 64)
                     for (int b = 0; b < TN; ++b)
                         acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(component(av[a][h2], e), component(bv[b][h2], e),
                                                                          acc[a][b], 0, 0, 0);
+                if constexpr (RED && (slice == 3 || slice == 7)) {
+                    if (rs_hit) {
+#pragma unroll
+                        for (int a = 0; a < TM; ++a)
+                            bsum[a] += (av[a][h2].x + av[a][h2].y) + (av[a][h2].z + av[a][h2].w);
+                    }
+                }
                 slice_tail(slice_tag);
             };
             using std::integral_constant;
@@ -602,6 +623,18 @@ __global__ __launch_bounds__(WGM *WGN * 64)
             }
         }
     };
+    if constexpr (RED && !SMALL) {
+        if (rs_on) {  // all of a wavefront or none
+            const long slots = (long)g.nsplit * g.tilesJ;
+            float *dst = g.rowsum_ws + ((long)split * g.tilesJ + tj);
+#pragma unroll
+            for (int a = 0; a < TM; ++a) {
+                const float total = bsum[a] + __shfl_xor(bsum[a], 32);  // the two halves hold different r
+                const int row = i0 + wm * (TM * 32) + a * 32 + l32;
+                if (half == 0 && row >= own_i0) dst[row * slots] = total;
+            }
+        }
+    }
     using std::integral_constant;
     if constexpr (LB == LD_XC_GATHER && !RED) {
         if (SMALL || g.scatter) {

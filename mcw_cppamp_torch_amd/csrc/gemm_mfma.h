@@ -66,6 +66,12 @@ struct GemmProblem {
     // the strides.  A mask is read at the same offsets (it is laid out exactly like C).  sC is unused.
     bool scatter = false;
     int scat_sH = 1, scat_sW = 1, scat_pH = 0, scat_pW = 0, scat_H = 0, scat_W = 0, scat_rows = 0;
+    // Reduction batching only: rowsum[i] += alpha * sum over the whole reduction of A(i, r), computed by the product's
+    // own workgroups from the first-operand tiles they load anyway (the bias gradient of a convolution is this sum
+    // over gradOutput).  *rowsum_done tells whether the launch took it on (a tiled reduction-batched kernel ran);
+    // when it is false the caller computes the sums itself.
+    float *rowsum = nullptr;
+    bool *rowsum_done = nullptr;
     const char *tag = "gemm";     // name used by per-kernel timing
     // Flops the per-kernel timing credits the launch with; 0 means the product's own 2*M*J*R*nb.  A
     // convolution pass sets its algorithmic 2*M*N*K*B here, which a gathered gradInput product (one
@@ -116,6 +122,7 @@ struct GemmArgs {
     int scatter;  // see GemmProblem
     int scat_sH, scat_sW, scat_pH, scat_pW, scat_H, scat_W, scat_rows;
     FastDiv divScatS, divScatW;  // a row index by sH*sW and its remainder by sW
+    float *rowsum_ws;            // partial row sums of A, [M][nsplit * tilesJ], or null
 };
 
 // Workgroups are handed to the 8 XCDs round-robin by linear id.  Remap so that

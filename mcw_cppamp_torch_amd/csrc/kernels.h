@@ -58,8 +58,11 @@ struct OutputThreshold {
 int conv_implicit_forward(const float *padded, const float *weight, const float *bias, float *output, long B, int C,
                           int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW,
                           OutputThreshold act = OutputThreshold(), OutputLayout out = OutputLayout());
+// gradBias (may be null) receives scale * the sums of gradOutput over images and positions when the product can
+// compute them on the side; *bias_done says whether it did.
 int conv_implicit_gradweight(const float *padded, const float *gradOutput, float *gradWeight, long B, int C, int H,
-                             int W, int M, int kH, int kW, int pH, int pW, int sH, int sW, float scale);
+                             int W, int M, int kH, int kW, int pH, int pW, int sH, int sW, float scale, float *gradBias,
+                             bool *bias_done);
 int conv_implicit_gradinput(const float *gradOutput, const float *weight, float *scratch, float *gradInput, long B,
                             int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW,
                             InputMask mask = InputMask());

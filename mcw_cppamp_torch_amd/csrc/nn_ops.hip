@@ -353,10 +353,13 @@ int conv_acc_grad_parameters(THGPUTensor *input, THGPUTensor *gradOutput, THGPUT
             }
             padded = dptr(finput);
         }
+        // The bias gradient is the row sums of the product's first operand: the GEMM computes them on the side
+        // when it runs a tiled reduction-batched kernel; otherwise the two-stage sum does.
+        bool bias_done = false;
         if (conv_implicit_gradweight(padded, dptr(go), dptr(gradWeight), s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH,
-                                     dW, scale))
+                                     dW, scale, tuning().gradbias_separate ? nullptr : dptr(gradBias), &bias_done))
             return 1;
-        return gradbias_launch(dptr(go), dptr(gradBias), s.B, s.M, s.N, scale);
+        return bias_done ? 0 : gradbias_launch(dptr(go), dptr(gradBias), s.B, s.M, s.N, scale);
     }
     if (!(reuse && is_columns(finput, s) && tensor_backed(finput))) {
         if (s.batched)
@@ -366,6 +369,7 @@ int conv_acc_grad_parameters(THGPUTensor *input, THGPUTensor *gradOutput, THGPUT
         if (!tensor_ready(finput, s.B * s.K * s.N)) return fail("SpatialConvolutionMM: could not size finput");
         if (im2col_launch(dptr(in), s.B, s.C, s.H, s.W, kH, kW, padH, padW, dH, dW, dptr(finput))) return 1;
     }
+    bool bias_done = false;
     {
         // gradWeight[m][k] += scale * sum_b sum_n gradOutput[b][m][n] * finput[b][k][n]
         GemmProblem p;
@@ -388,9 +392,11 @@ int conv_acc_grad_parameters(THGPUTensor *input, THGPUTensor *gradOutput, THGPUT
         p.beta = 1.0f;
         p.tag = "gemm_conv_gradweight";
         p.flops = 2.0 * s.M * (double)s.N * s.K * s.B;
+        p.rowsum = tuning().gradbias_separate ? nullptr : dptr(gradBias);
+        p.rowsum_done = &bias_done;
         if (gemm_launch(p)) return 1;
     }
-    return gradbias_launch(dptr(go), dptr(gradBias), s.B, s.M, s.N, scale);
+    return bias_done ? 0 : gradbias_launch(dptr(go), dptr(gradBias), s.B, s.M, s.N, scale);
 }
 
 }  // namespace

@@ -184,3 +184,47 @@ def test_products_of_96_rows_take_the_96_row_tile(gt, mode):
         assert lib.thgpu_conv_set_mode(before) == 0
     assert "tile=96x128 " in labels["gemm_conv_fwd"], labels
     assert "tile=96x128 " in labels["gemm_conv_gradweight"], labels
+
+
+@pytest.mark.parametrize("mode", [0, 2], ids=["columns", "gathered"])
+@pytest.mark.parametrize("name", ["second_layer_N729", "ragged_M130_K1188_N100", "first_layer_M96_N225"])
+def test_bias_gradient_rides_on_the_gradweight_product(gt, name, mode, switches):
+    """gradBias is the row sums of the gradWeight product's first operand (gpunn-impl/SpatialConvolutionMM.cpp:413-417
+    computes it with a gemv against ones): the tiled reduction-batched kernels sum it on the side and the reduction
+    launch finishes it, so no bias-gradient kernel of its own runs; the gradbias_separate switch brings the two-stage
+    sum back.  Both are exact on integers (checked inside run())."""
+    def kernels(separate):
+        switches("gradbias_separate", "1" if separate else None)
+        B, C, H, W, M, kH, kW, pH, pW, sH, sW = SHAPES[name]
+        x, w, b, go, gw0, gb0, out, gi, gw, gb = case(name)
+        lib = gt._lib.lib
+        before = lib.thgpu_conv_get_mode()
+        assert lib.thgpu_conv_set_mode(mode) == 0
+        try:
+            m = gt.nn.SpatialConvolutionMM(C, M, kW, kH, sW, sH, 0, padW=pW, padH=pH)
+            m._assign("weight", w)
+            m._assign("bias", b)
+            m.gradWeight[...] = gw0
+            m.gradBias[...] = gb0
+            m.gpu()
+            dx, dgo = dev(gt, x), dev(gt, go)
+            m.forward(dx)
+            gt.gputorch.synchronize()
+            gt.gputorch.prof_reset()
+            gt.gputorch.prof_enable(True)
+            try:
+                m.accGradParameters(dx, dgo, 2.0)
+                gt.gputorch.synchronize()
+                labels = sorted(gt.gputorch.prof_report())
+            finally:
+                gt.gputorch.prof_enable(False)
+                gt.gputorch.prof_reset()
+            assert np.array_equal(m.gradBias.float(), gb) and np.array_equal(m.gradWeight.float(), gw)
+        finally:
+            assert lib.thgpu_conv_set_mode(before) == 0
+        return labels
+
+    fused, separate = kernels(False), kernels(True)
+    assert not any(l.startswith("gradbias") for l in fused), fused
+    assert any(l.startswith("gemm_split_reduce") for l in fused), fused
+    assert any(l.startswith("gradbias") for l in separate), separate
