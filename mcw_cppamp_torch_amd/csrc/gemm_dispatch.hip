@@ -35,6 +35,7 @@ __device__ __forceinline__ void rowsum_reduce(const RowSumJob &j, unsigned block
     if (lane == 0) j.out[row] += j.alpha * sum;
 }
 
+template <bool quarters>
 __global__ __launch_bounds__(256) void split_reduce_kernel(const RowSumJob rs, const float *__restrict__ ws, float *__restrict__ C,
                                                            const float *__restrict__ bias, int M, int J, int N,
                                                            long sC, long bsC, FastDiv divJ, FastDiv divN, int nsplit,
@@ -46,19 +47,34 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(const RowSumJob rs, c
         rowsum_reduce(rs, blockIdx.x - rs.first_block);
         return;
     }
-    unsigned idx = blockIdx.x * blockDim.x + threadIdx.x;
+    // With `quarters` the four wavefronts of a workgroup share 64 outputs, each adding a contiguous quarter of the
+    // partial sums (for few outputs and many splits: one lane per output would leave the GPU idle behind a long
+    // chain of loads); the quarters are then added in order.  Either way the order of the adds is fixed.
     const unsigned total = (unsigned)M * (unsigned)J;
-    if (idx >= total) return;
+    const unsigned wave = threadIdx.x >> 6;
+    unsigned idx = quarters ? blockIdx.x * 64u + (threadIdx.x & 63u) : blockIdx.x * blockDim.x + threadIdx.x;
+    const bool valid = idx < total;
+    if (!quarters && !valid) return;
+    const int per = quarters ? (nsplit + 3) / 4 : nsplit;
+    const int s_begin = quarters ? (int)wave * per : 0;
+    const int s_end = s_begin + per < nsplit ? s_begin + per : nsplit;
     // Eight partials are requested before the first is added; the adds stay in split order.
     float sum = 0.0f;
-    const float *src = ws + idx;
-    for (int s0 = 0; s0 < nsplit; s0 += 8) {
+    const float *src = ws + (valid ? idx : 0);
+    for (int s0 = s_begin; s0 < s_end; s0 += 8) {
         float v[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = s0 + u < nsplit ? src[(long)(s0 + u) * total] : 0.0f;
+        for (int u = 0; u < 8; ++u) v[u] = s0 + u < s_end ? src[(long)(s0 + u) * total] : 0.0f;
 #pragma unroll
         for (int u = 0; u < 8; ++u)
-            if (s0 + u < nsplit) sum += v[u];
+            if (s0 + u < s_end) sum += v[u];
+    }
+    if (quarters) {
+        __shared__ float part[4][64];
+        part[wave][threadIdx.x & 63u] = sum;
+        __syncthreads();
+        if (wave != 0 || !valid) return;
+        sum = ((part[0][threadIdx.x] + part[1][threadIdx.x]) + part[2][threadIdx.x]) + part[3][threadIdx.x];
     }
     unsigned i, j;
     divJ.divmod(idx, i, j);
@@ -350,7 +366,9 @@ int gemm_launch(const GemmProblem &p) {
         const long n = g.nsplit > 1 ? (long)p.M * p.J : 0;  // an unsplit product has stored its own result
         RowSumJob rs;
         std::memset(&rs, 0, sizeof(rs));
-        unsigned blocks = (unsigned)cdiv(n, 256);
+        // few outputs, many splits: four wavefronts per 64 outputs
+        const int quarters = (n > 0 && n < 128 * 1024 && g.nsplit >= 32) ? 1 : 0;
+        unsigned blocks = (unsigned)cdiv(n, quarters ? 64 : 256);
         if (rowsum) {
             rs.ws = g.rowsum_ws;
             rs.out = p.rowsum;
@@ -362,7 +380,8 @@ int gemm_launch(const GemmProblem &p) {
         }
         {
             LaunchScope scope("gemm_split_reduce", 0.0, 4.0 * n * (g.nsplit + 2) + 4.0 * rowsum_floats);
-            hipLaunchKernelGGL(split_reduce_kernel, dim3(blocks), dim3(256), 0, s, rs, g.ws, p.C, p.bias,
+            auto kernel = quarters ? split_reduce_kernel<true> : split_reduce_kernel<false>;
+            hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, s, rs, g.ws, p.C, p.bias,
                                p.M, p.J, g.N, p.sC, p.bsC, FastDiv((uint32_t)p.J), g.divN, g.nsplit, p.alpha,
                                p.beta, g.act, g.act_threshold, g.act_value, g.mask, g.mask_threshold, g.c_pitch,
                                g.mask_pitch, g.mask_sC, g.mask_bsC, g.divCW);
