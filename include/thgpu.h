@@ -447,7 +447,8 @@ int thgpu_conv_gathers(long B, int C, int H, int W, int M, int kW, int kH, int d
  *   mode 0: that route; finput and fgradInput hold the K x N columns as in the reference.
  *   mode 1 (initial): per layer and pass, the GEMM gathers its second operand from a zero-padded copy
  *           of the image and no columns exist, where the shape allows it and it is the faster route
- *           (layers with fewer than 512 output planes); the column route otherwise.
+ *           (forward and gradWeight: wherever a tiled kernel takes the product; gradInput: layers whose input
+ *           planes fill the 64-row tiles and that are padded, or strided ones); the column route otherwise.
  *   mode 2: gathered wherever the shape allows it.
  * On the gathered route finput holds the padded input ([B,] C, H+2padH, W+2padW) and fgradInput the
  * padded gradOutput followed by the flipped kernels; outputs and gradients are the same sums of the

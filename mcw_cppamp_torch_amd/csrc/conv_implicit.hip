@@ -350,16 +350,15 @@ static bool gradinput_fits(long B, int C, int H, int W, int M, int kH, int kW, i
     return gemm_tiled_fits(gradinput_problem(B, C, H, W, M, kH, kW, pH, pW));
 }
 
-// Where the gathered route pays (measured on the AlexNet-, OverFeat- and VGG-style layers): the column
-// traffic it saves is proportional to K*N, the GEMM time it costs (the gathered gradWeight product runs
-// about 8 % under the one on r-contiguous columns; a gradInput product with few output planes leaves the
-// column route's GEMM a short reduction) to M*K*N, so it wins for layers with fewer than about 512
-// output planes and is a wash or a loss above.  The gathered gradInput product has one row per input
-// plane, so it also wants C to fill its 64-row tiles.
+// Where the gathered route pays (measured on the AlexNet-, OverFeat- and VGG-style layers and the reference's
+// benchmark set).  Forward and gradWeight: wherever a tiled kernel takes the product -- the gathered products run at
+// the rate of those on columns (0.84 - 0.92 of the matrix peak on the 512- and 1024-plane layers, either way), and
+// the columns' trip through memory is saved.  gradInput: the gathered product has one row per input plane, so it
+// wants C to fill its 64-row tiles, and one column per input pixel, so it wants the layer padded (see below).
 bool conv_use_gathered(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
     const int mode = conv_mode();
     if (mode == 0 || !forward_fits(B, C, H, W, M, kH, kW, pH, pW, sH, sW)) return false;
-    return mode == 2 || M < 512;
+    return true;
 }
 
 bool conv_use_gathered_gradinput(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
@@ -372,7 +371,7 @@ bool conv_use_gathered_gradinput(long B, int C, int H, int W, int M, int kH, int
         // the input written and read back: it pays while that excess stays small.
         const PhaseGeom q = phase_geom(C, H, W, kH, kW, pH, pW, sH, sW);
         const double excess = (double)q.rows_pad * q.A * q.Bk / ((double)C * kH * kW);
-        return M < 512 && excess <= 2.0;
+        return excess <= 2.0;
     }
     const long rows = (C + 63L) / 64 * 64;
     // An unpadded (or lightly padded) layer has fewer output positions than input pixels, and the gathered
@@ -383,7 +382,7 @@ bool conv_use_gathered_gradinput(long B, int C, int H, int W, int M, int kH, int
     // still 9 % ahead) and 150 (columns 19 % ahead).
     const long Ho = H + 2L * pH - kH + 1, Wo = W + 2L * pW - kW + 1;
     const bool inflation_ok = ((long)H * W - Ho * Wo) * M <= 110 * Ho * Wo;
-    return M < 512 && rows * 8 <= C * 9L && inflation_ok;
+    return rows * 8 <= C * 9L && inflation_ok;
 }
 
 long conv_implicit_gradinput_scratch(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH,

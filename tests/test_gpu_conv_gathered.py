@@ -226,13 +226,15 @@ def test_gathered_conv_every_tile_configuration(gt, gathered_route, tile, split,
     assert rel_err(got["gradWeight"], gw_ref) < gemm_tol(B * H * W)
 
 
-def test_mode_1_gathers_narrow_layers_only(gt):
+def test_mode_1_gathers_where_a_tiled_kernel_takes_the_product(gt):
+    """The library's own choice: narrow and wide layers alike compute without columns; a layer too small for the
+    tiled kernels (fewer than 64 output planes) stays on the column route."""
     lib = gt._lib.lib
     before = lib.thgpu_conv_get_mode()
     assert lib.thgpu_conv_set_mode(1) == 0
     try:
         rng = rng_for(46)
-        for M, gathers in ((128, True), (512, False)):
+        for M, gathers in ((128, True), (512, True), (24, False)):
             B, C, H, W, kH, kW = 2, 64, 8, 8, 3, 3
             geo = (kH, kW, 1, 1, 1, 1)
             x, w, b = uniform(rng, (B, C, H, W)), uniform(rng, (M, C * kH * kW), -0.05, 0.05), uniform(rng, (M,))
