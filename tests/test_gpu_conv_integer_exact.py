@@ -228,3 +228,62 @@ def test_bias_gradient_rides_on_the_gradweight_product(gt, name, mode, switches)
     assert not any(l.startswith("gradbias") for l in fused), fused
     assert any(l.startswith("gemm_split_reduce") for l in fused), fused
     assert any(l.startswith("gradbias") for l in separate), separate
+
+
+def random_layers(n, seed):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    out = []
+    for _ in range(n):
+        kH, kW = int(rng.integers(1, 12)), int(rng.integers(1, 12))
+        sH, sW = int(rng.integers(1, 5)), int(rng.integers(1, 5))
+        pH, pW = int(rng.integers(0, kH)), int(rng.integers(0, kW))
+        H, W = int(rng.integers(max(kH, 8), 90)), int(rng.integers(max(kW, 8), 90))
+        B = int(rng.integers(1, 9))
+        C = int(rng.choice([1, 2, 3, 4, 6, 12, 16, 33, 64, 70]))
+        M = int(rng.choice([8, 24, 48, 64, 96, 100, 110, 127, 128, 130, 192]))
+        out.append((B, C, H, W, M, kH, kW, pH, pW, sH, sW))
+    return out
+
+
+@pytest.mark.parametrize("cfg", random_layers(60, 4242))
+def test_random_layers_integer_exact_on_every_route(gt, cfg):
+    """Seeded random layers (plane counts around the tile heights, kernels up to 11, strides up to 4) on integer data:
+    output, gradInput, gradWeight and gradBias equal the oracle's bit for bit on the column route, on the library's
+    choice and with everything gathered that can be."""
+    B, C, H, W, M, kH, kW, pH, pW, sH, sW = cfg
+    K = C * kH * kW
+    geo = (kH, kW, pH, pW, sH, sW)
+    rng = rng_for(zlib.crc32(repr(cfg).encode()) % 100000)
+    ints = lambda lo, hi, shape: rng.integers(lo, hi + 1, size=shape).astype(np.float32)
+    x, w, b = ints(-2, 2, (B, C, H, W)), ints(-2, 2, (M, K)), ints(-3, 3, (M,))
+    oracle.use_blas(True)
+    try:
+        out, finput = oracle.conv_updateOutput(x, w, b, *geo)
+        go = ints(-2, 2, out.shape)
+        gi, _ = oracle.conv_updateGradInput(go, w, x.shape, *geo)
+        gw0, gb0 = ints(-5, 5, (M, K)), ints(-5, 5, (M,))
+        gw, gb = gw0.copy(), gb0.copy()
+        oracle.conv_accGradParameters(go, finput, gw, gb, 2.0)
+    finally:
+        oracle.use_blas(False)
+    assert max(np.abs(out).max(), np.abs(gi).max(), np.abs(gw).max(), np.abs(gb).max()) < 2 ** 24
+    lib = gt._lib.lib
+    before = lib.thgpu_conv_get_mode()
+    try:
+        for mode in (0, 1, 2):
+            assert lib.thgpu_conv_set_mode(mode) == 0
+            print("layer", cfg, "mode", mode, flush=True)
+            m = gt.nn.SpatialConvolutionMM(C, M, kW, kH, sW, sH, 0, padW=pW, padH=pH)
+            m._assign("weight", w)
+            m._assign("bias", b)
+            m.gradWeight[...] = gw0
+            m.gradBias[...] = gb0
+            m.gpu()
+            dx, dgo = dev(gt, x), dev(gt, go)
+            assert np.array_equal(m.forward(dx).float(), out), "output, mode %d" % mode
+            assert np.array_equal(m.updateGradInput(dx, dgo).float(), gi), "gradInput, mode %d" % mode
+            m.accGradParameters(dx, dgo, 2.0)
+            assert np.array_equal(m.gradWeight.float(), gw), "gradWeight, mode %d" % mode
+            assert np.array_equal(m.gradBias.float(), gb), "gradBias, mode %d" % mode
+    finally:
+        assert lib.thgpu_conv_set_mode(before) == 0
