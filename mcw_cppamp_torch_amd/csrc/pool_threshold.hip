@@ -437,6 +437,113 @@ bool plan_pool_bwd(const PoolGeom &g, long planes, int TH, PoolBwdPlan &p) {
     return true;
 }
 
+// The cell kernel: the default for the window shapes of the benchmark stacks (3x3 stride 2, 2x2 stride 2).  A lane
+// owns the DH x DW pixels of one stride cell (y, x) = (h / DH, w / DW) of a plane.  Only the TH x TW =
+// ceil(KH/DH) x ceil(KW/DW) windows (y - a, x - b) can name one of them: window (y - a, x - b) reaches pixel
+// (ph, pw) of the cell when its saved argmax is (ky, kx) = (ph + a*DH, pw + b*DW).  The lane requests the three
+// window arrays of those windows and the mask of its pixels up front (lanes run along x, so every request is a
+// contiguous run; neighbouring cells share windows through the vector cache, as the forward kernel's lanes share
+// rows), then adds the gradients that hit each pixel with a and b descending, i.e. windows in (i ascending, j
+// ascending) order: the float addition order of the CPU module's scatter (mcw_nn/generic/SpatialMaxPooling.c:165-174).
+// A window that does not hit adds +0.0f, which leaves a sum that started from +0.0f unchanged bit for bit.  No LDS,
+// no barrier, no atomics, no zero-fill pass; 3*TH*TW + DH*DW loads and DH*DW stores per DH*DW pixels.
+struct __attribute__((packed, aligned(4))) pool_float2u {  // two floats at a 4-byte aligned address
+    float x, y;
+};
+
+template <int KH, int KW, int DH, int DW>
+__global__ __launch_bounds__(256) void maxpool_bwd_cell_kernel(const float *__restrict__ gout,
+                                                               const float *__restrict__ indy,
+                                                               const float *__restrict__ indx,
+                                                               float *__restrict__ gin, const PoolGeom g,
+                                                               const FastDiv divXc, const FastDiv divCells, int Xc,
+                                                               unsigned total_cells, const InputMask mask) {
+    constexpr int TH = (KH + DH - 1) / DH, TW = (KW + DW - 1) / DW;
+    const unsigned cell = blockIdx.x * blockDim.x + threadIdx.x;
+    if (cell >= total_cells) return;
+    unsigned plane, rem, y, x;
+    divCells.divmod(cell, plane, rem);
+    divXc.divmod(rem, y, x);
+    const int h0 = (int)y * DH, w0 = (int)x * DW;
+    // ---- requests: the windows, then the mask -- every load unconditional, from an index clamped into its array
+    // (a load under a lane condition becomes a branch with its own wait, and the requests would go out one after
+    // the other); what a clamped index fetched is discarded by the selects below ------------------------------------
+    float wg[TH][TW], wy[TH][TW], wx[TH][TW];
+    bool win[TH][TW];
+    const long obase = (long)plane * g.Ho * g.Wo;
+#pragma unroll
+    for (int a = 0; a < TH; ++a)
+#pragma unroll
+        for (int b = 0; b < TW; ++b) {
+            const int i = (int)y - a, j = (int)x - b;
+            win[a][b] = i >= 0 && i < g.Ho && j >= 0 && j < g.Wo;
+            const int ic = i < 0 ? 0 : i < g.Ho ? i : g.Ho - 1, jc = j < 0 ? 0 : j < g.Wo ? j : g.Wo - 1;
+            const long o = obase + (long)ic * g.Wo + jc;
+            wg[a][b] = gout[o];
+            wy[a][b] = indy[o];
+            wx[a][b] = indx[o];
+        }
+    const long plane_px = (long)plane * g.H * g.W;
+    float mv[DH][DW];
+    if (mask.in) {
+#pragma unroll
+        for (int ph = 0; ph < DH; ++ph) {
+            const int h = h0 + ph < g.H ? h0 + ph : g.H - 1;
+            const float *m = mask.in + plane_px + (long)h * g.W;
+            if (DW == 2) {  // (W >= KW >= 2)
+                // one 64-bit load per row; the last cell of an odd row reads the pair that ends at its one pixel
+                const int wb = w0 + 1 < g.W ? w0 : g.W - 2;
+                const pool_float2u t = *reinterpret_cast<const pool_float2u *>(m + wb);
+                mv[ph][0] = wb == w0 ? t.x : t.y;
+                mv[ph][DW - 1] = t.y;
+            } else {
+#pragma unroll
+                for (int pw = 0; pw < DW; ++pw) mv[ph][pw] = m[w0 + pw < g.W ? w0 + pw : g.W - 1];
+            }
+        }
+    }
+    // ---- the adds: windows in (i, j) ascending order --------------------------------------------------------------
+    float acc[DH][DW];
+#pragma unroll
+    for (int ph = 0; ph < DH; ++ph)
+#pragma unroll
+        for (int pw = 0; pw < DW; ++pw) acc[ph][pw] = 0.0f;
+#pragma unroll
+    for (int a = TH - 1; a >= 0; --a)
+#pragma unroll
+        for (int b = TW - 1; b >= 0; --b) {
+            // the tap as a pixel of this cell; a window outside the plane names none
+            const int ky = win[a][b] ? (int)wy[a][b] - 1 - a * DH : -1, kx = (int)wx[a][b] - 1 - b * DW;
+#pragma unroll
+            for (int ph = 0; ph < DH; ++ph)
+#pragma unroll
+                for (int pw = 0; pw < DW; ++pw) {
+                    // taps beyond the window ((ph + a*DH, pw + b*DW) outside KH x KW) are never saved, so they never match
+                    if (ph + a * DH >= KH || pw + b * DW >= KW) continue;
+                    acc[ph][pw] += (ky == ph && kx == pw) ? wg[a][b] : 0.0f;
+                }
+        }
+    // ---- the cell's pixels leave row by row -----------------------------------------------------------------------
+#pragma unroll
+    for (int ph = 0; ph < DH; ++ph) {
+        if (h0 + ph >= g.H) continue;
+        float *dst = gin + plane_px + (long)(h0 + ph) * g.W + w0;
+#pragma unroll
+        for (int pw = 0; pw < DW; ++pw)
+            if (mask.in) acc[ph][pw] = mv[ph][pw] > mask.threshold ? acc[ph][pw] : 0.0f;
+        if (DW == 2 && w0 + 1 < g.W) {  // one 64-bit store per row: a wavefront writes whole runs of a row
+            pool_float2u t;
+            t.x = acc[ph][0];
+            t.y = acc[ph][DW - 1];
+            *reinterpret_cast<pool_float2u *>(dst) = t;
+        } else {
+#pragma unroll
+            for (int pw = 0; pw < DW; ++pw)
+                if (w0 + pw < g.W) dst[pw] = acc[ph][pw];
+        }
+    }
+}
+
 // The direct kernel, for geometries the tile kernel's plan does not take.  Every pixel visits the windows
 // covering it in (i ascending, j ascending) order.
 __global__ __launch_bounds__(256) void maxpool_bwd_direct_kernel(const float *__restrict__ gout,
@@ -715,8 +822,28 @@ int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int
     g.divDW = FastDiv((uint32_t)dW);
     const int th = (kH + dH - 1) / dH, tw = (kW + dW - 1) / dW;
     const double bytes = 4.0 * ((mask.in ? 2.0 : 1.0) * (double)total + 3.0 * ototal);
+    // The cell kernel takes the window shapes it is compiled for; the pool_bwd_tile and pool_bwd_direct switches force
+    // the LDS tile kernel and the direct kernel (testing and tuning aids).
+    const bool cell_shape = (kH == 3 && kW == 3 && dH == 2 && dW == 2) || (kH == 2 && kW == 2 && dH == 2 && dW == 2);
+    if (cell_shape && !tuning().pool_bwd_direct && !tuning().pool_bwd_tile && Ho > 0 && Wo > 0) {
+        const long Yc = (H + dH - 1) / dH, Xc = (W + dW - 1) / dW;
+        const long cells = planes * Yc * Xc;
+        if (cells < (1L << 31)) {
+            {
+                LaunchScope scope(pool_label("maxpool_bwd", g, planes), 0.0, bytes);
+                const dim3 grid((unsigned)((cells + 255) / 256)), block(256);
+                const FastDiv divXc((uint32_t)Xc), divCells((uint32_t)(Yc * Xc));
+#define THGPU_POOL_BWD_CELL(KH_, KW_, DH_, DW_)                                                                     \
+    hipLaunchKernelGGL((maxpool_bwd_cell_kernel<KH_, KW_, DH_, DW_>), grid, block, 0, s, gout, indices,             \
+                       indices + ototal, gin, g, divXc, divCells, (int)Xc, (unsigned)cells, mask)
+                if (kH == 3) THGPU_POOL_BWD_CELL(3, 3, 2, 2);
+                else THGPU_POOL_BWD_CELL(2, 2, 2, 2);
+#undef THGPU_POOL_BWD_CELL
+            }
+            return check_launch("maxpool_bwd");
+        }
+    }
     PoolBwdPlan plan;
-    // The pool_bwd_direct switch forces the direct kernel (a testing and tuning aid).
     if (!tuning().pool_bwd_direct && Ho > 0 && Wo > 0 && th * tw <= 64 && plan_pool_bwd(g, planes, th, plan)) {
         const long blocks = ((planes + plan.G - 1) / plan.G) * plan.tiles;
         if (blocks < (1L << 31)) {

@@ -152,10 +152,11 @@ def test_every_kernel_that_stores_a_masked_gradient_or_a_thresholded_output(gt, 
         assert lib.thgpu_conv_set_mode(before) == 0
 
 
-@pytest.mark.parametrize("direct", [None, "1"], ids=["tile", "direct"])
+@pytest.mark.parametrize("kernel", ["auto", "tile", "direct"])
 @pytest.mark.parametrize("pool", [(3, 2), (2, 2), (3, 1)])
-def test_masked_pooling_backward(gt, pool, direct, switches):
-    switches("pool_bwd_direct", direct)
+def test_masked_pooling_backward(gt, pool, kernel, switches):
+    switches("pool_bwd_direct", "1" if kernel == "direct" else None)
+    switches("pool_bwd_tile", "1" if kernel == "tile" else None)
     spec = [("conv", 3, 8, 3, 1, 1), ("relu",), ("pool",) + pool]
     x = uniform(rng_for(94), (3, 3, 29, 31))
     _, out_u, gi_u, _, grads_u, go = run(gt, spec, x, 95, False)

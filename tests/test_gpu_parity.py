@@ -307,12 +307,14 @@ POOLS = [(2, 3, 7, 7, 3, 3, 2, 2), (3, 2, 9, 8, 2, 2, 2, 2), (2, 2, 10, 11, 3, 2
          (3, 2, 40, 64, 3, 3, 1, 2), (2, 2, 33, 33, 2, 2, 1, 1), (1, 1, 64, 64, 64, 64, 1, 1)]
 
 
-@pytest.fixture(params=[None, "1"], ids=["auto", "direct"])
+@pytest.fixture(params=["auto", "direct", "tile"])
 def pool_bwd_kernel(request, switches):
-    """Runs a test with the library's own forward and backward kernel choice (direct forward, tile backward), then with
-    the other pair forced (wavefront-level tile forward, direct backward)."""
-    switches("pool_fwd_wave", request.param)
-    switches("pool_bwd_direct", request.param)
+    """Runs a test with the library's own forward and backward kernel choice (direct forward; cell backward where a
+    window shape has one, else the LDS tile kernel), then with the wavefront-level tile forward and the direct backward
+    kernel forced, then with the LDS tile backward kernel forced."""
+    switches("pool_fwd_wave", "1" if request.param == "direct" else None)
+    switches("pool_bwd_direct", "1" if request.param == "direct" else None)
+    switches("pool_bwd_tile", "1" if request.param == "tile" else None)
     return request.param
 
 
