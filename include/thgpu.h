@@ -62,7 +62,9 @@ typedef struct THGPUTensor {
 } THGPUTensor;
 
 /* Host-side TH types that appear in the copy signatures.  Same layouts
- * (TH/generic/THStorage.h:23-31, TH/generic/THTensor.h), host pointers. */
+ * (TH/generic/THStorage.h:23-31, TH/generic/THTensor.h), host pointers.  A translation unit that has included
+ * Torch's own TH.h (the luaT bindings do) already has them and skips these declarations. */
+#ifndef TH_INC
 #define THGPU_DECLARE_HOST_TYPES(Name, ctype)                                              \
     typedef struct TH##Name##Storage {                                                     \
         ctype *data;                                                                       \
@@ -88,6 +90,7 @@ THGPU_DECLARE_HOST_TYPES(Int, int)
 THGPU_DECLARE_HOST_TYPES(Long, long)
 THGPU_DECLARE_HOST_TYPES(Float, float)
 THGPU_DECLARE_HOST_TYPES(Double, double)
+#endif /* TH_INC */
 
 /* ---- runtime --------------------------------------------------------------- */
 
@@ -174,6 +177,12 @@ void THGPUStorage_retain(THGPUStorage *self);                         /* THCStor
 void THGPUStorage_free(THGPUStorage *self);                           /* THCStorage.cpp:118-140 */
 void THGPUStorage_resize(THGPUStorage *self, long size);              /* THCStorage.cpp:154-198: new buffer, D2D copy of min(old,new) */
 void THGPUStorage_fill(THGPUStorage *self, float value);              /* THCStorage.cpp:142-152 */
+
+/* Blocking copies of n floats between a host buffer and device memory, replacing gpuMemcpy
+ * (gputorch/lib/THC/copyHelpers.cpp:14-85) where a binding moves raw data itself: GPUStorage:write / :read stage the
+ * floats through host memory around THFile_writeFloatRaw / readFloatRaw (gputorch/Storage.cpp:15-31). */
+int thgpu_memcpy_h2d(float *dst_device, const float *src_host, long n);
+int thgpu_memcpy_d2h(float *dst_host, const float *src_device, long n);
 
 /* gputorch/lib/THC/THCStorageCopy.h:9-26, THCStorageCopy.cpp:5-75 */
 void THGPUStorage_rawCopy(THGPUStorage *self, float *src); /* src is a DEVICE pointer (THCStorageCopy.cpp:56-62) */
@@ -319,6 +328,15 @@ void THGPUTensor_addmm(THGPUTensor *self, float beta, THGPUTensor *t, float alph
                        THGPUTensor *mat2);
 void THGPUTensor_addr(THGPUTensor *self, float beta, THGPUTensor *t, float alpha, THGPUTensor *vec1,
                       THGPUTensor *vec2);
+
+/* gputorch/lib/THC/THCTensorMath.h:28,91-93 (THCTensorMath.cpp:269-280,1331-1465): the rest of what Torch's generic
+ * tensor binding calls (torch/generic/Tensor.c:405-454 `index`, `indexCopy`, `indexFill`; TensorOperator.c:120 `*`).
+ * dot sums in two fixed-shape stages (reruns are bit-identical) and blocks; the index operations take a HOST vector of
+ * 1-based indices and work slice by slice, like TH/generic/THTensorMath.c:69-176. */
+float THGPUTensor_dot(THGPUTensor *self, THGPUTensor *src);
+void THGPUTensor_indexCopy(THGPUTensor *res_, int dim, struct THLongTensor *indices, THGPUTensor *src);
+void THGPUTensor_indexFill(THGPUTensor *tensor, int dim, struct THLongTensor *index, float val);
+void THGPUTensor_indexSelect(THGPUTensor *tensor, THGPUTensor *src, int dim, struct THLongTensor *index);
 
 /* ---- BLAS ------------------------------------------------------------------ */
 

@@ -178,6 +178,12 @@ _SIGNATURES = {
     "THGPUTensor_addmv": (None, [TensorP, c_float, TensorP, c_float, TensorP, TensorP]),
     "THGPUTensor_addmm": (None, [TensorP, c_float, TensorP, c_float, TensorP, TensorP]),
     "THGPUTensor_addr": (None, [TensorP, c_float, TensorP, c_float, TensorP, TensorP]),
+    "THGPUTensor_dot": (c_float, [TensorP, TensorP]),
+    "THGPUTensor_indexSelect": (None, [TensorP, TensorP, c_int, ctypes.POINTER(HostTensor["Long"])]),
+    "THGPUTensor_indexCopy": (None, [TensorP, c_int, ctypes.POINTER(HostTensor["Long"]), TensorP]),
+    "THGPUTensor_indexFill": (None, [TensorP, c_int, ctypes.POINTER(HostTensor["Long"]), c_float]),
+    "thgpu_memcpy_h2d": (c_int, [f32p, f32p, c_long]),
+    "thgpu_memcpy_d2h": (c_int, [f32p, f32p, c_long]),
     "THGPUBlas_gemm": (None, [c_char, c_char, c_long, c_long, c_long, c_float, f32p, c_long, f32p, c_long,
                               c_float, f32p, c_long]),
     "THGPUBlas_axpy": (None, [c_long, c_float, f32p, c_long, f32p, c_long]),

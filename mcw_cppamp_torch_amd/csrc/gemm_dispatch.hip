@@ -462,6 +462,9 @@ extern "C" int thgpu_gemm_noalloc(char transa, char transb, long m, long n, long
     size_t cap = 0;
     float *ws = static_scratch(&cap);
     if (!ws) return fail("thgpu_gemm_noalloc: call thgpu_init() first (this entry point sets nothing up itself)");
+    // (dimensions are range-checked before they are multiplied)
+    if (m >= (1L << 31) || n >= (1L << 31) || k >= (1L << 31))
+        return fail("thgpu_gemm_noalloc: dimension exceeds 2^31");
     if (m > 0 && n > 0 && m * n > (long)cap)
         return fail("thgpu_gemm_noalloc: a result of %ld x %ld elements exceeds the limit of %zu elements (%zu MiB)", m,
                     n, cap, cap * sizeof(float) >> 20);

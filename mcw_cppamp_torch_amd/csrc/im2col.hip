@@ -784,11 +784,14 @@ extern "C" {
 
 int thgpu_im2col(const float *im, long B, int C, int H, int W, int kH, int kW, int padH, int padW, int sH, int sW,
                  float *col) {
+    // a null operand with a valid geometry would reach a launch and fault there
+    if (!im || !col) return fail("thgpu_im2col: null operand");
     return im2col_launch(im, B, C, H, W, kH, kW, padH, padW, sH, sW, col);
 }
 
 int thgpu_col2im(const float *col, long B, int C, int H, int W, int kH, int kW, int padH, int padW, int sH, int sW,
                  float *im) {
+    if (!im || !col) return fail("thgpu_col2im: null operand");
     return col2im_launch(col, B, C, H, W, kH, kW, padH, padW, sH, sW, im, InputMask());
 }
 

@@ -339,6 +339,20 @@ int thgpu_empty_cache(void) {
 
 long thgpu_cached_bytes(void) { return (long)g_cached_bytes; }
 
+int thgpu_memcpy_h2d(float *dst_device, const float *src_host, long n) {
+    if (n < 0) return fail("thgpu_memcpy_h2d: negative count");
+    if (n == 0) return 0;
+    if (!dst_device || !src_host) return fail("thgpu_memcpy_h2d: null pointer");
+    return copy_h2d(dst_device, src_host, n);
+}
+
+int thgpu_memcpy_d2h(float *dst_host, const float *src_device, long n) {
+    if (n < 0) return fail("thgpu_memcpy_d2h: negative count");
+    if (n == 0) return 0;
+    if (!dst_host || !src_device) return fail("thgpu_memcpy_d2h: null pointer");
+    return copy_d2h(dst_host, src_device, n);
+}
+
 }  // extern "C"
 
 extern "C" int thgpu_fill_many(THGPUTensor **tensors, int count, float value) {

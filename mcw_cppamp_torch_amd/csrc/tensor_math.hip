@@ -7,6 +7,8 @@
 // flags of THGPUBlas_gemm, anything else goes through a dense copy.
 #include "common.h"
 
+#include <vector>
+
 using namespace thgpu;
 
 namespace {
@@ -95,6 +97,58 @@ __global__ __launch_bounds__(256) void gemv_t_kernel(long m, long n, float alpha
     for (long j = lane; j < m; j += 64) sum += x[j * incx] * col[j];
     for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off, 64);
     if (lane == 0) y[i * incy] = beta * y[i * incy] + alpha * sum;
+}
+
+// dot product in two fixed-shape stages, so that reruns are bit-identical: every workgroup sums one contiguous chunk
+// (lanes strided over it, then a tree over the 256 lane sums), a single workgroup adds the chunk sums the same way.
+__global__ __launch_bounds__(256) void dot_partial_kernel(const float *__restrict__ a, const float *__restrict__ b,
+                                                          long n, long chunk, float *__restrict__ part) {
+    const long lo = (long)blockIdx.x * chunk;
+    const long hi = lo + chunk < n ? lo + chunk : n;
+    float sum = 0.0f;
+    for (long i = lo + threadIdx.x; i < hi; i += 256) sum += a[i] * b[i];
+    __shared__ float red[256];
+    red[threadIdx.x] = sum;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) part[blockIdx.x] = red[0];
+}
+
+__global__ __launch_bounds__(256) void dot_final_kernel(const float *__restrict__ part, int nparts,
+                                                        float *__restrict__ out) {
+    float sum = 0.0f;
+    for (int i = threadIdx.x; i < nparts; i += 256) sum += part[i];
+    __shared__ float red[256];
+    red[threadIdx.x] = sum;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[0] = red[0];
+}
+
+// The 1-based entries of a host index vector, checked against the size they index.
+bool host_indices(const THLongTensor *index, long limit, std::vector<long> &out, const char *who) {
+    const long n = index->size[0];
+    const long st = index->stride ? index->stride[0] : 1;
+    if (n > 0 && (!index->storage || !index->storage->data)) {
+        raise("%s: index tensor has no storage", who);
+        return false;
+    }
+    out.resize((size_t)n);
+    for (long i = 0; i < n; ++i) {
+        const long v = index->storage->data[index->storageOffset + i * st];
+        if (v < 1 || v > limit) {
+            raise("%s: index %ld out of range [1, %ld]", who, v, limit);
+            return false;
+        }
+        out[(size_t)i] = v - 1;
+    }
+    return true;
 }
 
 int launch_grid(long work) {
@@ -297,6 +351,101 @@ void THGPUTensor_addr(THGPUTensor *r_, float beta, THGPUTensor *t, float alpha, 
     THGPUTensor_free(x);
     THGPUTensor_free(y);
     THGPUTensor_freeCopyTo(r, r_);
+}
+
+// gputorch/lib/THC/THCTensorMath.cpp:269-280 (a Bolt inner product there).  Blocking: the value goes to the host.
+float THGPUTensor_dot(THGPUTensor *self, THGPUTensor *src) {
+    if (!self || !src) {
+        raise("THGPUTensor_dot: null tensor");
+        return 0.0f;
+    }
+    const long n = THGPUTensor_nElement(self);
+    THGPU_ARGCHECK(n == THGPUTensor_nElement(src), 2, "size do not match", 0.0f);
+    if (n == 0) return 0.0f;
+    hipStream_t st = stream();
+    if (!st) {
+        raise("%s", thgpu_last_error());
+        return 0.0f;
+    }
+    THGPUTensor *a = THGPUTensor_newContiguous(self);
+    THGPUTensor *b = THGPUTensor_newContiguous(src);
+    float result = 0.0f;
+    long parts = (n + 4095) / 4096;
+    if (parts > 1024) parts = 1024;
+    const long chunk = (n + parts - 1) / parts;
+    parts = (n + chunk - 1) / chunk;
+    float *ws = a && b && tensor_backed(a) && tensor_backed(b) ? workspace(sizeof(float) * (size_t)(parts + 1)) : nullptr;
+    if (ws) {
+        {
+            LaunchScope scope("dot", 2.0 * n, 8.0 * n);
+            hipLaunchKernelGGL(dot_partial_kernel, dim3((unsigned)parts), dim3(256), 0, st, THGPUTensor_data(a),
+                               THGPUTensor_data(b), n, chunk, ws);
+            hipLaunchKernelGGL(dot_final_kernel, dim3(1), dim3(256), 0, st, ws, (int)parts, ws + parts);
+        }
+        if (check_launch("dot") || copy_d2h(&result, ws + parts, 1)) raise("%s", thgpu_last_error());
+    } else {
+        raise("THGPUTensor_dot: %s", a && b ? thgpu_last_error() : "could not make the operands contiguous");
+    }
+    if (a) THGPUTensor_free(a);
+    if (b) THGPUTensor_free(b);
+    return result;
+}
+
+// Index operations along one dimension with a host vector of 1-based indices, slice by slice like
+// TH/generic/THTensorMath.c:69-176 (the reference's kernels: gputorch/lib/THC/THCTensorMath.cpp:1331-1465).
+void THGPUTensor_indexSelect(THGPUTensor *res_, THGPUTensor *src, int dim, THLongTensor *index) {
+    if (!res_ || !src || !index) return raise("THGPUTensor_indexSelect: null tensor");
+    THGPU_ARGCHECK(index->nDimension == 1, 3, "expecting vector of indices", );
+    THGPU_ARGCHECK(src->nDimension > 0, 2, "Source tensor is empty", );
+    THGPU_ARGCHECK(dim >= 0 && dim < src->nDimension, 4, "Indexing dim is out of bounds", );
+    std::vector<long> idx;
+    if (!host_indices(index, src->size[dim], idx, "indexSelect")) return;
+    std::vector<long> size(src->size, src->size + src->nDimension);
+    size[(size_t)dim] = (long)idx.size();
+    THLongStorage sz;
+    sz.data = size.data();
+    sz.size = (long)size.size();
+    THGPUTensor_resize(res_, &sz, nullptr);
+    for (size_t k = 0; k < idx.size(); ++k) {
+        THGPUTensor *d = THGPUTensor_newNarrow(res_, dim, (long)k, 1);
+        THGPUTensor *s = THGPUTensor_newNarrow(src, dim, idx[k], 1);
+        if (d && s) THGPUTensor_copy(d, s);
+        if (d) THGPUTensor_free(d);
+        if (s) THGPUTensor_free(s);
+    }
+}
+
+void THGPUTensor_indexCopy(THGPUTensor *res_, int dim, THLongTensor *index, THGPUTensor *src) {
+    if (!res_ || !src || !index) return raise("THGPUTensor_indexCopy: null tensor");
+    THGPU_ARGCHECK(index->nDimension == 1, 3, "expecting vector of indices", );
+    THGPU_ARGCHECK(src->nDimension > 0, 2, "Source tensor is empty", );
+    THGPU_ARGCHECK(dim >= 0 && dim < src->nDimension && dim < res_->nDimension, 4, "Indexing dim is out of bounds", );
+    THGPU_ARGCHECK(index->size[0] == src->size[dim], 4, "length of src.size[dim] is not equal to length of indices", );
+    std::vector<long> idx;
+    if (!host_indices(index, res_->size[dim], idx, "indexCopy")) return;
+    for (size_t k = 0; k < idx.size(); ++k) {
+        THGPUTensor *d = THGPUTensor_newNarrow(res_, dim, idx[k], 1);
+        THGPUTensor *s = THGPUTensor_newNarrow(src, dim, (long)k, 1);
+        if (d && s) THGPUTensor_copy(d, s);
+        if (d) THGPUTensor_free(d);
+        if (s) THGPUTensor_free(s);
+    }
+}
+
+void THGPUTensor_indexFill(THGPUTensor *res_, int dim, THLongTensor *index, float val) {
+    if (!res_ || !index) return raise("THGPUTensor_indexFill: null tensor");
+    THGPU_ARGCHECK(index->nDimension == 1, 3, "Index is supposed to be a vector", );
+    THGPU_ARGCHECK(res_->nDimension > 0, 2, "Source tensor is empty", );
+    THGPU_ARGCHECK(dim >= 0 && dim < res_->nDimension, 4, "Indexing dim is out of bounds", );
+    std::vector<long> idx;
+    if (!host_indices(index, res_->size[dim], idx, "indexFill")) return;
+    for (size_t k = 0; k < idx.size(); ++k) {
+        THGPUTensor *d = THGPUTensor_newNarrow(res_, dim, idx[k], 1);
+        if (d) {
+            THGPUTensor_fill(d, val);
+            THGPUTensor_free(d);
+        }
+    }
 }
 
 }  // extern "C"

@@ -461,6 +461,39 @@ class GPUTensor(object):
         _lib.check()
         return self
 
+    def dot(self, other):
+        """torch.dot / the `*` of two vectors (gputorch/torch/generic/TensorOperator.c:120)."""
+        v = lib.THGPUTensor_dot(self._p, other._p)
+        _lib.check()
+        return float(v)
+
+    @staticmethod
+    def _index_vector(index):
+        # a host LongTensor of 1-based indices, as the Lua methods take (gputorch/torch/generic/Tensor.c:393-456)
+        arr = np.ascontiguousarray(np.asarray(index, np.int64).reshape(-1))
+        return _host_tensor_struct(arr)
+
+    def index(self, dim, index):
+        """tensor:index(dim, index): a new tensor of the slices `index` names along `dim` (0-based here, entries of
+        `index` 1-based as in Lua)."""
+        _, th, keep = self._index_vector(index)
+        out = GPUTensor()
+        lib.THGPUTensor_indexSelect(out._p, self._p, dim, ctypes.byref(th))
+        _lib.check()
+        return out
+
+    def indexCopy(self, dim, index, src):
+        _, th, keep = self._index_vector(index)
+        lib.THGPUTensor_indexCopy(self._p, dim, ctypes.byref(th), src._p)
+        _lib.check()
+        return self
+
+    def indexFill(self, dim, index, value):
+        _, th, keep = self._index_vector(index)
+        lib.THGPUTensor_indexFill(self._p, dim, ctypes.byref(th), float(value))
+        _lib.check()
+        return self
+
     def __getitem__(self, idx):  # 0-based element access (slow, blocking)
         if np.isscalar(idx):
             idx = (idx,)

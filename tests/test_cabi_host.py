@@ -136,6 +136,50 @@ def test_noalloc_gemm_refuses_to_run_before_init_or_beyond_its_limit(pkg):
     assert rc != 0 and (b"thgpu_init" in L.lib.thgpu_last_error() or b"null operand" in L.lib.thgpu_last_error())
 
 
+def test_flat_entry_points_refuse_null_operands_before_any_launch(pkg):
+    """Every flat entry point that takes raw device pointers or tensor handles returns an error for a null one while
+    its other arguments are valid: the refusal comes before the library is initialised or anything is enqueued (a null
+    pointer that reached a kernel would fault on the GPU)."""
+    L = pkg._lib
+    lib = L.lib
+    null = ctypes.POINTER(ctypes.c_float)()
+    buf = (ctypes.c_float * 16)()          # a host buffer standing in for "some non-null pointer": never dereferenced
+    ptr = ctypes.cast(buf, ctypes.POINTER(ctypes.c_float))
+    geom = [1, 1, 4, 4, 3, 3, 1, 1, 1, 1]  # B, C, H, W, kH, kW, padH, padW, sH, sW
+    for fn in (lib.thgpu_im2col, lib.thgpu_col2im):
+        for a, b in ((null, ptr), (ptr, null), (null, null)):
+            assert fn(a, *(geom + [b])) != 0 and b"null operand" in lib.thgpu_last_error()
+    rc = lib.thgpu_gemm_strided_batched(b"n", b"n", 4, 4, 4, 1.0, null, 4, 16, ptr, 4, 0, 0.0, ptr, 4, 16, 2)
+    assert rc != 0 and b"null operand" in lib.thgpu_last_error()
+    rc = lib.thgpu_gemm_strided_batched(b"n", b"n", 4, 4, 4, 1.0, ptr, 4, 16, ptr, 4, 0, 0.0, null, 4, 16, 2)
+    assert rc != 0 and b"null operand" in lib.thgpu_last_error()
+    # an overflowing m * n is caught by the range check, not by the product
+    rc = lib.thgpu_gemm_noalloc(b"n", b"n", 1 << 40, 1 << 40, 4, 1.0, ptr, 4, ptr, 4, 0.0, ptr, 4)
+    assert rc != 0
+    # operators on tensor handles: a null handle in any position
+    nullt = L.TensorP()
+    t = [pkg.GPUTensor() for _ in range(7)]
+    P = [x._p for x in t]
+    conv_geom = [3, 3, 1, 1, 0, 0]
+    cases = [
+        (lib.thgpu_SpatialConvolutionMM_updateOutput, 6, conv_geom),
+        (lib.thgpu_SpatialConvolutionMM_updateOutputFused, 6, conv_geom + [0, 0.0, 0.0]),
+        (lib.thgpu_SpatialConvolutionMM_updateGradInput, 6, conv_geom),
+        (lib.thgpu_SpatialConvolutionMM_updateGradInputFused, 6, conv_geom + [0, 0.0]),
+        (lib.thgpu_SpatialConvolutionMM_accGradParameters, 6, conv_geom + [1.0]),
+        (lib.thgpu_SpatialConvolutionMM_accGradParametersFused, 6, conv_geom + [1.0, 0]),
+        (lib.thgpu_SpatialMaxPooling_updateOutput, 3, [2, 2, 2, 2]),
+        (lib.thgpu_SpatialMaxPooling_updateGradInput, 4, [2, 2, 2, 2]),
+        (lib.thgpu_SpatialMaxPooling_updateGradInputMasked, 4, [2, 2, 2, 2, 0.0]),
+        (lib.thgpu_Threshold_updateOutput, 2, [0.0, 0.0]),
+        (lib.thgpu_Threshold_updateGradInput, 3, [0.0]),
+    ]
+    for fn, ntens, rest in cases:
+        for hole in range(ntens):
+            args = [nullt if i == hole else P[i] for i in range(ntens)]
+            assert fn(*(args + rest)) != 0, (fn.__name__, hole)
+
+
 def test_module_defaults_follow_the_lua_constructors(pkg):
     nn = pkg.nn
     c = nn.SpatialConvolutionMM(3, 8, 5, 7)

@@ -8,7 +8,7 @@ padded input kept in finput bit-exact; repeated runs bit-identical.
 import numpy as np
 import pytest
 
-from helpers import check_close, gemm_tol, oracle_stack, rel_err, rng_for, uniform
+from helpers import check_close, gemm_tol, oracle_stack, rel_err, both_rel_err, rng_for, uniform
 
 pytestmark = pytest.mark.gpu
 
@@ -141,9 +141,9 @@ def test_gathered_non_batch_input(gt, gathered_route):
     got = run_conv(gt, x, w, b, go[0], geo)
     assert got["output"].shape == out_ref.shape[1:] and got["gradInput"].shape == x.shape
     assert got["finput"].shape == (C, H + 2, W + 2)
-    assert rel_err(got["output"], out_ref[0]) < gemm_tol(C * kH * kW)
-    assert rel_err(got["gradInput"], gi_ref[0]) < gemm_tol(M * kH * kW)
-    assert rel_err(got["gradWeight"], gw_ref) < gemm_tol(H * W)
+    assert both_rel_err(got["output"], out_ref[0]) < gemm_tol(C * kH * kW)
+    assert both_rel_err(got["gradInput"], gi_ref[0]) < gemm_tol(M * kH * kW)
+    assert both_rel_err(got["gradWeight"], gw_ref) < gemm_tol(H * W)
 
 
 def test_gathered_gradweight_without_forward_rebuilds_the_padded_input(gt, gathered_route):
@@ -156,9 +156,9 @@ def test_gathered_gradweight_without_forward_rebuilds_the_padded_input(gt, gathe
     got = run_conv(gt, x, w, b, go, geo, 2.0, gw0, gb0, forward_first=False)
     assert got["finput"].shape != (B, C, H + 2, W + 2)   # no forward pass has filled it
     assert np.array_equal(bits(got["finput_after"]), bits(padded(x, 1, 1)))
-    assert rel_err(got["gradWeight"], gw_ref) < gemm_tol(B * H * W)
-    assert rel_err(got["gradBias"], gb_ref) < gemm_tol(B * H * W)
-    assert rel_err(got["gradInput"], gi_ref) < gemm_tol(M * kH * kW)
+    assert both_rel_err(got["gradWeight"], gw_ref) < gemm_tol(B * H * W)
+    assert both_rel_err(got["gradBias"], gb_ref) < gemm_tol(B * H * W)
+    assert both_rel_err(got["gradInput"], gi_ref) < gemm_tol(M * kH * kW)
 
 
 def random_gathered_geometries(n, seed):
@@ -197,10 +197,10 @@ def test_gathered_conv_random_geometry(gt, gathered_route, cfg):
         assert got["finput"].size <= 1            # an unpadded dense input is gathered from where it lies: no copy
     else:
         assert np.array_equal(bits(got["finput"]), bits(padded(x, pH, pW)))
-    assert rel_err(got["output"], out_ref) < gemm_tol(K)
-    assert rel_err(got["gradInput"], gi_ref) < gemm_tol(M * kH * kW)
-    assert rel_err(got["gradWeight"], gw_ref) < gemm_tol(B * N)
-    assert rel_err(got["gradBias"], gb_ref) < gemm_tol(B * N)
+    assert both_rel_err(got["output"], out_ref) < gemm_tol(K)
+    assert both_rel_err(got["gradInput"], gi_ref) < gemm_tol(M * kH * kW)
+    assert both_rel_err(got["gradWeight"], gw_ref) < gemm_tol(B * N)
+    assert both_rel_err(got["gradBias"], gb_ref) < gemm_tol(B * N)
 
 
 @pytest.mark.parametrize("split", [1, 3])
@@ -221,9 +221,9 @@ def test_gathered_conv_every_tile_configuration(gt, gathered_route, tile, split,
     out_ref, go, gi_ref, gw_ref, gb_ref = reference(x, w, b, rng, geo, 1.0, gw0, gb0)
     got = run_conv(gt, x, w, b, go, geo, 1.0, gw0, gb0)
     assert got["finput"].shape == (B, C, H + 2, W + 2)
-    assert rel_err(got["output"], out_ref) < gemm_tol(K)
-    assert rel_err(got["gradInput"], gi_ref) < gemm_tol(M * kH * kW)
-    assert rel_err(got["gradWeight"], gw_ref) < gemm_tol(B * H * W)
+    assert both_rel_err(got["output"], out_ref) < gemm_tol(K)
+    assert both_rel_err(got["gradInput"], gi_ref) < gemm_tol(M * kH * kW)
+    assert both_rel_err(got["gradWeight"], gw_ref) < gemm_tol(B * H * W)
 
 
 def test_mode_1_gathers_where_a_tiled_kernel_takes_the_product(gt):
@@ -242,9 +242,9 @@ def test_mode_1_gathers_where_a_tiled_kernel_takes_the_product(gt):
             out_ref, go, gi_ref, gw_ref, gb_ref = reference(x, w, b, rng, geo, 1.0, gw0, gb0)
             got = run_conv(gt, x, w, b, go, geo)
             assert got["finput"].shape == ((B, C, H + 2, W + 2) if gathers else (B, C * kH * kW, H * W))
-            assert rel_err(got["output"], out_ref) < gemm_tol(C * kH * kW)
-            assert rel_err(got["gradInput"], gi_ref) < gemm_tol(M * kH * kW)
-            assert rel_err(got["gradWeight"], gw_ref) < gemm_tol(B * H * W)
+            assert both_rel_err(got["output"], out_ref) < gemm_tol(C * kH * kW)
+            assert both_rel_err(got["gradInput"], gi_ref) < gemm_tol(M * kH * kW)
+            assert both_rel_err(got["gradWeight"], gw_ref) < gemm_tol(B * H * W)
     finally:
         assert lib.thgpu_conv_set_mode(before) == 0
 
@@ -277,8 +277,8 @@ def test_route_switched_between_forward_and_accgradparameters(gt):
                 assert m.finput.nElement() == 0       # the unpadded dense input is gathered in place
             assert lib.thgpu_conv_set_mode(acc_mode) == 0
             m.accGradParameters(dx, dgo, 1.0)
-            assert rel_err(out, out_ref) < gemm_tol(C * k * k)
-            assert rel_err(m.gradWeight.float(), gw_ref) < gemm_tol(B * out_ref.shape[2] * out_ref.shape[3])
+            assert both_rel_err(out, out_ref) < gemm_tol(C * k * k)
+            assert both_rel_err(m.gradWeight.float(), gw_ref) < gemm_tol(B * out_ref.shape[2] * out_ref.shape[3])
     finally:
         assert lib.thgpu_conv_set_mode(before) == 0
 

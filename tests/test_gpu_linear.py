@@ -8,7 +8,7 @@ length).
 import numpy as np
 import pytest
 
-from helpers import gemm_tol, rel_err, rng_for, uniform
+from helpers import gemm_tol, rel_err, both_rel_err, rng_for, uniform
 
 pytestmark = pytest.mark.gpu
 
@@ -77,10 +77,10 @@ def test_addmm_tolerance_and_separate_result(gt, mnk):
     r.addmm(0.5, dev(gt, t), 1.5, dev(gt, m1), dev(gt, m2))          # r is resized to t and takes its values
     assert r.size() == (m, n)
     ref = 0.5 * t.astype(np.float64) + 1.5 * (m1.astype(np.float64) @ m2.astype(np.float64))
-    assert rel_err(r.float(), ref) < gemm_tol(k)
+    assert both_rel_err(r.float(), ref) < gemm_tol(k)
     oracle.use_blas(k >= 1024)
     try:
-        assert rel_err(r.float(), oracle.addmm(0.5, t, 1.5, m1, m2)) < gemm_tol(k)
+        assert both_rel_err(r.float(), oracle.addmm(0.5, t, 1.5, m1, m2)) < gemm_tol(k)
     finally:
         oracle.use_blas(False)
 
@@ -155,12 +155,12 @@ def test_linear_fwd_bwd_matches_oracle(gt, shape):
     dx, dgo = dev(gt, x), dev(gt, go)
     out = m.forward(dx).float()
     gi = m.backward(dx, dgo, 0.5).float()
-    assert rel_err(out, oracle.linear_updateOutput(x, w, b)) < gemm_tol(I)
-    assert rel_err(gi, oracle.linear_updateGradInput(go, w)) < gemm_tol(O)
+    assert both_rel_err(out, oracle.linear_updateOutput(x, w, b)) < gemm_tol(I)
+    assert both_rel_err(gi, oracle.linear_updateGradInput(go, w)) < gemm_tol(O)
     gw, gb = gw0.copy(), gb0.copy()
     oracle.linear_accGradParameters(x, go, gw, gb, 0.5)
-    assert rel_err(m.gradWeight.float(), gw) < gemm_tol(B)
-    assert rel_err(m.gradBias.float(), gb) < gemm_tol(B)
+    assert both_rel_err(m.gradWeight.float(), gw) < gemm_tol(B)
+    assert both_rel_err(m.gradBias.float(), gb) < gemm_tol(B)
 
 
 def test_linear_vector_input(gt):
@@ -173,8 +173,8 @@ def test_linear_vector_input(gt):
     m.zeroGradParameters()
     out = m.forward(dev(gt, x)).float()
     gi = m.backward(dev(gt, x), dev(gt, go)).float()
-    assert rel_err(out, oracle.addmv(1.0, b, 1.0, w, x)) < gemm_tol(I)
-    assert rel_err(gi, oracle.addmv_t(0.0, np.zeros(I, np.float32), 1.0, w, go)) < gemm_tol(O)
+    assert both_rel_err(out, oracle.addmv(1.0, b, 1.0, w, x)) < gemm_tol(I)
+    assert both_rel_err(gi, oracle.addmv_t(0.0, np.zeros(I, np.float32), 1.0, w, go)) < gemm_tol(O)
     assert rel_err(m.gradWeight.float(), np.outer(go, x)) < 1e-6
     assert np.array_equal(m.gradBias.float(), go)
 
@@ -196,12 +196,12 @@ def test_alexnet_classifier_sizes(gt):
             out = m.forward(dx).float()
             gi = m.backward(dx, dev(gt, go)).float()
             ref = oracle.linear_updateOutput(x, w, b)
-            assert rel_err(out, ref) < gemm_tol(I)
-            assert rel_err(gi, oracle.linear_updateGradInput(go, w)) < gemm_tol(O)
+            assert both_rel_err(out, ref) < gemm_tol(I)
+            assert both_rel_err(gi, oracle.linear_updateGradInput(go, w)) < gemm_tol(O)
             gw, gb = np.zeros_like(w), np.zeros_like(b)
             oracle.linear_accGradParameters(x, go, gw, gb, 1.0)
-            assert rel_err(m.gradWeight.float(), gw) < gemm_tol(B)
-            assert rel_err(m.gradBias.float(), gb) < gemm_tol(B)
+            assert both_rel_err(m.gradWeight.float(), gw) < gemm_tol(B)
+            assert both_rel_err(m.gradBias.float(), gb) < gemm_tol(B)
             x = np.maximum(ref, 0)
     finally:
         oracle.use_blas(False)
@@ -323,3 +323,75 @@ def test_blas_ger_and_axpy(gt):
     ref = v.copy()
     ref[::3] = ref[::3] + f(1.5) * u[::2]
     assert np.array_equal(dv.float(), ref)
+
+
+# ---- dot and the index operations (what Torch's generic tensor binding calls besides the above) ------------------
+@pytest.mark.parametrize("n", [1, 5, 255, 4096, 4097, 100003, 5000000])
+def test_dot_against_float64_and_exact_on_integers(gt, n):
+    rng = rng_for(300 + n % 97)
+    a, b = uniform(rng, (n,)), uniform(rng, (n,))
+    ref = float(np.dot(a.astype(np.float64), b.astype(np.float64)))
+    got = dev(gt, a).dot(dev(gt, b))
+    scale = float(np.sum(np.abs(a.astype(np.float64) * b)))
+    assert abs(got - ref) <= 1e-6 * scale + 1e-30
+    assert dev(gt, a).dot(dev(gt, b)) == got                       # fixed summation shape: reruns are bit-identical
+    ia, ib = ints(rng, (n,)), ints(rng, (n,))
+    assert dev(gt, ia).dot(dev(gt, ib)) == float(np.dot(ia.astype(np.float64), ib))
+    # a strided view and a matrix of the same element count (newContiguous on both sides)
+    if n == 4096:
+        m = uniform(rng, (64, 128))
+        assert abs(dev(gt, m).t().dot(dev(gt, m.T.copy())) - float(np.sum(m.astype(np.float64) ** 2))) < 1e-3
+    with pytest.raises(gt.THGPUError, match="size do not match"):
+        dev(gt, a).dot(dev(gt, np.zeros(n + 1, np.float32)))
+
+
+@pytest.mark.parametrize("shape,dim", [((7,), 0), ((5, 9), 0), ((5, 9), 1), ((3, 4, 6), 1), ((2, 3, 4, 5), 3)])
+def test_index_select_copy_fill_bit_exact(gt, shape, dim):
+    rng = rng_for(310 + len(shape) * 7 + dim)
+    x = uniform(rng, shape)
+    n = shape[dim]
+    idx = rng.integers(1, n + 1, size=n + 2)                       # 1-based, repeats allowed
+    got = dev(gt, x).index(dim, idx).float()
+    assert np.array_equal(got, np.take(x, idx - 1, axis=dim))
+    # a non-contiguous source
+    if len(shape) == 2:
+        got_t = dev(gt, x.T.copy()).t().index(dim, idx).float()
+        assert np.array_equal(got_t, np.take(x, idx - 1, axis=dim))
+    # indexCopy: distinct targets, slices of src in order
+    perm = rng.permutation(n)[:max(1, n // 2)] + 1
+    src_shape = list(shape)
+    src_shape[dim] = len(perm)
+    src = uniform(rng, src_shape)
+    ref = x.copy()
+    sl = [slice(None)] * len(shape)
+    for k, p in enumerate(perm):
+        sl[dim] = p - 1
+        ss = list(sl)
+        ss[dim] = k
+        ref[tuple(sl)] = src[tuple(ss)]
+    d = dev(gt, x)
+    assert np.array_equal(d.indexCopy(dim, perm, dev(gt, src)).float(), ref)
+    # indexFill
+    ref2 = x.copy()
+    for p in perm:
+        sl[dim] = p - 1
+        ref2[tuple(sl)] = 2.5
+    assert np.array_equal(dev(gt, x).indexFill(dim, perm, 2.5).float(), ref2)
+    with pytest.raises(gt.THGPUError, match="out of range"):
+        dev(gt, x).index(dim, [n + 1])
+    with pytest.raises(gt.THGPUError, match="out of bounds"):
+        dev(gt, x).index(len(shape), [1])
+
+
+def test_raw_memcpy_entry_points_round_trip(gt):
+    import ctypes
+    lib = gt._lib.lib
+    x = uniform(rng_for(320), (1000,))
+    d = gt.GPUTensor(1000)
+    f32p = ctypes.POINTER(ctypes.c_float)
+    assert lib.thgpu_memcpy_h2d(lib.THGPUTensor_data(d._p), x.ctypes.data_as(f32p), 1000) == 0
+    back = np.zeros(1000, np.float32)
+    assert lib.thgpu_memcpy_d2h(back.ctypes.data_as(f32p), lib.THGPUTensor_data(d._p), 1000) == 0
+    assert np.array_equal(back, x) and np.array_equal(d.float(), x)
+    assert lib.thgpu_memcpy_d2h(back.ctypes.data_as(f32p), None, 4) != 0 and b"null" in lib.thgpu_last_error()
+    assert lib.thgpu_memcpy_h2d(None, x.ctypes.data_as(f32p), 0) == 0
