@@ -127,6 +127,10 @@ int thgpu_synchronize(void);
  * and when an allocation fails.  No counterpart in the reference, whose array_views freed eagerly. */
 int thgpu_empty_cache(void);
 long thgpu_cached_bytes(void);
+/* How many times the library has called hipMalloc or hipFree since it was loaded (storage blocks, the split-reduction
+ * workspace, the offset tables of the gathered convolutions: every allocation it makes).  A caller that must not
+ * allocate can verify an entry point against it; no counterpart in the reference. */
+long thgpu_device_alloc_calls(void);
 
 /* Device name / compute-unit count / total memory, replacing the stubbed
  * getDeviceProperties (gputorch/init.cpp:40-66). */
@@ -495,7 +499,7 @@ int thgpu_SpatialMaxPooling_updateGradInput(THGPUTensor *input, THGPUTensor *gra
                                             THGPUTensor *indices, int kW, int kH, int dW, int dH);
 
 /* updateGradInput with the backward of a Threshold in front of the pooling layer applied as gradInput is stored:
- * gradInput = input > threshold ? g : 0 (see thgpu_SpatialConvolutionMM_updateGradInputMasked). */
+ * gradInput = input > threshold ? g : 0 (see thgpu_SpatialConvolutionMM_updateGradInputFused). */
 int thgpu_SpatialMaxPooling_updateGradInputMasked(THGPUTensor *input, THGPUTensor *gradOutput,
                                                   THGPUTensor *gradInput, THGPUTensor *indices, int kW, int kH,
                                                   int dW, int dH, float threshold);

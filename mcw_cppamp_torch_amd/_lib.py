@@ -65,6 +65,7 @@ _SIGNATURES = {
     "thgpu_synchronize": (c_int, []),
     "thgpu_empty_cache": (c_int, []),
     "thgpu_cached_bytes": (c_long, []),
+    "thgpu_device_alloc_calls": (c_long, []),
     "thgpu_debug_set": (c_int, [c_char_p, c_char_p]),
     "thgpu_conv_set_mode": (c_int, [c_int]),
     "thgpu_conv_get_mode": (c_int, []),

@@ -56,30 +56,63 @@ def build(verbose=False, jobs=None):
     return LIB_PATH
 
 
+def _first_dir_with(names, roots):
+    """The first of `roots` that holds every file of `names`, or None."""
+    for r in roots:
+        if r and os.path.isdir(r) and all(os.path.exists(os.path.join(r, n)) for n in names):
+            return r
+    return None
+
+
 def _lua_include_dirs():
-    """Directories holding lua.h and luaT.h, or None: LUA_INCDIR / TORCH_INSTALL first, then the usual prefixes."""
-    roots = [os.environ.get("LUA_INCDIR"), os.path.join(os.environ.get("TORCH_INSTALL", ""), "include"),
+    """Where the luaT glue finds its headers, or None when Lua or luaT is missing: LUA_INCDIR / TORCH_INSTALL first,
+    then the usual prefixes.  Keys: lua (lua.h, lauxlib.h), luaT (luaT.h), and -- for the tensor half only -- TH (TH.h
+    with its configured THGeneral.h) and templates (the directory that holds Torch's generic/Tensor.c and
+    generic/Storage.c: gputorch/torch of a Torch7 source tree, TORCH7_SRC)."""
+    install = os.environ.get("TORCH_INSTALL", "")
+    src = os.environ.get("TORCH7_SRC", "")
+    roots = [os.environ.get("LUA_INCDIR"), os.path.join(install, "include") if install else None,
              "/usr/include/luajit-2.1", "/usr/include/luajit-2.0", "/usr/include/lua5.1", "/usr/local/include",
              "/usr/include", os.path.expanduser("~/torch/install/include")]
-    roots = [r for r in roots if r and os.path.isdir(r)]
-    lua = next((r for r in roots if os.path.exists(os.path.join(r, "lua.h"))), None)
-    luat = next((r for r in roots if os.path.exists(os.path.join(r, "luaT.h"))), None)
-    return [lua, luat] if lua and luat else None
+    found = {"lua": _first_dir_with(["lua.h", "lauxlib.h"], roots), "luaT": _first_dir_with(["luaT.h"], roots)}
+    if not found["lua"] or not found["luaT"]:
+        return None
+    found["TH"] = _first_dir_with(["TH.h", "THGeneral.h"], [os.path.join(r, "TH") for r in roots if r] + roots)
+    found["templates"] = _first_dir_with([os.path.join("generic", "Tensor.c"), os.path.join("generic", "Storage.c")],
+                                         [os.environ.get("GPUTORCH_TEMPLATES"),
+                                          os.path.join(src, "gputorch", "torch") if src else None,
+                                          os.path.join(src, "torch") if src else None])
+    return found
 
 
 def build_lua_glue(verbose=False):
-    """Compiles lua/gpunn_glue.cpp into libgpunn.so where the Lua and luaT headers exist; returns its path or None
-    (no Lua toolchain: the glue is source only, the Python mirror in nn.py / gputorch.py is the host side)."""
+    """Compiles the luaT glue where the Lua and luaT headers exist: lua/gpunn_glue.cpp into libgpunn.so
+    (luaopen_libgpunn) and, where the TH headers and Torch's binding templates are found as well,
+    lua/gputorch_glue.cpp into libgputorch.so (luaopen_libgputorch).  Returns the list of libraries built (empty
+    without a Lua toolchain: the glue is then source only, syntax-checked by tests/test_lua_glue_syntax.py, and the
+    Python mirror in nn.py / gputorch.py is the host side)."""
     inc = _lua_include_dirs()
     if inc is None:
         if verbose:
-            print("lua.h / luaT.h not found: lua/gpunn_glue.cpp not built")
-        return None
+            print("lua.h / luaT.h not found: lua/gpunn_glue.cpp and lua/gputorch_glue.cpp not built")
+        return []
+    common = ["g++", "-O2", "-fPIC", "-shared", "-std=c++11"]
+    link = ["-L" + HERE, "-lthgpu", "-lluaT", "-Wl,-rpath," + HERE]
+    built = []
     out = os.path.join(HERE, "libgpunn.so")
-    cmd = ["g++", "-O2", "-fPIC", "-shared", "-std=c++11", os.path.join(HERE, "lua", "gpunn_glue.cpp"), "-o", out,
-           "-L" + HERE, "-lthgpu", "-lluaT", "-Wl,-rpath," + HERE] + ["-I" + d for d in dict.fromkeys(inc)]
-    subprocess.check_call(cmd)
-    return out
+    dirs = list(dict.fromkeys([inc["lua"], inc["luaT"]]))
+    subprocess.check_call(common + [os.path.join(HERE, "lua", "gpunn_glue.cpp"), "-o", out] + link +
+                          ["-I" + d for d in dirs])
+    built.append(out)
+    if inc["TH"] and inc["templates"]:
+        out = os.path.join(HERE, "libgputorch.so")
+        dirs = list(dict.fromkeys([inc["lua"], inc["luaT"], inc["TH"], inc["templates"]]))
+        subprocess.check_call(common + [os.path.join(HERE, "lua", "gputorch_glue.cpp"), "-o", out] + link + ["-lTH"] +
+                              ["-I" + d for d in dirs])
+        built.append(out)
+    elif verbose:
+        print("TH.h or Torch's generic/Tensor.c not found (TORCH_INSTALL, TORCH7_SRC): lua/gputorch_glue.cpp not built")
+    return built
 
 
 if __name__ == "__main__":

@@ -54,6 +54,13 @@ hipStream_t stream();
 // kernels that use it because everything runs on the one library stream.
 float *workspace(size_t bytes);
 int num_cus();
+// Returns the storage block cache's kept buffers to the device (draining the stream first); true when there were
+// any.  Every hipMalloc of the library that fails calls this and tries once more (storage.hip).
+bool drop_cached_blocks();
+// hipMalloc / hipFree as the library calls them: counted, so that a test can show that an entry point made neither
+// (thgpu_device_alloc_calls).
+hipError_t device_malloc(void **p, size_t bytes);
+void device_free(void *p);
 // The fixed device array behind the entry points that must not allocate (runtime.hip): its device
 // address and size in floats once the library is initialised, nullptr before (never initialises).
 float *static_scratch(size_t *floats);

@@ -146,7 +146,12 @@ const int *table(int kind, int a, int b, int c, int d, int e, long count) {
     hipStream_t s = stream();
     if (!s) return nullptr;
     int *t = nullptr;
-    if (hipMalloc(reinterpret_cast<void **>(&t), sizeof(int) * (size_t)count) != hipSuccess) {
+    hipError_t err = device_malloc(reinterpret_cast<void **>(&t), sizeof(int) * (size_t)count);
+    if (err != hipSuccess) {
+        (void)hipGetLastError();
+        if (drop_cached_blocks()) err = device_malloc(reinterpret_cast<void **>(&t), sizeof(int) * (size_t)count);
+    }
+    if (err != hipSuccess) {
         (void)hipGetLastError();
         fail("offset table allocation of %ld entries failed", count);
         return nullptr;
@@ -157,7 +162,7 @@ const int *table(int kind, int a, int b, int c, int d, int e, long count) {
     else
         hipLaunchKernelGGL(pixel_table_kernel, dim3(blocks), dim3(256), 0, s, t, a, b, c, d);
     if (check_launch("conv offset table")) {
-        (void)hipFree(t);
+        device_free(t);
         return nullptr;
     }
     g_tables[key] = t;
@@ -172,7 +177,7 @@ int trim_tables() {
     hipStream_t s = stream();
     if (!s) return 1;
     THGPU_HIP_TRY(hipStreamSynchronize(s));
-    for (auto &kv : g_tables) (void)hipFree(kv.second);
+    for (auto &kv : g_tables) device_free(kv.second);
     g_tables.clear();
     return 0;
 }

@@ -135,6 +135,18 @@ int num_cus() {
     return g_cus > 0 ? g_cus : 256;
 }
 
+static long g_alloc_calls = 0;
+
+hipError_t device_malloc(void **p, size_t bytes) {
+    ++g_alloc_calls;
+    return hipMalloc(p, bytes);
+}
+
+void device_free(void *p) {
+    ++g_alloc_calls;
+    (void)hipFree(p);
+}
+
 static float *g_ws = nullptr;
 static size_t g_ws_bytes = 0;
 
@@ -144,12 +156,17 @@ float *workspace(size_t bytes) {
     if (g_ws) {
         // Kernels still in flight may read the old buffer.
         if (hipStreamSynchronize(g_stream) != hipSuccess) return nullptr;
-        (void)hipFree(g_ws);
+        device_free(g_ws);
         g_ws = nullptr;
         g_ws_bytes = 0;
     }
     size_t want = bytes + bytes / 4;
-    const hipError_t e = hipMalloc(reinterpret_cast<void **>(&g_ws), want);
+    hipError_t e = device_malloc(reinterpret_cast<void **>(&g_ws), want);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        // freed storage buffers may be sitting in the block cache: give them back and try once more
+        if (drop_cached_blocks()) e = device_malloc(reinterpret_cast<void **>(&g_ws), want);
+    }
     if (e != hipSuccess) {
         (void)hipGetLastError();  // or the next launch check would report this failure as its own
         fail("workspace allocation of %zu bytes failed: %s", want, hipGetErrorString(e));
@@ -310,6 +327,8 @@ long thgpu_selftest_index_math(void) {
     }
     return bad;
 }
+
+long thgpu_device_alloc_calls(void) { return g_alloc_calls; }
 
 long thgpu_selftest_launch_plans(void) { return im2col_plan_selftest() + pool_plan_selftest(); }
 

@@ -106,12 +106,12 @@ constexpr size_t kCacheLimit = size_t(8) << 30;
 std::unordered_map<size_t, std::vector<float *>> g_free_blocks;
 size_t g_cached_bytes = 0;
 
-void drop_cached_blocks() {
+void drop_cached_blocks_impl() {
     if (g_free_blocks.empty()) return;
     hipStream_t s = thgpu::stream();
     if (s) (void)hipStreamSynchronize(s);
     for (auto &kv : g_free_blocks)
-        for (float *p : kv.second) (void)hipFree(p);
+        for (float *p : kv.second) device_free(p);
     g_free_blocks.clear();
     g_cached_bytes = 0;
 }
@@ -127,11 +127,11 @@ hipError_t acquire_block(long floats, float **out) {
         g_cached_bytes -= bytes;
         return hipSuccess;
     }
-    hipError_t e = hipMalloc(reinterpret_cast<void **>(out), bytes);
+    hipError_t e = device_malloc(reinterpret_cast<void **>(out), bytes);
     if (e != hipSuccess && !g_free_blocks.empty()) {
         (void)hipGetLastError();
-        drop_cached_blocks();
-        e = hipMalloc(reinterpret_cast<void **>(out), bytes);
+        drop_cached_blocks_impl();
+        e = device_malloc(reinterpret_cast<void **>(out), bytes);
     }
     if (e != hipSuccess) (void)hipGetLastError();
     return e;
@@ -143,8 +143,8 @@ void release_block(float *p, long floats) {
     if (floats <= 0 || g_cached_bytes + bytes > kCacheLimit) {
         hipStream_t s = thgpu::stream();
         if (s) (void)hipStreamSynchronize(s);  // work enqueued earlier may still use the buffer
-        (void)hipFree(p);
-        if (g_cached_bytes + bytes > kCacheLimit) drop_cached_blocks();
+        device_free(p);
+        if (g_cached_bytes + bytes > kCacheLimit) drop_cached_blocks_impl();
         return;
     }
     g_free_blocks[bytes].push_back(p);
@@ -152,6 +152,16 @@ void release_block(float *p, long floats) {
 }
 
 }  // namespace
+
+namespace thgpu {
+// For the library's other allocations (the split-reduction workspace, the offset tables): the kept blocks go back to
+// the device, so that a hipMalloc that has just failed can be tried once more.  Returns whether anything was freed.
+bool drop_cached_blocks() {
+    const bool had = !g_free_blocks.empty();
+    drop_cached_blocks_impl();
+    return had;
+}
+}  // namespace thgpu
 
 static void release_buffer(THGPUStorage *self) {
     release_block(self->data, self->size);

@@ -1,6 +1,6 @@
 -- gpunn.fuse(net): lets the neighbours of every nn.Threshold / nn.ReLU of an nn.Sequential do its work while they
--- store their own results (see include/thgpu.h, thgpu_SpatialConvolutionMM_updateOutputThreshold and the *Masked
--- entry points).  The Threshold modules stay in place and pass tensors through, so nn.Sequential:updateOutput /
+-- store their own results (see include/thgpu.h, thgpu_SpatialConvolutionMM_updateOutputFused / _updateGradInputFused
+-- and thgpu_SpatialMaxPooling_updateGradInputMasked).  The Threshold modules stay in place and pass tensors through, so nn.Sequential:updateOutput /
 -- :updateGradInput (mcw_nn/Sequential.lua:33-68) and every result downstream are unchanged bit for bit.
 -- Needs value <= threshold (true of nn.ReLU, mcw_nn/ReLU.lua:4).  gpunn.unfuse(net) undoes it.
 require 'nn'
@@ -39,23 +39,40 @@ local function link(producer, consumer)
             self.paddedOutput = b
             self.output = b:narrow(b:dim() - 1, pH + 1, H):narrow(b:dim(), pW + 1, W)
          end
-         consumer.inputInPaddedBuffer = true
       else
          if self.paddedOutput then self.output = input.new(); self.paddedOutput = nil end
-         consumer.inputInPaddedBuffer = nil
       end
       return class_updateOutput(self, input)
    end
    producer.linkedConsumer = consumer
+   -- The consumer decides call by call whether its input lies in the padded buffer: only the producer's own current
+   -- output view does (the very object nn.Sequential hands on, mcw_nn/Sequential.lua:33-68); any other input, e.g.
+   -- net:get(i):forward(x) on a tensor of the caller's, takes the ordinary route.
+   local function in_padded_buffer(input)
+      return producer.paddedOutput ~= nil and rawequal(input, producer.output) or nil
+   end
+   local consumer_updateOutput, consumer_accGradParameters = consumer.updateOutput, consumer.accGradParameters
+   consumer.updateOutput = function(self, input)
+      self.inputInPaddedBuffer = in_padded_buffer(input)
+      return consumer_updateOutput(self, input)
+   end
+   consumer.accGradParameters = function(self, input, gradOutput, scale)
+      self.inputInPaddedBuffer = in_padded_buffer(input)
+      return consumer_accGradParameters(self, input, gradOutput, scale)
+   end
+   consumer.linkedProducer = producer
 end
 
 function gpunn.unfuse(net)
    for _, m in ipairs(net.modules) do
       if m.modules then gpunn.unfuse(m) end
       if m.linkedConsumer then
-         m.linkedConsumer.inputInPaddedBuffer = nil
          m.linkedConsumer, m.updateOutput = nil, nil
          if m.paddedOutput then m.output = m.output.new(); m.paddedOutput = nil end
+      end
+      if m.linkedProducer then
+         m.linkedProducer, m.inputInPaddedBuffer = nil, nil
+         m.updateOutput, m.accGradParameters = nil, nil     -- back to the class methods
       end
       if threshold(m) and (m.fusedForward or m.fusedBackward) then
          m.output = m.output.new()

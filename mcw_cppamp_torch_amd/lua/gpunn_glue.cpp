@@ -70,130 +70,195 @@ PoolFields pool_fields(lua_State *L) {
                       luaT_getfieldcheckint(L, 1, "dW"), luaT_getfieldcheckint(L, 1, "dH")};
 }
 
+// Every operator fetches the module's tensors into named locals, one statement each (each fetch pushes the value on
+// the Lua stack, and the order of evaluation of function arguments is unspecified in C++), and returns the field the
+// reference's Lua wrappers return (mcw_nn/SpatialConvolutionMM.lua:48-55), pushed explicitly.
+int returning(lua_State *L, const char *field_name) {
+    lua_getfield(L, 1, field_name);
+    return 1;
+}
+
 // ---- nn.SpatialConvolutionMM -------------------------------------------------------------------------------------
 int conv_updateOutput(lua_State *L) {
     THGPUTensor *input = arg(L, 2);
     const ConvFields f = conv_fields(L);
+    THGPUTensor *weight = field(L, "weight");
+    THGPUTensor *bias = field(L, "bias");
+    THGPUTensor *finput = field(L, "finput");
+    THGPUTensor *fgradInput = field(L, "fgradInput");
+    THGPUTensor *output = field(L, "output");
     const int flags = (has_field(L, "fusedThreshold") ? THGPU_FUSE_THRESHOLD : 0) |
                       (has_field(L, "inputInPaddedBuffer") ? THGPU_INPUT_IN_PADDED_BUFFER : 0);
-    if (flags)
-        fail(L, thgpu_SpatialConvolutionMM_updateOutputFused(
-                    input, field(L, "weight"), field(L, "bias"), field(L, "finput"), field(L, "fgradInput"),
-                    field(L, "output"), f.kW, f.kH, f.dW, f.dH, f.padW, f.padH, flags,
-                    static_cast<float>(opt_number(L, "fusedThreshold", 0)), static_cast<float>(opt_number(L, "fusedValue", 0))));
-    else
-        fail(L, thgpu_SpatialConvolutionMM_updateOutput(input, field(L, "weight"), field(L, "bias"), field(L, "finput"),
-                                                        field(L, "fgradInput"), field(L, "output"), f.kW, f.kH, f.dW,
-                                                        f.dH, f.padW, f.padH));
-    return 1;
+    int rc;
+    if (flags) {
+        const float threshold = static_cast<float>(opt_number(L, "fusedThreshold", 0));
+        const float value = static_cast<float>(opt_number(L, "fusedValue", 0));
+        rc = thgpu_SpatialConvolutionMM_updateOutputFused(input, weight, bias, finput, fgradInput, output, f.kW, f.kH,
+                                                          f.dW, f.dH, f.padW, f.padH, flags, threshold, value);
+    } else {
+        rc = thgpu_SpatialConvolutionMM_updateOutput(input, weight, bias, finput, fgradInput, output, f.kW, f.kH, f.dW,
+                                                     f.dH, f.padW, f.padH);
+    }
+    fail(L, rc);
+    return returning(L, "output");
 }
 int conv_updateGradInput(lua_State *L) {
-    THGPUTensor *input = arg(L, 2), *gradOutput = arg(L, 3);
+    THGPUTensor *input = arg(L, 2);
+    THGPUTensor *gradOutput = arg(L, 3);
     const ConvFields f = conv_fields(L);
-    if (has_field(L, "inputThreshold"))
-        fail(L, thgpu_SpatialConvolutionMM_updateGradInputFused(
-                    input, gradOutput, field(L, "weight"), field(L, "finput"), field(L, "fgradInput"),
-                    field(L, "gradInput"), f.kW, f.kH, f.dW, f.dH, f.padW, f.padH, THGPU_FUSE_INPUT_MASK,
-                    static_cast<float>(opt_number(L, "inputThreshold", 0))));
-    else
-        fail(L, thgpu_SpatialConvolutionMM_updateGradInput(input, gradOutput, field(L, "weight"), field(L, "finput"),
-                                                           field(L, "fgradInput"), field(L, "gradInput"), f.kW, f.kH,
-                                                           f.dW, f.dH, f.padW, f.padH));
-    return 1;
+    THGPUTensor *weight = field(L, "weight");
+    THGPUTensor *finput = field(L, "finput");
+    THGPUTensor *fgradInput = field(L, "fgradInput");
+    THGPUTensor *gradInput = field(L, "gradInput");
+    int rc;
+    if (has_field(L, "inputThreshold")) {
+        const float threshold = static_cast<float>(opt_number(L, "inputThreshold", 0));
+        rc = thgpu_SpatialConvolutionMM_updateGradInputFused(input, gradOutput, weight, finput, fgradInput, gradInput,
+                                                             f.kW, f.kH, f.dW, f.dH, f.padW, f.padH,
+                                                             THGPU_FUSE_INPUT_MASK, threshold);
+    } else {
+        rc = thgpu_SpatialConvolutionMM_updateGradInput(input, gradOutput, weight, finput, fgradInput, gradInput, f.kW,
+                                                        f.kH, f.dW, f.dH, f.padW, f.padH);
+    }
+    fail(L, rc);
+    return returning(L, "gradInput");
 }
 int conv_accGradParameters(lua_State *L) {
-    THGPUTensor *input = arg(L, 2), *gradOutput = arg(L, 3);
+    THGPUTensor *input = arg(L, 2);
+    THGPUTensor *gradOutput = arg(L, 3);
     const float scale = static_cast<float>(luaL_optnumber(L, 4, 1));  // SpatialConvolutionMM.cpp:326
     const ConvFields f = conv_fields(L);
-    fail(L, thgpu_SpatialConvolutionMM_accGradParametersFused(
-                input, gradOutput, field(L, "gradWeight"), field(L, "gradBias"), field(L, "finput"), field(L, "fgradInput"),
-                f.kW, f.kH, f.dW, f.dH, f.padW, f.padH, scale,
-                has_field(L, "inputInPaddedBuffer") ? THGPU_INPUT_IN_PADDED_BUFFER : 0));
+    THGPUTensor *gradWeight = field(L, "gradWeight");
+    THGPUTensor *gradBias = field(L, "gradBias");
+    THGPUTensor *finput = field(L, "finput");
+    THGPUTensor *fgradInput = field(L, "fgradInput");
+    const int flags = has_field(L, "inputInPaddedBuffer") ? THGPU_INPUT_IN_PADDED_BUFFER : 0;
+    fail(L, thgpu_SpatialConvolutionMM_accGradParametersFused(input, gradOutput, gradWeight, gradBias, finput,
+                                                              fgradInput, f.kW, f.kH, f.dW, f.dH, f.padW, f.padH, scale,
+                                                              flags));
     return 0;
 }
 
 // ---- nn.SpatialMaxPooling ------------------------------------------------------------------------------------------
 int pool_updateOutput(lua_State *L) {
+    THGPUTensor *input = arg(L, 2);
     const PoolFields f = pool_fields(L);
-    fail(L, thgpu_SpatialMaxPooling_updateOutput(arg(L, 2), field(L, "output"), field(L, "indices"), f.kW, f.kH, f.dW,
-                                                 f.dH));
-    return 1;
+    THGPUTensor *output = field(L, "output");
+    THGPUTensor *indices = field(L, "indices");
+    fail(L, thgpu_SpatialMaxPooling_updateOutput(input, output, indices, f.kW, f.kH, f.dW, f.dH));
+    return returning(L, "output");
 }
 int pool_updateGradInput(lua_State *L) {
+    THGPUTensor *input = arg(L, 2);
+    THGPUTensor *gradOutput = arg(L, 3);
     const PoolFields f = pool_fields(L);
-    if (has_field(L, "inputThreshold"))
-        fail(L, thgpu_SpatialMaxPooling_updateGradInputMasked(arg(L, 2), arg(L, 3), field(L, "gradInput"),
-                                                              field(L, "indices"), f.kW, f.kH, f.dW, f.dH,
-                                                              static_cast<float>(opt_number(L, "inputThreshold", 0))));
-    else
-        fail(L, thgpu_SpatialMaxPooling_updateGradInput(arg(L, 2), arg(L, 3), field(L, "gradInput"), field(L, "indices"),
-                                                        f.kW, f.kH, f.dW, f.dH));
-    return 1;
+    THGPUTensor *gradInput = field(L, "gradInput");
+    THGPUTensor *indices = field(L, "indices");
+    int rc;
+    if (has_field(L, "inputThreshold")) {
+        const float threshold = static_cast<float>(opt_number(L, "inputThreshold", 0));
+        rc = thgpu_SpatialMaxPooling_updateGradInputMasked(input, gradOutput, gradInput, indices, f.kW, f.kH, f.dW, f.dH,
+                                                           threshold);
+    } else {
+        rc = thgpu_SpatialMaxPooling_updateGradInput(input, gradOutput, gradInput, indices, f.kW, f.kH, f.dW, f.dH);
+    }
+    fail(L, rc);
+    return returning(L, "gradInput");
 }
 
 // ---- nn.Threshold / nn.ReLU ------------------------------------------------------------------------------------------
 int thr_updateOutput(lua_State *L) {
-    fail(L, thgpu_Threshold_updateOutput(arg(L, 2), field(L, "output"),
-                                         static_cast<float>(luaT_getfieldchecknumber(L, 1, "threshold")),
-                                         static_cast<float>(luaT_getfieldchecknumber(L, 1, "val"))));
-    return 1;
+    THGPUTensor *input = arg(L, 2);
+    THGPUTensor *output = field(L, "output");
+    const float threshold = static_cast<float>(luaT_getfieldchecknumber(L, 1, "threshold"));
+    const float value = static_cast<float>(luaT_getfieldchecknumber(L, 1, "val"));
+    fail(L, thgpu_Threshold_updateOutput(input, output, threshold, value));
+    return returning(L, "output");
 }
 int thr_updateGradInput(lua_State *L) {
-    fail(L, thgpu_Threshold_updateGradInput(arg(L, 2), arg(L, 3), field(L, "gradInput"),
-                                            static_cast<float>(luaT_getfieldchecknumber(L, 1, "threshold"))));
-    return 1;
+    THGPUTensor *input = arg(L, 2);
+    THGPUTensor *gradOutput = arg(L, 3);
+    THGPUTensor *gradInput = field(L, "gradInput");
+    const float threshold = static_cast<float>(luaT_getfieldchecknumber(L, 1, "threshold"));
+    fail(L, thgpu_Threshold_updateGradInput(input, gradOutput, gradInput, threshold));
+    return returning(L, "gradInput");
 }
 
 // ---- nn.SpatialAveragePooling / nn.SpatialSubSampling ------------------------------------------------------------------
 int avg_updateOutput(lua_State *L) {
+    THGPUTensor *input = arg(L, 2);
     const PoolFields f = pool_fields(L);
-    fail(L, thgpu_SpatialAveragePooling_updateOutput(arg(L, 2), field(L, "output"), f.kW, f.kH, f.dW, f.dH));
-    return 1;
+    THGPUTensor *output = field(L, "output");
+    fail(L, thgpu_SpatialAveragePooling_updateOutput(input, output, f.kW, f.kH, f.dW, f.dH));
+    return returning(L, "output");
 }
 int avg_updateGradInput(lua_State *L) {
+    THGPUTensor *input = arg(L, 2);
+    THGPUTensor *gradOutput = arg(L, 3);
     const PoolFields f = pool_fields(L);
-    fail(L, thgpu_SpatialAveragePooling_updateGradInput(arg(L, 2), arg(L, 3), field(L, "gradInput"), f.kW, f.kH, f.dW,
-                                                        f.dH));
-    return 1;
+    THGPUTensor *gradInput = field(L, "gradInput");
+    fail(L, thgpu_SpatialAveragePooling_updateGradInput(input, gradOutput, gradInput, f.kW, f.kH, f.dW, f.dH));
+    return returning(L, "gradInput");
 }
 int sub_updateOutput(lua_State *L) {
+    THGPUTensor *input = arg(L, 2);
     const PoolFields f = pool_fields(L);
-    fail(L, thgpu_SpatialSubSampling_updateOutput(arg(L, 2), field(L, "weight"), field(L, "bias"), field(L, "output"),
-                                                  f.kW, f.kH, f.dW, f.dH));
-    return 1;
+    THGPUTensor *weight = field(L, "weight");
+    THGPUTensor *bias = field(L, "bias");
+    THGPUTensor *output = field(L, "output");
+    fail(L, thgpu_SpatialSubSampling_updateOutput(input, weight, bias, output, f.kW, f.kH, f.dW, f.dH));
+    return returning(L, "output");
 }
 int sub_updateGradInput(lua_State *L) {
+    THGPUTensor *input = arg(L, 2);
+    THGPUTensor *gradOutput = arg(L, 3);
     const PoolFields f = pool_fields(L);
-    fail(L, thgpu_SpatialSubSampling_updateGradInput(arg(L, 2), arg(L, 3), field(L, "weight"), field(L, "gradInput"),
-                                                     f.kW, f.kH, f.dW, f.dH));
-    return 1;
+    THGPUTensor *weight = field(L, "weight");
+    THGPUTensor *gradInput = field(L, "gradInput");
+    fail(L, thgpu_SpatialSubSampling_updateGradInput(input, gradOutput, weight, gradInput, f.kW, f.kH, f.dW, f.dH));
+    return returning(L, "gradInput");
 }
 int sub_accGradParameters(lua_State *L) {
+    THGPUTensor *input = arg(L, 2);
+    THGPUTensor *gradOutput = arg(L, 3);
+    const float scale = static_cast<float>(luaL_optnumber(L, 4, 1));
     const PoolFields f = pool_fields(L);
-    fail(L, thgpu_SpatialSubSampling_accGradParameters(arg(L, 2), arg(L, 3), field(L, "gradWeight"), field(L, "gradBias"),
-                                                       f.kW, f.kH, f.dW, f.dH,
-                                                       static_cast<float>(luaL_optnumber(L, 4, 1))));
+    THGPUTensor *gradWeight = field(L, "gradWeight");
+    THGPUTensor *gradBias = field(L, "gradBias");
+    fail(L, thgpu_SpatialSubSampling_accGradParameters(input, gradOutput, gradWeight, gradBias, f.kW, f.kH, f.dW, f.dH,
+                                                       scale));
     return 0;
 }
 
 // ---- nn.LogSoftMax / nn.ClassNLLCriterion ----------------------------------------------------------------------------------
 int lsm_updateOutput(lua_State *L) {
-    fail(L, thgpu_LogSoftMax_updateOutput(arg(L, 2), field(L, "output")));
-    return 1;
+    THGPUTensor *input = arg(L, 2);
+    THGPUTensor *output = field(L, "output");
+    fail(L, thgpu_LogSoftMax_updateOutput(input, output));
+    return returning(L, "output");
 }
 int lsm_updateGradInput(lua_State *L) {
-    fail(L, thgpu_LogSoftMax_updateGradInput(arg(L, 3), field(L, "output"), field(L, "gradInput")));
-    return 1;
+    THGPUTensor *gradOutput = arg(L, 3);
+    THGPUTensor *output = field(L, "output");
+    THGPUTensor *gradInput = field(L, "gradInput");
+    fail(L, thgpu_LogSoftMax_updateGradInput(gradOutput, output, gradInput));
+    return returning(L, "gradInput");
 }
 int nll_updateOutput(lua_State *L) {
-    fail(L, thgpu_ClassNLLCriterion_updateOutput(arg(L, 2), arg(L, 3), field(L, "outputTensor"),
-                                                 luaT_getfieldcheckboolean(L, 1, "sizeAverage")));
-    return 1;
+    THGPUTensor *input = arg(L, 2);
+    THGPUTensor *target = arg(L, 3);
+    THGPUTensor *outputTensor = field(L, "outputTensor");
+    const int size_average = luaT_getfieldcheckboolean(L, 1, "sizeAverage");
+    fail(L, thgpu_ClassNLLCriterion_updateOutput(input, target, outputTensor, size_average));
+    return returning(L, "outputTensor");
 }
 int nll_updateGradInput(lua_State *L) {
-    fail(L, thgpu_ClassNLLCriterion_updateGradInput(arg(L, 2), arg(L, 3), field(L, "gradInput"),
-                                                    luaT_getfieldcheckboolean(L, 1, "sizeAverage")));
-    return 1;
+    THGPUTensor *input = arg(L, 2);
+    THGPUTensor *target = arg(L, 3);
+    THGPUTensor *gradInput = field(L, "gradInput");
+    const int size_average = luaT_getfieldcheckboolean(L, 1, "sizeAverage");
+    fail(L, thgpu_ClassNLLCriterion_updateGradInput(input, target, gradInput, size_average));
+    return returning(L, "gradInput");
 }
 
 const struct luaL_Reg kOps[] = {

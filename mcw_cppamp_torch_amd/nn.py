@@ -188,15 +188,26 @@ class Sequential(Module):
         self.modules[0].accUpdateGradParameters(input, cur, lr)
 
     def zeroGradParameters(self):
-        # mcw_nn/Sequential.lua:85-89 zeroes module by module; the dense GPU gradients of all modules go in one launch
-        _, grads = self.parameters()
-        gpu = [g for g in grads or [] if isinstance(g, GPUTensor) and g.isContiguous()]
+        # mcw_nn/Sequential.lua:85-89 calls every module's zeroGradParameters.  Modules that keep Module's own
+        # implementation are served together -- their dense GPU gradients go in one launch; a module (or nested
+        # container) that overrides the method has its own called.
+        plain, grads = [], []
+        for m in self.modules:
+            if type(m).zeroGradParameters is Module.zeroGradParameters and type(m).parameters in (
+                    Module.parameters,):
+                plain.append(m)
+            else:
+                m.zeroGradParameters()
+        for m in plain:
+            _, g = m.parameters()
+            grads.extend(g or [])
+        gpu = [g for g in grads if isinstance(g, GPUTensor) and g.isContiguous()]
         if len(gpu) > 1:
             arr = (_lib.TensorP * len(gpu))(*[g._p for g in gpu])
             _lib.check_status(lib.thgpu_fill_many(arr, len(gpu), 0.0))
         else:
             gpu = []
-        for g in grads or []:
+        for g in grads:
             if isinstance(g, GPUTensor):
                 if not any(g is h for h in gpu):
                     g.zero()

@@ -42,9 +42,13 @@ def run_both(gt, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc):
     gt.gputorch.prof_reset()
     gt.gputorch.prof_enable(True)
     try:
+        # the property the entry point exists for: no hipMalloc / hipFree by the library during the call, the block
+        # cache untouched (the counter covers storage blocks, the growing split workspace and the offset tables)
+        allocs, cached = lib.thgpu_device_alloc_calls(), lib.thgpu_cached_bytes()
         rc = lib.thgpu_gemm_noalloc(ta.encode(), tb.encode(), m, n, k, alpha, ptr(gt, da), lda, ptr(gt, db), ldb, beta,
                                     ptr(gt, c_new), ldc)
         gt._lib.check_status(rc)
+        assert lib.thgpu_device_alloc_calls() == allocs and lib.thgpu_cached_bytes() == cached
         gt.gputorch.synchronize()
         labels = [key for key in gt.gputorch.prof_report() if key.startswith("gemm_blas_noalloc")]
     finally:
