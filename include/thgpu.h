@@ -460,6 +460,32 @@ int thgpu_SpatialConvolutionMM_accGradParametersFused(THGPUTensor *input, THGPUT
                                                       THGPUTensor *gradWeight, THGPUTensor *gradBias,
                                                       THGPUTensor *finput, THGPUTensor *fgradInput, int kW, int kH,
                                                       int dW, int dH, int padW, int padH, float scale, int flags);
+/* The padded gradient without a copy (no counterpart in the reference).  On the gathered route updateGradInput reads
+ * gradOutput from a zero-bordered copy at the head of fgradInput.  Inside a container that knows which module
+ * produces a layer's gradOutput, that producer can store its result there as well while it stores it densely:
+ *   1. thgpu_SpatialConvolutionMM_gradOutputTwin (the layer's own input, weight, fgradInput and geometry): sizes
+ *      fgradInput for the gathered gradInput product, zeroes its padded region unless it is known to be zero-bordered
+ *      for this geometry already, and makes `twin` a [B,] M, Ho, Wo view of gradOutput's place in it.  *available is 0
+ *      (and nothing is touched) when the layer's gradInput does not take the gathered route.
+ *   2. the producer's updateGradInput -- thgpu_SpatialMaxPooling_updateGradInputTwin or
+ *      thgpu_SpatialConvolutionMM_updateGradInputTwin with that `twin` -- stores every value of its gradInput a second
+ *      time through the view; *wrote_twin says whether the kernel that ran could (the max-pooling cell kernel and the
+ *      unit-stride gathered gradInput product can; otherwise only the dense result is written).
+ *   3. the layer's thgpu_SpatialConvolutionMM_updateGradInputTwin with THGPU_GRADOUTPUT_IN_TWIN, called with that
+ *      dense gradInput as gradOutput before anything else touches either tensor: no padded copy is made.  The flag
+ *      is the caller's word for the contents; it is ignored (the copy is made) unless fgradInput is still the buffer
+ *      step 1 prepared for this geometry.
+ * Results are bit-identical to the plain entry points'.  `twin` may be NULL in the *Twin entry points (no second
+ * copy); flags also take THGPU_FUSE_INPUT_MASK with `threshold` as in updateGradInputFused / ...Masked. */
+#define THGPU_GRADOUTPUT_IN_TWIN 8 /* SpatialConvolutionMM_updateGradInputTwin */
+int thgpu_SpatialConvolutionMM_gradOutputTwin(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *fgradInput,
+                                              THGPUTensor *twin, int kW, int kH, int dW, int dH, int padW, int padH,
+                                              int *available);
+int thgpu_SpatialConvolutionMM_updateGradInputTwin(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *weight,
+                                                   THGPUTensor *finput, THGPUTensor *fgradInput,
+                                                   THGPUTensor *gradInput, int kW, int kH, int dW, int dH, int padW,
+                                                   int padH, int flags, float threshold, THGPUTensor *twin,
+                                                   int *wrote_twin);
 /* 1 when updateOutput / accGradParameters of a layer with these sizes would gather from the padded image in the
  * current mode (and so profit from an input that already lies in a padded buffer), 0 otherwise. */
 int thgpu_conv_gathers(long B, int C, int H, int W, int M, int kW, int kH, int dW, int dH, int padW, int padH);
@@ -500,6 +526,10 @@ int thgpu_SpatialMaxPooling_updateGradInput(THGPUTensor *input, THGPUTensor *gra
 
 /* updateGradInput with the backward of a Threshold in front of the pooling layer applied as gradInput is stored:
  * gradInput = input > threshold ? g : 0 (see thgpu_SpatialConvolutionMM_updateGradInputFused). */
+/* ... and with a second copy of gradInput stored through `twin` (see thgpu_SpatialConvolutionMM_gradOutputTwin). */
+int thgpu_SpatialMaxPooling_updateGradInputTwin(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *gradInput,
+                                                THGPUTensor *indices, int kW, int kH, int dW, int dH, int flags,
+                                                float threshold, THGPUTensor *twin, int *wrote_twin);
 int thgpu_SpatialMaxPooling_updateGradInputMasked(THGPUTensor *input, THGPUTensor *gradOutput,
                                                   THGPUTensor *gradInput, THGPUTensor *indices, int kW, int kH,
                                                   int dW, int dH, float threshold);

@@ -204,6 +204,11 @@ _SIGNATURES = {
     "thgpu_SpatialConvolutionMM_updateGradInputFused": (c_int, [TensorP] * 6 + [c_int] * 7 + [c_float]),
     "thgpu_SpatialConvolutionMM_accGradParametersFused": (c_int, [TensorP] * 6 + [c_int] * 6 + [c_float, c_int]),
     "thgpu_conv_gathers": (c_int, [c_long] + [c_int] * 10),
+    "thgpu_SpatialConvolutionMM_gradOutputTwin": (c_int, [TensorP] * 4 + [c_int] * 6 + [ctypes.POINTER(c_int)]),
+    "thgpu_SpatialConvolutionMM_updateGradInputTwin": (c_int, [TensorP] * 6 + [c_int] * 7 + [c_float, TensorP,
+                                                               ctypes.POINTER(c_int)]),
+    "thgpu_SpatialMaxPooling_updateGradInputTwin": (c_int, [TensorP] * 4 + [c_int] * 5 + [c_float, TensorP,
+                                                            ctypes.POINTER(c_int)]),
     "thgpu_SpatialMaxPooling_updateGradInputMasked": (c_int, [TensorP] * 4 + [c_int] * 4 + [c_float]),
     "thgpu_SpatialMaxPooling_updateOutput": (c_int, [TensorP] * 3 + [c_int] * 4),
     "thgpu_SpatialMaxPooling_updateGradInput": (c_int, [TensorP] * 4 + [c_int] * 4),

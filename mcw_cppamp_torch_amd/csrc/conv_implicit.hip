@@ -25,6 +25,7 @@
 // other products times (A*dH/kH)*(Bk*dW/kW) (taps rounded up to whole strides).
 #include "gemm_mfma.h"
 #include "kernels.h"
+#include "side_jobs.h"
 
 #include <array>
 #include <cstdlib>
@@ -74,40 +75,6 @@ __device__ __forceinline__ void pad_four(const PadJob &j, unsigned block) {
 }
 
 __global__ __launch_bounds__(256) void pad_planes_kernel(const PadJob j) { pad_four(j, blockIdx.x); }
-
-// The kernel bank as the first operand of a gradInput product, one element per lane:
-//   unit stride:  wt[c][m][kh][kw] = w[m][c][kH-1-kh][kW-1-kw]
-//   strided:      wt[(c, ph, pw)][(m, a', b')] = w[m][c][ph + sH*(A-1-a')][pw + sW*(Bk-1-b')], zero where that tap lies
-//                 outside the kernel and in the rows beyond C*sH*sW (the product's rows are padded to a whole tile).
-struct WeightJob {
-    const float *w;
-    float *wt;
-    int M, C, kH, kW;
-    int sH, sW, A, Bk, rows, rows_pad;  // strided form only (sH = 0: unit stride)
-    unsigned count;                     // elements of wt
-};
-
-__device__ __forceinline__ void reorder_weight(const WeightJob &j, unsigned idx) {
-    if (idx >= j.count) return;
-    if (j.sH == 0) {
-        const unsigned kk = (unsigned)(j.kH * j.kW);
-        const unsigned tap = idx % kk, cm = idx / kk;
-        const unsigned m = cm % j.M, c = cm / j.M;
-        const unsigned kh = tap / j.kW, kw = tap % j.kW;
-        j.wt[idx] = j.w[((long)m * j.C + c) * kk + (j.kH - 1 - kh) * j.kW + (j.kW - 1 - kw)];
-        return;
-    }
-    const unsigned R = (unsigned)(j.M * j.A * j.Bk);
-    const unsigned row = idx / R, r = idx % R;
-    float v = 0.0f;
-    if (row < (unsigned)j.rows) {
-        const unsigned pw = row % j.sW, ph = (row / j.sW) % j.sH, c = row / (j.sW * j.sH);
-        const unsigned bb = r % j.Bk, aa = (r / j.Bk) % j.A, m = r / (j.Bk * j.A);
-        const unsigned kh = ph + j.sH * (j.A - 1 - aa), kw = pw + j.sW * (j.Bk - 1 - bb);
-        if (kh < (unsigned)j.kH && kw < (unsigned)j.kW) v = j.w[(((long)m * j.C + c) * j.kH + kh) * j.kW + kw];
-    }
-    j.wt[idx] = v;
-}
 
 // Both preparations of a gradInput product in one launch (they are independent, and the kernel bank alone is a
 // launch of a few microseconds of work): the first pad_blocks workgroups pad gradOutput, the rest re-order the bank.
@@ -313,7 +280,72 @@ GemmProblem gradinput_strided_problem(long B, int C, int H, int W, int M, int kH
     return p;
 }
 
+WeightJob bank_job(const float *weight, float *wt, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH,
+                   int sW) {
+    WeightJob wj;
+    wj.w = weight;
+    wj.wt = wt;
+    wj.M = M;
+    wj.C = C;
+    wj.kH = kH;
+    wj.kW = kW;
+    if (sH != 1 || sW != 1) {
+        const PhaseGeom q = phase_geom(C, H, W, kH, kW, pH, pW, sH, sW);
+        wj.sH = sH;
+        wj.sW = sW;
+        wj.A = q.A;
+        wj.Bk = q.Bk;
+        wj.rows = q.rows;
+        wj.rows_pad = q.rows_pad;
+        wj.count = (unsigned)((long)q.rows_pad * M * q.A * q.Bk);
+    } else {
+        wj.sH = wj.sW = wj.A = wj.Bk = wj.rows = wj.rows_pad = 0;
+        wj.count = (unsigned)((long)M * C * kH * kW);
+    }
+    return wj;
+}
+
+// The pending bank job, and the bank that the last carrier re-ordered (see side_jobs.h).  Two records: a convolution
+// that consumes a carried job is, in the same call, the producer whose launch carries the next layer's.
+WeightJob g_bank_job = {};
+bool g_bank_pending = false;
+const float *g_bank_carried = nullptr;
+
 }  // namespace
+
+void offer_bank_job(const WeightJob &job) {
+    g_bank_job = job;
+    g_bank_pending = job.count > 0;
+    if (g_bank_carried == job.wt) g_bank_carried = nullptr;  // a record left over from a pass that never reached its product
+}
+
+bool take_bank_job(WeightJob &job) {
+    if (!g_bank_pending) return false;
+    job = g_bank_job;
+    g_bank_pending = false;
+    g_bank_carried = job.wt;
+    return true;
+}
+
+bool bank_job_done(const float *wt) {
+    const bool done = g_bank_carried == wt && wt != nullptr;
+    g_bank_carried = nullptr;
+    if (g_bank_pending && g_bank_job.wt == wt) g_bank_pending = false;  // nobody carried it: the product does it itself
+    return done;
+}
+
+void conv_implicit_offer_bank(const float *weight, float *scratch, long B, int C, int H, int W, int M, int kH, int kW,
+                              int pH, int pW, int sH, int sW) {
+    int top, left, Hq, Wq;
+    conv_implicit_q_layout(C, H, W, kH, kW, pH, pW, sH, sW, &top, &left, &Hq, &Wq);
+    long nw = (long)M * C * kH * kW;
+    if (sH != 1 || sW != 1) {
+        const PhaseGeom q = phase_geom(C, H, W, kH, kW, pH, pW, sH, sW);
+        nw = (long)q.rows_pad * M * q.A * q.Bk;
+    }
+    if (nw >= (1L << 31)) return;  // the product itself will refuse
+    offer_bank_job(bank_job(weight, scratch + B * M * (long)Hq * Wq, C, H, W, M, kH, kW, pH, pW, sH, sW));
+}
 
 int conv_mode() {
     if (g_mode < 0) {
@@ -409,8 +441,9 @@ static int pad_planes_into(const float *in, long planes, int H, int W, int top, 
     if (total <= 0 && !wj) return 0;
     if (total >= (1L << 31)) return fail("pad: %ld elements exceed 32-bit indexing", total);
     {
-        const char *label = prof_enabled() ? prof_label("pad_planes planes=%ld %dx%d p=%dx%d", planes, H, W, top, left)
-                                           : "pad_planes";
+        const char *label = planes == 0 ? "kernel_bank_reorder"
+                            : prof_enabled() ? prof_label("pad_planes planes=%ld %dx%d p=%dx%d", planes, H, W, top, left)
+                                             : "pad_planes";
         const double wbytes = wj ? 4.0 * (wj->count + (double)wj->M * wj->C * wj->kH * wj->kW) : 0.0;
         LaunchScope scope(label, 0.0, 4.0 * (total + planes * H * W) + wbytes);
         PadJob pj;
@@ -436,6 +469,22 @@ static int pad_planes_into(const float *in, long planes, int H, int W, int top, 
         }
     }
     return check_launch("pad_planes");
+}
+
+void conv_implicit_q_layout(int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW, int *top, int *left,
+                            int *Hq, int *Wq) {
+    if (sH != 1 || sW != 1) {
+        const PhaseGeom q = phase_geom(C, H, W, kH, kW, pH, pW, sH, sW);
+        *top = q.A - 1;
+        *left = q.Bk - 1;
+        *Hq = q.Hq;
+        *Wq = q.Wq;
+        return;
+    }
+    *top = kH - 1 - pH;
+    *left = kW - 1 - pW;
+    *Hq = H + kH - 1;
+    *Wq = W + kW - 1;
 }
 
 int pad_planes_launch(const float *in, long planes, int H, int W, int pH, int pW, float *out) {
@@ -492,7 +541,7 @@ int conv_implicit_gradweight(const float *padded, const float *gradOutput, float
 // gradInput of a strided layer as one product over the residue classes of the pixel coordinates.
 static int conv_implicit_gradinput_strided(const float *gradOutput, const float *weight, float *scratch,
                                            float *gradInput, long B, int C, int H, int W, int M, int kH, int kW, int pH,
-                                           int pW, int sH, int sW, InputMask mask) {
+                                           int pW, int sH, int sW, InputMask mask, bool q_ready) {
     hipStream_t s = stream();
     if (!s) return 1;
     if (mask.in && (mask.pitch > 0 || (mask.plane > 0 && mask.plane != (long)H * W)))
@@ -503,21 +552,13 @@ static int conv_implicit_gradinput_strided(const float *gradOutput, const float 
     float *Wt = scratch + B * M * (long)q.Hq * q.Wq;
     const long nw = (long)q.rows_pad * M * q.A * q.Bk;
     if (nw >= (1L << 31)) return fail("SpatialConvolutionMM: kernel bank too large for the strided gradInput product");
-    WeightJob wj;
-    wj.w = weight;
-    wj.wt = Wt;
-    wj.M = M;
-    wj.C = C;
-    wj.kH = kH;
-    wj.kW = kW;
-    wj.sH = sH;
-    wj.sW = sW;
-    wj.A = q.A;
-    wj.Bk = q.Bk;
-    wj.rows = q.rows;
-    wj.rows_pad = q.rows_pad;
-    wj.count = (unsigned)nw;
-    if (pad_planes_into(gradOutput, B * M, Ho, Wo, q.A - 1, q.Bk - 1, q.Hq, q.Wq, Q, &wj)) return 1;
+    const WeightJob wj = bank_job(weight, Wt, C, H, W, M, kH, kW, pH, pW, sH, sW);
+    // With gradOutput already in place only the kernel bank is re-ordered (zero planes to pad), unless a launch before
+    // this one has carried that job along.
+    const bool bank_done = bank_job_done(Wt);
+    if (!(q_ready && bank_done) &&
+        pad_planes_into(gradOutput, q_ready ? 0 : B * M, Ho, Wo, q.A - 1, q.Bk - 1, q.Hq, q.Wq, Q, &wj))
+        return 1;
     if (trim_tables()) return 1;
     GemmProblem p = gradinput_strided_problem(B, C, H, W, M, kH, kW, pH, pW, sH, sW);
     p.A = Wt;
@@ -532,10 +573,12 @@ static int conv_implicit_gradinput_strided(const float *gradOutput, const float 
 }
 
 int conv_implicit_gradinput(const float *gradOutput, const float *weight, float *scratch, float *gradInput, long B,
-                            int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW, InputMask mask) {
-    if (sH != 1 || sW != 1)
+                            int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW, InputMask mask,
+                            bool q_ready, TwinOutput twin, bool *wrote_twin) {
+    if (wrote_twin) *wrote_twin = false;
+    if (sH != 1 || sW != 1)  // (the scattered store keeps no second copy)
         return conv_implicit_gradinput_strided(gradOutput, weight, scratch, gradInput, B, C, H, W, M, kH, kW, pH, pW, sH,
-                                               sW, mask);
+                                               sW, mask, q_ready);
     hipStream_t s = stream();
     if (!s) return 1;
     const int Ho = H + 2 * pH - kH + 1, Wo = W + 2 * pW - kW + 1;
@@ -545,16 +588,10 @@ int conv_implicit_gradinput(const float *gradOutput, const float *weight, float 
     float *Wt = scratch + B * M * (long)Hq * Wq;
     const long nw = (long)M * C * kH * kW;
     if (nw >= (1L << 31)) return fail("SpatialConvolutionMM: kernel bank too large for the gradInput product");
-    WeightJob wj;
-    wj.w = weight;
-    wj.wt = Wt;
-    wj.M = M;
-    wj.C = C;
-    wj.kH = kH;
-    wj.kW = kW;
-    wj.sH = wj.sW = wj.A = wj.Bk = wj.rows = wj.rows_pad = 0;
-    wj.count = (unsigned)nw;
-    if (pad_planes_into(gradOutput, B * M, Ho, Wo, qH, qW, Hq, Wq, Q, &wj)) return 1;
+    const WeightJob wj = bank_job(weight, Wt, C, H, W, M, kH, kW, pH, pW, sH, sW);
+    const bool bank_done = bank_job_done(Wt);
+    if (!(q_ready && bank_done) && pad_planes_into(gradOutput, q_ready ? 0 : B * M, Ho, Wo, qH, qW, Hq, Wq, Q, &wj))
+        return 1;
     if (trim_tables()) return 1;
     GemmProblem p = gradinput_problem(B, C, H, W, M, kH, kW, pH, pW);
     p.A = Wt;
@@ -572,6 +609,15 @@ int conv_implicit_gradinput(const float *gradOutput, const float *weight, float 
     if (mask.in && mask.pitch > 0) {
         p.mask_pitch = mask.pitch;
         p.c_w = W;
+    }
+    if (twin.base) {
+        p.C2 = twin.base;
+        p.c2_sC = twin.plane;
+        p.c2_bsC = (long)C * twin.plane;
+        p.c2_pitch = twin.pitch;
+        p.c_w = W;
+        if (!gemm_tiled_fits(p)) p.C2 = nullptr;  // the copy's offsets exceed the kernels' addressing: do without
+        if (wrote_twin) *wrote_twin = p.C2 != nullptr;
     }
     return gemm_launch(p);
 }

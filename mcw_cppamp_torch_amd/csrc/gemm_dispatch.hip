@@ -3,6 +3,7 @@
 // when the reduction was split, the fixed-order reduction of the partial sums.
 // Also the THGPUBlas_gemm entry point.
 #include "gemm_mfma.h"
+#include "side_jobs.h"
 
 #include <cstring>
 
@@ -42,7 +43,14 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(const RowSumJob rs, c
                                                            float alpha, float beta, int act, float act_threshold,
                                                            float act_value, const float *__restrict__ mask,
                                                            float mask_threshold, int c_pitch, int mask_pitch,
-                                                           long mask_sC, long mask_bsC, FastDiv divCW) {
+                                                           long mask_sC, long mask_bsC, FastDiv divCW,
+                                                           float *__restrict__ C2, long c2_sC, long c2_bsC, int c2_pitch,
+                                                           const unsigned side_first_block, const WeightJob side) {
+    // workgroups behind the reduction's carry a job of the next layer's (side_jobs.h)
+    if (blockIdx.x >= side_first_block) {
+        reorder_weight(side, (blockIdx.x - side_first_block) * 256u + threadIdx.x);
+        return;
+    }
     if (rs.out && blockIdx.x >= rs.first_block) {
         rowsum_reduce(rs, blockIdx.x - rs.first_block);
         return;
@@ -78,13 +86,14 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(const RowSumJob rs, c
     }
     unsigned i, j;
     divJ.divmod(idx, i, j);
-    long coff = j, moff = j;
-    if (N != J || c_pitch || mask_pitch) {
+    long coff = j, moff = j, toff = 0;
+    if (N != J || c_pitch || mask_pitch || C2) {
         unsigned im, n, y, x;
         divN.divmod(j, im, n);
         divCW.divmod(n, y, x);
         coff = (long)im * bsC + (c_pitch ? (long)y * c_pitch + x : (long)n);
         moff = (long)im * mask_bsC + (mask_pitch ? (long)y * mask_pitch + x : (long)n);
+        toff = (long)im * c2_bsC + (long)y * c2_pitch + x;
     }
     float *c = C + (long)i * sC + coff;
     float val = alpha * sum;
@@ -93,6 +102,7 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(const RowSumJob rs, c
     if (act) val = val > act_threshold ? val : act_value;
     if (mask) val = mask[(long)i * mask_sC + moff] > mask_threshold ? val : 0.0f;
     *c = val;
+    if (C2) C2[(long)i * c2_sC + toff] = val;  // the second copy (GemmProblem::C2)
 }
 
 struct TileCfg {
@@ -193,7 +203,8 @@ GemmPlan plan_gemm(const GemmProblem &p, int steps_total) {
                           : p.b_rc ? (long)(bn - 1) * p.sB + GEMM_BK
                                    : (long)(GEMM_BK - 1) * p.sB + span * p.bsB + n_img;
         const long offC = 4 * (p.sC > p.J ? p.sC : (long)p.J) + span * p.bsC + n_img;
-        return offA < (1L << 30) && offB < (1L << 30) && offC < (1L << 30);
+        const long offC2 = p.C2 ? 4 * p.c2_sC + span * p.c2_bsC + (p.c_w > 0 ? n_img / p.c_w : 0) * p.c2_pitch + p.c_w : 0;
+        return offA < (1L << 30) && offB < (1L << 30) && offC < (1L << 30) && offC2 < (1L << 30);
     };
     const bool fast_ok = p.R == 0 || p.R >= GEMM_BK;
     const int layout = gather ? 4 : p.a_rc ? (p.b_rc ? 2 : 0) : (p.b_rc ? 3 : 1);
@@ -281,6 +292,14 @@ int gemm_launch(const GemmProblem &p) {
     g.mask_sC = p.mask_sC ? p.mask_sC : p.sC;
     g.mask_bsC = p.mask_bsC ? p.mask_bsC : p.bsC;
     g.divCW = FastDiv((uint32_t)g.c_w);
+    if (p.C2) {
+        if (red || p.scatter || p.c_w <= 0 || g.N % p.c_w != 0 || p.c2_pitch < p.c_w || p.c2_sC <= 0 || p.c2_bsC <= 0)
+            return fail("gemm: a second copy of the result needs column batching, a plane width and the copy's strides");
+        g.C2 = p.C2;
+        g.c2_sC = p.c2_sC;
+        g.c2_bsC = p.c2_bsC;
+        g.c2_pitch = p.c2_pitch;
+    }
     if (p.scatter) {
         if (!gather || red || p.bias || p.beta != 0.0f || p.c_pitch || p.mask_pitch || p.c_w <= 0 || g.N % p.c_w != 0 ||
             p.scat_sH <= 0 || p.scat_sW <= 0 || p.scat_H <= 0 || p.scat_W <= 0 || p.scat_rows <= 0 || p.scat_rows > p.M ||
@@ -350,6 +369,7 @@ int gemm_launch(const GemmProblem &p) {
     const int la = p.a_rc ? LD_RC_VEC : LD_XC_SCALAR;
     const int lb = p.b_rc ? LD_RC_VEC : gather ? LD_XC_GATHER : LD_XC_SCALAR;
     if (gather && !best) return fail("gemm: a gathered B needs a shape the tiled kernel takes (M, J >= 64, R >= 16)");
+    if (p.C2 && !best) return fail("gemm: a second copy of the result needs a shape the tiled kernel takes");
 
     int rc;
     {
@@ -378,13 +398,24 @@ int gemm_launch(const GemmProblem &p) {
             rs.first_block = blocks;
             blocks += (unsigned)cdiv(p.M, 4);
         }
+        // A product that stores a second copy of its result for the next layer's gradInput product also carries that
+        // layer's pending kernel-bank job, if there is one.
+        WeightJob side = {};
+        const unsigned side_first = blocks;
+        double side_bytes = 0.0;
+        if (g.C2 && n > 0 && take_bank_job(side)) {
+            blocks += (side.count + 255u) / 256u;
+            side_bytes = 4.0 * (side.count + (double)side.M * side.C * side.kH * side.kW);
+        }
         {
-            LaunchScope scope("gemm_split_reduce", 0.0, 4.0 * n * (g.nsplit + 2) + 4.0 * rowsum_floats);
+            LaunchScope scope("gemm_split_reduce", 0.0,
+                              4.0 * n * (g.nsplit + 2 + (g.C2 ? 1 : 0)) + 4.0 * rowsum_floats + side_bytes);
             auto kernel = quarters ? split_reduce_kernel<true> : split_reduce_kernel<false>;
             hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, s, rs, g.ws, p.C, p.bias,
                                p.M, p.J, g.N, p.sC, p.bsC, FastDiv((uint32_t)p.J), g.divN, g.nsplit, p.alpha,
                                p.beta, g.act, g.act_threshold, g.act_value, g.mask, g.mask_threshold, g.c_pitch,
-                               g.mask_pitch, g.mask_sC, g.mask_bsC, g.divCW);
+                               g.mask_pitch, g.mask_sC, g.mask_bsC, g.divCW, g.C2, g.c2_sC, g.c2_bsC, g.c2_pitch,
+                               side_first, side);
         }
         if (check_launch("gemm_split_reduce")) return 1;
     }

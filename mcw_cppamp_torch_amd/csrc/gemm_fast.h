@@ -517,28 +517,33 @@ __global__ __launch_bounds__(WGM *WGN * 64)
         const long mask_row_bytes = g.mask_sC * 4;
         unsigned img0 = 0, n0 = 0;
         // columns are (image, position) pairs, or positions of an image plane whose rows are kept apart
-        const bool per_image = MODE != 0 && !RED && (g.N != g.J || g.c_pitch != 0 || g.mask_pitch != 0);
+        const bool twin = MODE != 0 && !RED && g.C2 != nullptr;  // a second copy of the result (GemmProblem::C2)
+        const long twin_row_bytes = g.c2_sC * 4;
+        const bool per_image = MODE != 0 && !RED && (g.N != g.J || g.c_pitch != 0 || g.mask_pitch != 0 || twin);
         if (per_image) g.divN.divmod((unsigned)j0, img0, n0);
         char *const out = out0 + (per_image ? (long)img0 * g.bsC : (long)j0) * 4;
         const char *const msk = reinterpret_cast<const char *>(g.mask) + (per_image ? (long)img0 * g.mask_bsC : (long)j0) * 4;
+        char *const out2 = reinterpret_cast<char *>(g.C2) + (long)img0 * g.c2_bsC * 4;
         // Per 32-column block of the wavefront: the lane's byte offset (into C, into the mask) and whether this tile
         // owns the column.
-        unsigned voff[TN], mvoff[TN];
+        unsigned voff[TN], mvoff[TN], tvoff[TN];
         bool own[TN];
 #pragma unroll
         for (int b = 0; b < TN; ++b) {
             const int jg = j0 + wn * (TN * 32) + b * 32 + l32;
             own[b] = jg >= own_j0;  // else the neighbouring tile stores it
-            long col = jg - j0, mcol = jg - j0;
+            long col = jg - j0, mcol = jg - j0, tcol = 0;
             if (per_image) {
                 unsigned im, n, y, x;
                 g.divN.divmod((unsigned)jg, im, n);
                 g.divCW.divmod(n, y, x);
                 col = (long)(im - img0) * g.bsC + (g.c_pitch ? (long)y * g.c_pitch + x : (long)n);
                 mcol = (long)(im - img0) * g.mask_bsC + (g.mask_pitch ? (long)y * g.mask_pitch + x : (long)n);
+                tcol = (long)(im - img0) * g.c2_bsC + (long)y * g.c2_pitch + x;
             }
             voff[b] = (unsigned)(col * 4 + 4 * half * row_bytes);
             mvoff[b] = (unsigned)(mcol * 4 + 4 * half * mask_row_bytes);
+            tvoff[b] = (unsigned)(tcol * 4 + 4 * half * twin_row_bytes);
         }
         // Rows outermost, the wavefront's column blocks innermost: the stores of one output row follow each other
         // directly, so a cache line that two neighbouring 128-byte segments share (rows are rarely 128-byte aligned)
@@ -573,6 +578,7 @@ __global__ __launch_bounds__(WGM *WGN * 64)
                         val = mv > g.mask_threshold ? val : 0.0f;
                     }
                     *c = val;
+                    if (twin) *reinterpret_cast<float *>(out2 + (long)ir * twin_row_bytes + tvoff[b]) = val;
                 }
             }
         }

@@ -57,6 +57,13 @@ struct GemmProblem {
     // (0: those of C).
     int c_w = 0, c_pitch = 0, mask_pitch = 0;
     long mask_sC = 0, mask_bsC = 0;
+    // Column batching with c_w set: a second copy of every final value (after alpha, bias, beta, act and mask) goes to
+    // C2, element (row i, image, y, x) at C2[image*c2_bsC + i*c2_sC + y*c2_pitch + x] -- the same image planes kept
+    // in another layout, e.g. the interior of a zero-bordered buffer that the next product gathers from, so that no
+    // padded copy of C has to be made afterwards.  nullptr: off.  Not with a scattered store.
+    float *C2 = nullptr;
+    long c2_sC = 0, c2_bsC = 0;
+    int c2_pitch = 0;
     // Scattered store (column batching, no bias, beta = 0, never split): row i of the product is a (plane, row
     // phase, column phase) triple, i = (c*scat_sH + ph)*scat_sW + pw, column n of an image a cell (y, x) of a grid
     // c_w wide, and element (i, (image, y, x)) goes to
@@ -119,6 +126,9 @@ struct GemmArgs {
     int c_w, c_pitch, mask_pitch;
     long mask_sC, mask_bsC;
     FastDiv divCW;
+    float *C2;  // see GemmProblem
+    long c2_sC, c2_bsC;
+    int c2_pitch;
     int scatter;  // see GemmProblem
     int scat_sH, scat_sW, scat_pH, scat_pW, scat_H, scat_W, scat_rows;
     FastDiv divScatS, divScatW;  // a row index by sH*sW and its remainder by sW

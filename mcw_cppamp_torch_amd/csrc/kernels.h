@@ -24,6 +24,16 @@ struct OutputLayout {
     int pitch = 0;
 };
 
+// A second copy of a [B, C, H, W] result kept inside another buffer: element (plane, y, x) at
+// base[plane*plane_stride + y*pitch + x] (planes of all images evenly spaced).  base == nullptr: none.  This is how
+// the producer of a gradient writes it straight into the zero-bordered buffer that the convolution in front gathers
+// its gradInput product from, so that no padded copy is made afterwards.
+struct TwinOutput {
+    float *base = nullptr;
+    long plane = 0;
+    int pitch = 0;
+};
+
 int im2col_launch(const float *im, long B, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW,
                   float *col);
 int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW,
@@ -31,8 +41,10 @@ int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW,
 // out_plane / out_pitch: floats between the output's planes and rows when it is not densely packed (0: dense).
 int maxpool_fwd_launch(const float *in, long planes, int H, int W, int kH, int kW, int dH, int dW, float *out,
                        float *indices, long out_plane = 0, int out_pitch = 0);
+// *wrote_twin (when twin.base is set) says whether the kernel that ran also stored the second copy.
 int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int H, int W, int Ho, int Wo, int kH,
-                       int kW, int dH, int dW, float *gin, InputMask mask = InputMask());
+                       int kW, int dH, int dW, float *gin, InputMask mask = InputMask(), TwinOutput twin = TwinOutput(),
+                       bool *wrote_twin = nullptr);
 int threshold_fwd_launch(const float *in, float *out, long n, float th, float val);
 int threshold_bwd_launch(const float *in, const float *gout, float *gin, long n, float th);
 int gradbias_launch(const float *gout, float *gbias, long B, int M, long N, float scale);
@@ -63,9 +75,24 @@ int conv_implicit_forward(const float *padded, const float *weight, const float 
 int conv_implicit_gradweight(const float *padded, const float *gradOutput, float *gradWeight, long B, int C, int H,
                              int W, int M, int kH, int kW, int pH, int pW, int sH, int sW, float scale, float *gradBias,
                              bool *bias_done);
+// q_ready: the head of `scratch` already holds gradOutput in the padded layout conv_implicit_q_layout describes
+// (its producer wrote it there through a TwinOutput, borders zero), so no padded copy is made.  twin: a second copy of
+// gradInput (unit-stride layers only; *wrote_twin says whether it was stored).
 int conv_implicit_gradinput(const float *gradOutput, const float *weight, float *scratch, float *gradInput, long B,
                             int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW,
-                            InputMask mask = InputMask());
+                            InputMask mask = InputMask(), bool q_ready = false, TwinOutput twin = TwinOutput(),
+                            bool *wrote_twin = nullptr);
+// Where gradOutput [B, M, Ho, Wo] lies inside the padded buffer the gathered gradInput product reads (the head of its
+// scratch): planes of Hq x Wq, the dense plane at row `top`, column `left`, zeros around it.
+void conv_implicit_q_layout(int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW, int *top, int *left,
+                            int *Hq, int *Wq);
+// Offers the re-ordering of the layer's kernel bank (into the tail of `scratch`, where the gradInput product expects
+// it) to the launches that come before that product (side_jobs.h).
+void conv_implicit_offer_bank(const float *weight, float *scratch, long B, int C, int H, int W, int M, int kH, int kW,
+                              int pH, int pW, int sH, int sW);
+// Forgets what is known about a device buffer that is being released (nn_ops.hip keeps track of buffers whose borders
+// it has zeroed).
+void conv_forget_buffer(const float *p);
 
 // Host-only checks of the launch planners (no GPU needed); each returns the number of violations.
 long im2col_plan_selftest();

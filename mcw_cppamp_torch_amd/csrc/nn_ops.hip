@@ -8,6 +8,8 @@
 #include "gemm_mfma.h"
 #include "kernels.h"
 
+#include <map>
+
 using namespace thgpu;
 
 namespace {
@@ -129,6 +131,49 @@ void set_output_layout(GemmProblem &p, const PlaneLayout &l, int planes_per_imag
     }
 }
 
+// ---- gradOutput delivered in the padded layout of the gathered gradInput product ("the twin") --------------------
+// Geometry of that layout for one layer, and the buffers (by device address of fgradInput's first element) whose
+// padded region is known to have zero borders: zeroed here, or written whole by the padding kernel.  A buffer leaves
+// the list when its memory is released (conv_forget_buffer) or when another route writes something else into it.
+struct TwinGeom {
+    long B;
+    int M, Ho, Wo, top, left, Hq, Wq;
+    bool operator==(const TwinGeom &o) const {
+        return B == o.B && M == o.M && Ho == o.Ho && Wo == o.Wo && top == o.top && left == o.left && Hq == o.Hq &&
+               Wq == o.Wq;
+    }
+};
+std::map<const float *, TwinGeom> g_zero_bordered;
+
+TwinGeom twin_geom(const ConvShape &s, int kH, int kW, int padH, int padW, int dH, int dW) {
+    TwinGeom t;
+    t.B = s.B;
+    t.M = s.M;
+    t.Ho = s.Ho;
+    t.Wo = s.Wo;
+    conv_implicit_q_layout(s.C, s.H, s.W, kH, kW, padH, padW, dH, dW, &t.top, &t.left, &t.Hq, &t.Wq);
+    return t;
+}
+
+bool zero_bordered(const float *q, const TwinGeom &t) {
+    auto it = g_zero_bordered.find(q);
+    return it != g_zero_bordered.end() && it->second == t;
+}
+
+// `twin` as a kernel operand when it is a usable second copy of a [B,] C, H, W result: same sizes, rows contiguous,
+// planes evenly spaced, memory behind it, and no overlap with the result itself.
+bool twin_output(const THGPUTensor *twin, const THGPUTensor *like, TwinOutput &out) {
+    PlaneLayout l;
+    if (!twin || !like || twin->nDimension != like->nDimension || !plane_layout(twin, l)) return false;
+    for (int d = 0; d < like->nDimension; ++d)
+        if (twin->size[d] != like->size[d]) return false;
+    if (twin->storage == like->storage) return false;
+    out.base = THGPUTensor_data(twin);
+    out.plane = l.plane;
+    out.pitch = (int)l.pitch;
+    return true;
+}
+
 int conv_update_output(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias, THGPUTensor *finput,
                        THGPUTensor *fgradInput, THGPUTensor *output, int kW, int kH, int dW, int dH, int padW,
                        int padH, OutputThreshold act, bool input_in_padded_buffer) {
@@ -212,9 +257,15 @@ int conv_update_output(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bia
 }
 
 // mask_on: gradInput is zeroed where `input` does not exceed mask_threshold.
+// twin_ready: the caller says that gradOutput's producer also wrote it into fgradInput through the view
+// thgpu_SpatialConvolutionMM_gradOutputTwin handed out (honoured only while the buffer is known to be zero-bordered
+// for this geometry; otherwise the padded copy is made as usual).  twin: a second copy of gradInput to keep, or null;
+// *wrote_twin says whether it was stored.
 int conv_update_grad_input(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *weight, THGPUTensor *finput,
                            THGPUTensor *fgradInput, THGPUTensor *gradInput, int kW, int kH, int dW, int dH,
-                           int padW, int padH, bool mask_on, float mask_threshold) {
+                           int padW, int padH, bool mask_on, float mask_threshold, bool twin_ready = false,
+                           THGPUTensor *twin = nullptr, int *wrote_twin = nullptr) {
+    if (wrote_twin) *wrote_twin = 0;
     (void)finput;
     ConvShape s;
     if (conv_shape(s, input, weight, kW, kH, dW, dH, padW, padH)) return 1;
@@ -261,14 +312,25 @@ int conv_update_grad_input(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTen
             THGPUTensor_resize4d(gradInput, s.B, s.C, s.H, s.W);
         else
             THGPUTensor_resize3d(gradInput, s.C, s.H, s.W);
+        // a delivered gradOutput is only trusted in the buffer it was handed out in: same memory, same geometry
+        const TwinGeom tg = twin_geom(s, kH, kW, padH, padW, dH, dW);
+        const bool q_ready = twin_ready && tensor_ready(fgradInput, need) && zero_bordered(dptr(fgradInput), tg);
         THGPUTensor_resize1d(fgradInput, need);
         if (!tensor_ready(fgradInput, need) || !tensor_ready(gradInput, s.B * (long)s.C * s.H * s.W))
             return fail("SpatialConvolutionMM: could not size gradInput/fgradInput");
         if (!(tensor_backed(go) && tensor_backed(weight)))
             return fail("SpatialConvolutionMM: a tensor's shape exceeds its storage");
-        return conv_implicit_gradinput(dptr(go), dptr(weight), dptr(fgradInput), dptr(gradInput), s.B, s.C, s.H, s.W,
-                                       s.M, kH, kW, padH, padW, dH, dW, mask);
+        TwinOutput second;
+        if (twin && !twin_output(twin, gradInput, second)) second = TwinOutput();
+        bool wrote = false;
+        const int rc = conv_implicit_gradinput(dptr(go), dptr(weight), dptr(fgradInput), dptr(gradInput), s.B, s.C, s.H,
+                                               s.W, s.M, kH, kW, padH, padW, dH, dW, mask, q_ready, second, &wrote);
+        // either way the padded region now holds this gradOutput between zero borders
+        if (!rc) g_zero_bordered[dptr(fgradInput)] = tg;
+        if (wrote_twin) *wrote_twin = !rc && wrote ? 1 : 0;
+        return rc;
     }
+    g_zero_bordered.erase(dptr(fgradInput));  // the gradient columns go there instead
     if (s.batched) {
         THGPUTensor_resize4d(gradInput, s.B, s.C, s.H, s.W);
         THGPUTensor_resize3d(fgradInput, s.B, s.K, s.N);
@@ -280,6 +342,7 @@ int conv_update_grad_input(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTen
         return fail("SpatialConvolutionMM: could not size gradInput/fgradInput");
     if (!(tensor_backed(go) && tensor_backed(weight)))
         return fail("SpatialConvolutionMM: a tensor's shape exceeds its storage");
+    g_zero_bordered.erase(dptr(fgradInput));
     {
         // fgradInput[b][k][n] = sum_m weight[m][k] * gradOutput[b][m][n]
         GemmProblem p;
@@ -401,6 +464,12 @@ int conv_acc_grad_parameters(THGPUTensor *input, THGPUTensor *gradOutput, THGPUT
 
 }  // namespace
 
+namespace thgpu {
+void conv_forget_buffer(const float *p) {
+    if (!g_zero_bordered.empty()) g_zero_bordered.erase(p);
+}
+}  // namespace thgpu
+
 extern "C" {
 
 int thgpu_SpatialConvolutionMM_updateOutput(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias,
@@ -438,6 +507,50 @@ int thgpu_SpatialConvolutionMM_updateGradInputFused(THGPUTensor *input, THGPUTen
     if (flags & ~THGPU_FUSE_INPUT_MASK) return fail("SpatialConvolutionMM: unknown flags");
     return conv_update_grad_input(input, gradOutput, weight, finput, fgradInput, gradInput, kW, kH, dW, dH, padW,
                                   padH, (flags & THGPU_FUSE_INPUT_MASK) != 0, threshold);
+}
+
+int thgpu_SpatialConvolutionMM_gradOutputTwin(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *fgradInput,
+                                              THGPUTensor *twin, int kW, int kH, int dW, int dH, int padW, int padH,
+                                              int *available) {
+    if (available) *available = 0;
+    ConvShape s;
+    if (conv_shape(s, input, weight, kW, kH, dW, dH, padW, padH)) return 1;
+    if (!fgradInput || !twin || !available) return fail("SpatialConvolutionMM: null argument");
+    if (!conv_use_gathered_gradinput(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW)) return 0;
+    const long need = conv_implicit_gradinput_scratch(s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW);
+    const TwinGeom tg = twin_geom(s, kH, kW, padH, padW, dH, dW);
+    const long q_floats = s.B * s.M * (long)tg.Hq * tg.Wq;
+    THGPUTensor_resize1d(fgradInput, need);
+    if (!tensor_ready(fgradInput, need)) return fail("SpatialConvolutionMM: could not size fgradInput");
+    float *q = dptr(fgradInput);
+    if (!zero_bordered(q, tg)) {
+        if (fill_device(q, q_floats, 0.0f)) return 1;
+        g_zero_bordered[q] = tg;
+    }
+    // the view of gradOutput's place inside the padded planes
+    const long off = fgradInput->storageOffset + (long)tg.top * tg.Wq + tg.left;
+    const long plane = (long)tg.Hq * tg.Wq;
+    if (s.batched)
+        THGPUTensor_setStorage4d(twin, fgradInput->storage, off, s.B, s.M * plane, s.M, plane, tg.Ho, tg.Wq, tg.Wo, 1);
+    else
+        THGPUTensor_setStorage3d(twin, fgradInput->storage, off, s.M, plane, tg.Ho, tg.Wq, tg.Wo, 1);
+    if (!tensor_backed(twin)) return fail("SpatialConvolutionMM: could not place the gradOutput view");
+    // the producer's launch may as well re-order this layer's kernel bank for the product that follows
+    if (require_contiguous(weight, "weight") || !tensor_backed(weight)) return 1;
+    conv_implicit_offer_bank(dptr(weight), q, s.B, s.C, s.H, s.W, s.M, kH, kW, padH, padW, dH, dW);
+    *available = 1;
+    return 0;
+}
+
+int thgpu_SpatialConvolutionMM_updateGradInputTwin(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *weight,
+                                                   THGPUTensor *finput, THGPUTensor *fgradInput,
+                                                   THGPUTensor *gradInput, int kW, int kH, int dW, int dH, int padW,
+                                                   int padH, int flags, float threshold, THGPUTensor *twin,
+                                                   int *wrote_twin) {
+    if (flags & ~(THGPU_FUSE_INPUT_MASK | THGPU_GRADOUTPUT_IN_TWIN)) return fail("SpatialConvolutionMM: unknown flags");
+    return conv_update_grad_input(input, gradOutput, weight, finput, fgradInput, gradInput, kW, kH, dW, dH, padW, padH,
+                                  (flags & THGPU_FUSE_INPUT_MASK) != 0, threshold,
+                                  (flags & THGPU_GRADOUTPUT_IN_TWIN) != 0, twin, wrote_twin);
 }
 
 int thgpu_SpatialConvolutionMM_accGradParameters(THGPUTensor *input, THGPUTensor *gradOutput,
@@ -501,7 +614,8 @@ int thgpu_SpatialMaxPooling_updateOutput(THGPUTensor *input, THGPUTensor *output
 
 static int pool_update_grad_input(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *gradInput,
                                   THGPUTensor *indices, int kW, int kH, int dW, int dH, bool mask_on,
-                                  float mask_threshold) {
+                                  float mask_threshold, THGPUTensor *twin = nullptr, int *wrote_twin = nullptr) {
+    if (wrote_twin) *wrote_twin = 0;
     if (!input || !gradOutput || !gradInput || !indices) return fail("SpatialMaxPooling: null tensor");
     if (!(input->nDimension == 3 || input->nDimension == 4)) return fail("3D or 4D (batch) tensor expected");
     if (kW <= 0 || kH <= 0 || dW <= 0 || dH <= 0) return fail("SpatialMaxPooling: invalid kernel/stride");
@@ -532,8 +646,14 @@ static int pool_update_grad_input(THGPUTensor *input, THGPUTensor *gradOutput, T
             mask.threshold = mask_threshold;
         }
     }
-    if (!rc)
-        rc = maxpool_bwd_launch(dptr(go), dptr(indices), B * C, H, W, Ho, Wo, kH, kW, dH, dW, dptr(gradInput), mask);
+    if (!rc) {
+        TwinOutput second;
+        if (twin && !twin_output(twin, gradInput, second)) second = TwinOutput();
+        bool wrote = false;
+        rc = maxpool_bwd_launch(dptr(go), dptr(indices), B * C, H, W, Ho, Wo, kH, kW, dH, dW, dptr(gradInput), mask,
+                                second, &wrote);
+        if (wrote_twin) *wrote_twin = !rc && wrote ? 1 : 0;
+    }
     if (in) THGPUTensor_free(in);
     THGPUTensor_free(go);
     return rc;
@@ -548,6 +668,14 @@ int thgpu_SpatialMaxPooling_updateGradInputMasked(THGPUTensor *input, THGPUTenso
                                                   THGPUTensor *gradInput, THGPUTensor *indices, int kW, int kH,
                                                   int dW, int dH, float threshold) {
     return pool_update_grad_input(input, gradOutput, gradInput, indices, kW, kH, dW, dH, true, threshold);
+}
+
+int thgpu_SpatialMaxPooling_updateGradInputTwin(THGPUTensor *input, THGPUTensor *gradOutput, THGPUTensor *gradInput,
+                                                THGPUTensor *indices, int kW, int kH, int dW, int dH, int flags,
+                                                float threshold, THGPUTensor *twin, int *wrote_twin) {
+    if (flags & ~THGPU_FUSE_INPUT_MASK) return fail("SpatialMaxPooling: unknown flags");
+    return pool_update_grad_input(input, gradOutput, gradInput, indices, kW, kH, dW, dH,
+                                  (flags & THGPU_FUSE_INPUT_MASK) != 0, threshold, twin, wrote_twin);
 }
 
 int thgpu_Threshold_updateOutput(THGPUTensor *input, THGPUTensor *output, float threshold, float val) {

@@ -23,6 +23,7 @@
 // be applied on the way (InputMask).
 #include "common.h"
 #include "kernels.h"
+#include "side_jobs.h"
 
 #include <cmath>
 
@@ -457,7 +458,14 @@ __global__ __launch_bounds__(256) void maxpool_bwd_cell_kernel(const float *__re
                                                                const float *__restrict__ indx,
                                                                float *__restrict__ gin, const PoolGeom g,
                                                                const FastDiv divXc, const FastDiv divCells, int Xc,
-                                                               unsigned total_cells, const InputMask mask) {
+                                                               unsigned total_cells, const InputMask mask,
+                                                               const TwinOutput twin, const unsigned cell_blocks,
+                                                               const WeightJob side) {
+    // workgroups behind the cells' carry a job of the next layer's (side_jobs.h)
+    if (blockIdx.x >= cell_blocks) {
+        reorder_weight(side, (blockIdx.x - cell_blocks) * 256u + threadIdx.x);
+        return;
+    }
     constexpr int TH = (KH + DH - 1) / DH, TW = (KW + DW - 1) / DW;
     const unsigned cell = blockIdx.x * blockDim.x + threadIdx.x;
     if (cell >= total_cells) return;
@@ -531,15 +539,21 @@ __global__ __launch_bounds__(256) void maxpool_bwd_cell_kernel(const float *__re
 #pragma unroll
         for (int pw = 0; pw < DW; ++pw)
             if (mask.in) acc[ph][pw] = mv[ph][pw] > mask.threshold ? acc[ph][pw] : 0.0f;
+        // the second copy (TwinOutput): the same row inside another buffer
+        float *dst2 = twin.base ? twin.base + (long)plane * twin.plane + (long)(h0 + ph) * twin.pitch + w0 : nullptr;
         if (DW == 2 && w0 + 1 < g.W) {  // one 64-bit store per row: a wavefront writes whole runs of a row
             pool_float2u t;
             t.x = acc[ph][0];
             t.y = acc[ph][DW - 1];
             *reinterpret_cast<pool_float2u *>(dst) = t;
+            if (dst2) *reinterpret_cast<pool_float2u *>(dst2) = t;
         } else {
 #pragma unroll
             for (int pw = 0; pw < DW; ++pw)
-                if (w0 + pw < g.W) dst[pw] = acc[ph][pw];
+                if (w0 + pw < g.W) {
+                    dst[pw] = acc[ph][pw];
+                    if (dst2) dst2[pw] = acc[ph][pw];
+                }
         }
     }
 }
@@ -804,7 +818,8 @@ long pool_plan_selftest() {
 }
 
 int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int H, int W, int Ho, int Wo, int kH,
-                       int kW, int dH, int dW, float *gin, InputMask mask) {
+                       int kW, int dH, int dW, float *gin, InputMask mask, TwinOutput twin, bool *wrote_twin) {
+    if (wrote_twin) *wrote_twin = false;
     hipStream_t s = stream();
     if (!s) return 1;
     PoolGeom g;
@@ -821,7 +836,7 @@ int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int
     g.divDH = FastDiv((uint32_t)dH);
     g.divDW = FastDiv((uint32_t)dW);
     const int th = (kH + dH - 1) / dH, tw = (kW + dW - 1) / dW;
-    const double bytes = 4.0 * ((mask.in ? 2.0 : 1.0) * (double)total + 3.0 * ototal);
+    double bytes = 4.0 * ((mask.in ? 2.0 : 1.0) * (double)total + 3.0 * ototal);
     // The cell kernel takes the window shapes it is compiled for; the pool_bwd_tile and pool_bwd_direct switches force
     // the LDS tile kernel and the direct kernel (testing and tuning aids).
     const bool cell_shape = (kH == 3 && kW == 3 && dH == 2 && dW == 2) || (kH == 2 && kW == 2 && dH == 2 && dW == 2);
@@ -829,13 +844,25 @@ int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int
         const long Yc = (H + dH - 1) / dH, Xc = (W + dW - 1) / dW;
         const long cells = planes * Yc * Xc;
         if (cells < (1L << 31)) {
+            WeightJob side = {};
+            unsigned side_blocks = 0;
+            if (twin.base) {  // only this kernel keeps a second copy; it is part of the launch's traffic
+                bytes += 4.0 * (double)total;
+                if (wrote_twin) *wrote_twin = true;
+                // ... and whoever reads that copy next may have a kernel bank to re-order: this launch carries it
+                if (take_bank_job(side)) {
+                    side_blocks = (side.count + 255u) / 256u;
+                    bytes += 4.0 * (side.count + (double)side.M * side.C * side.kH * side.kW);
+                }
+            }
             {
                 LaunchScope scope(pool_label("maxpool_bwd", g, planes), 0.0, bytes);
-                const dim3 grid((unsigned)((cells + 255) / 256)), block(256);
+                const unsigned cell_blocks = (unsigned)((cells + 255) / 256);
+                const dim3 grid(cell_blocks + side_blocks), block(256);
                 const FastDiv divXc((uint32_t)Xc), divCells((uint32_t)(Yc * Xc));
 #define THGPU_POOL_BWD_CELL(KH_, KW_, DH_, DW_)                                                                     \
     hipLaunchKernelGGL((maxpool_bwd_cell_kernel<KH_, KW_, DH_, DW_>), grid, block, 0, s, gout, indices,             \
-                       indices + ototal, gin, g, divXc, divCells, (int)Xc, (unsigned)cells, mask)
+                       indices + ototal, gin, g, divXc, divCells, (int)Xc, (unsigned)cells, mask, twin, cell_blocks, side)
                 if (kH == 3) THGPU_POOL_BWD_CELL(3, 3, 2, 2);
                 else THGPU_POOL_BWD_CELL(2, 2, 2, 2);
 #undef THGPU_POOL_BWD_CELL

@@ -3,6 +3,7 @@
 // THCStorageCopy.cpp; the device buffer replaces the array_view that the
 // reference kept in allocatorContext.
 #include "common.h"
+#include "kernels.h"
 
 #include <cstdlib>
 #include <cstring>
@@ -139,6 +140,7 @@ hipError_t acquire_block(long floats, float **out) {
 
 void release_block(float *p, long floats) {
     if (!p) return;
+    thgpu::conv_forget_buffer(p);  // whatever was known about its contents ends with this owner
     const size_t bytes = sizeof(float) * (size_t)floats;
     if (floats <= 0 || g_cached_bytes + bytes > kCacheLimit) {
         hipStream_t s = thgpu::stream();

@@ -18,6 +18,7 @@ with host tensors (numpy float32, like torch.Tensor) and moved with :gpu();
 only torch.GPUTensor inputs are computed -- there is no CPU implementation in
 this package.
 """
+import ctypes
 import math
 
 import numpy as np
@@ -165,10 +166,27 @@ class Sequential(Module):
         return cur
 
     def updateGradInput(self, input, gradOutput):
+        # mcw_nn/Sequential.lua:45-57.  After fuse(), a module whose gradInput is the gradOutput of a convolution in
+        # front of it (_grad_consumer) also stores it in the padded layout that convolution's gradInput product
+        # gathers from, and the convolution is told so -- only here, where nothing can touch either copy in between;
+        # a module called on its own always takes the ordinary route.
         cur = gradOutput
-        for i in range(len(self.modules) - 1, 0, -1):
-            cur = self.modules[i].updateGradInput(self.modules[i - 1].output, cur)
-        cur = self.modules[0].updateGradInput(input, cur)
+        ready_for = None                 # the convolution whose fgradInput already holds `cur` in padded form
+        for i in range(len(self.modules) - 1, -1, -1):
+            m = self.modules[i]
+            inp = self.modules[i - 1].output if i > 0 else input
+            link = getattr(m, "_grad_consumer", None)
+            twin = None
+            if link is not None:
+                consumer, ci = link
+                twin = consumer._gradOutputTwin(self.modules[ci - 1].output if ci > 0 else input)
+            if twin is not None or (ready_for is m and ready_for is not None):
+                cur = m._updateGradInputTwin(inp, cur, twin, ready_for is m)
+                ready_for = link[0] if (twin is not None and m._wrote_twin) else None
+            else:
+                cur = m.updateGradInput(inp, cur)
+                if not (isinstance(m, Threshold) and m.fusedBackward):   # that one hands its gradOutput on untouched
+                    ready_for = None
         self.gradInput = cur
         return cur
 
@@ -245,6 +263,17 @@ class Sequential(Module):
                 j += 1
             if j < len(mods) and isinstance(mods[j], SpatialConvolutionMM):
                 m._consumer = mods[j]
+        # Backward: the module whose gradInput reaches a convolution's updateGradInput as gradOutput unchanged
+        # (directly, or through a Threshold whose backward that module applies itself).
+        for i, m in enumerate(mods):
+            if not isinstance(m, SpatialConvolutionMM) or m.gradInput is None:
+                continue
+            j = i + 1
+            if j < len(mods) and isinstance(mods[j], Threshold) and mods[j].fusedBackward:
+                j += 1
+            if j < len(mods) and j > i and isinstance(mods[j], (SpatialConvolutionMM, SpatialMaxPooling)) and (
+                    j == i + 1 or mods[j].inputThreshold is not None):
+                mods[j]._grad_consumer = (m, i)
         return self
 
     def unfuse(self):
@@ -261,6 +290,7 @@ class Sequential(Module):
                 m.inputThreshold = None
             if isinstance(m, (SpatialConvolutionMM, SpatialMaxPooling)):
                 m._consumer = None
+                m._grad_consumer = None
                 if getattr(m.output, "_zero_border", None) is not None:
                     m.output = type(m.output)()
         return self
@@ -415,6 +445,36 @@ class SpatialConvolutionMM(Module):
             *self._geom()))
         return self.gradInput
 
+    def _gradOutputTwin(self, input):
+        """The view through which the producer of this layer's gradOutput can store it in the padded layout at the
+        head of fgradInput (thgpu_SpatialConvolutionMM_gradOutputTwin), or None when this layer's gradInput does not
+        take the gathered route."""
+        if self.gradInput is None or not all(isinstance(t, GPUTensor) for t in (input, self.weight, self.fgradInput)):
+            return None
+        twin = getattr(self, "_twin_view", None)
+        if twin is None:
+            twin = self._twin_view = GPUTensor()
+        available = ctypes.c_int(0)
+        _lib.check_status(lib.thgpu_SpatialConvolutionMM_gradOutputTwin(
+            input._p, self.weight._p, self.fgradInput._p, twin._p, *(self._geom() + (ctypes.byref(available),))))
+        return twin if available.value else None
+
+    def _updateGradInputTwin(self, input, gradOutput, twin, ready):
+        """updateGradInput inside a fused Sequential: `twin` (or None) receives a second copy of gradInput, `ready`
+        says that gradOutput already lies in this layer's fgradInput (see Sequential.updateGradInput)."""
+        self._wrote_twin = False
+        if self.gradInput is None:
+            return None
+        _require_gpu(input, gradOutput, self.weight, self.finput, self.fgradInput, self.gradInput)
+        flags = (1 if self.inputThreshold is not None else 0) | (8 if ready else 0)
+        wrote = ctypes.c_int(0)
+        _lib.check_status(lib.thgpu_SpatialConvolutionMM_updateGradInputTwin(
+            input._p, gradOutput._p, self.weight._p, self.finput._p, self.fgradInput._p, self.gradInput._p,
+            *(self._geom() + (flags, float(self.inputThreshold or 0.0), twin._p if twin is not None else None,
+                              ctypes.byref(wrote)))))
+        self._wrote_twin = bool(wrote.value)
+        return self.gradInput
+
     def accGradParameters(self, input, gradOutput, scale=1):
         _require_gpu(input, gradOutput, self.gradWeight, self.gradBias, self.finput, self.fgradInput)
         if _in_padded_buffer(input, self.padH, self.padW):
@@ -529,6 +589,18 @@ class SpatialMaxPooling(Module):
             return self.gradInput
         _lib.check_status(lib.thgpu_SpatialMaxPooling_updateGradInput(
             input._p, gradOutput._p, self.gradInput._p, self.indices._p, self.kW, self.kH, self.dW, self.dH))
+        return self.gradInput
+
+
+    def _updateGradInputTwin(self, input, gradOutput, twin, ready):
+        """updateGradInput that also stores gradInput through `twin` (see Sequential.updateGradInput)."""
+        _require_gpu(input, gradOutput, self.gradInput, self.indices)
+        wrote = ctypes.c_int(0)
+        _lib.check_status(lib.thgpu_SpatialMaxPooling_updateGradInputTwin(
+            input._p, gradOutput._p, self.gradInput._p, self.indices._p, self.kW, self.kH, self.dW, self.dH,
+            1 if self.inputThreshold is not None else 0, float(self.inputThreshold or 0.0),
+            twin._p if twin is not None else None, ctypes.byref(wrote)))
+        self._wrote_twin = bool(wrote.value)
         return self.gradInput
 
 

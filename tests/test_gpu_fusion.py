@@ -218,3 +218,125 @@ def test_padded_buffer_claims_are_checked_and_a_column_route_producer_can_feed_a
             assert np.array_equal(bits(gw_u), bits(gw_f)) and np.array_equal(bits(gb_u), bits(gb_f))
     finally:
         assert lib.thgpu_conv_set_mode(before) == 0
+
+
+# ---- gradients delivered in the padded layout of the next gathered gradInput product ("twin") ----------------------
+def kernel_labels(gt, fn):
+    """Runs fn with per-kernel timing on; returns {label: launches}."""
+    gp = gt.gputorch
+    gp.synchronize()
+    gp.prof_reset()
+    gp.prof_enable(True)
+    try:
+        fn()
+        gp.synchronize()
+        return {k: v["calls"] for k, v in gp.prof_report().items()}
+    finally:
+        gp.prof_enable(False)
+        gp.prof_reset()
+
+
+TWIN_SPEC = [("conv", 3, 64, 5, 2, 2), ("relu",), ("pool", 3, 2), ("conv", 64, 128, 3, 1, 1), ("relu",),
+             ("conv", 128, 64, 3, 1, 1), ("relu",), ("pool", 2, 2), ("conv", 64, 64, 5, 1, 2), ("relu",), ("pool", 3, 2)]
+
+
+@pytest.mark.parametrize("forced", [{}, {"gemm_split": "3"}, {"gemm_split": "1"}, {"pool_bwd_tile": "1"}],
+                         ids=["auto", "split", "unsplit", "pool_tile"])
+def test_gradients_written_into_the_next_products_padded_buffer(gt, forced, switches):
+    """In a fused Sequential on the gathered route every producer of a convolution's gradOutput (max-pooling backward,
+    a unit-stride convolution's gradInput product through its epilogue or its split reduction) also stores it in that
+    convolution's zero-bordered buffer: results stay bit-identical to the unfused stack, and the padding launches of
+    those layers disappear from the backward pass.  A producer whose kernel keeps no second copy (the LDS tile pooling
+    kernel) leaves the padded copy to be made as before."""
+    for k, v in forced.items():
+        switches(k, v)
+    lib = gt._lib.lib
+    before = lib.thgpu_conv_get_mode()
+    assert lib.thgpu_conv_set_mode(2) == 0
+    try:
+        x = uniform(rng_for(190), (4, 3, 61, 57))
+        net_u, out_u, gi_u, outs_u, grads_u, go = run(gt, TWIN_SPEC, x, 191, False)
+        net_f = build(gt, TWIN_SPEC, 191).gpu().fuse()
+        dx, dgo = dev(gt, x), dev(gt, go)
+        for step in range(3):                         # the buffers and their zero borders are reused step after step
+            net_f.zeroGradParameters()
+            out_f = net_f.forward(dx).float()
+            labels = kernel_labels(gt, lambda: net_f.backward(dx, dgo))
+            gi_f = net_f.gradInput.float()
+            assert np.array_equal(bits(out_u), bits(out_f)) and np.array_equal(bits(gi_u), bits(gi_f)), step
+            grads_f = [(m.gradWeight.float(), m.gradBias.float()) for m in net_f.modules if hasattr(m, "gradWeight")]
+            for (gw_u, gb_u), (gw_f, gb_f) in zip(grads_u, grads_f):
+                assert np.array_equal(bits(gw_u), bits(gw_f)) and np.array_equal(bits(gb_u), bits(gb_f)), step
+            pads = sum(n for k, n in labels.items() if k.startswith("pad_planes"))
+            reorders = labels.get("kernel_bank_reorder", 0)
+            # backward of four convolutions: their gradOutput arrives from the last pooling layer (conv4), the second
+            # (conv3), conv3's gradInput product (conv2: through its epilogue or split reduction) and the first
+            # pooling layer (conv1: the strided layer's own layout)
+            # The kernel bank of the receiving layer is re-ordered by workgroups that ride in the delivering launch
+            # (pooling kernel, split reduction); only an unsplit product, which delivers from its own epilogue, leaves
+            # that to a small launch of the receiver's.
+            split3 = any("gemm_conv_gradinput M=128" in k and "split=1" not in k for k in labels)
+            if "pool_bwd_tile" in forced:
+                assert pads == 3 + 1 and reorders == (0 if split3 else 1), labels   # only conv3's product delivers
+            else:
+                assert pads == 1 and reorders == (0 if split3 else 1), labels   # left: conv1's accGradParameters input
+            if "gemm_split" in forced:
+                assert split3 == (forced["gemm_split"] != "1"), labels
+        # a module called on its own takes the ordinary route and gives the same result
+        conv3 = net_f.get(5)
+        labels = kernel_labels(gt, lambda: conv3.updateGradInput(net_f.get(4).output, net_f.get(7).gradInput))
+        assert any(k.startswith("pad_planes") for k in labels), labels
+        ref3 = net_u.get(4).gradInput.float()          # (the fused layer's gradInput carries the ReLU's mask)
+        assert np.array_equal(bits(conv3.gradInput.float()), bits(ref3))
+        # and the fused pass still works afterwards (the padded copy just made keeps the borders zero)
+        net_f.zeroGradParameters()
+        net_f.forward(dx)
+        assert np.array_equal(bits(net_f.backward(dx, dgo).float()), bits(gi_u))
+        # another batch size: new buffers, new borders
+        x2 = uniform(rng_for(192), (2, 3, 61, 57))
+        net_u2, out_u2, gi_u2, _, grads_u2, go2 = run(gt, TWIN_SPEC, x2, 191, False)
+        net_f.zeroGradParameters()
+        assert np.array_equal(bits(net_f.forward(dev(gt, x2)).float()), bits(out_u2))
+        assert np.array_equal(bits(net_f.backward(dev(gt, x2), dev(gt, go2)).float()), bits(gi_u2))
+        # unfuse(): no deliveries any more
+        net_f.unfuse()
+        net_f.zeroGradParameters()
+        net_f.forward(dx)
+        labels = kernel_labels(gt, lambda: net_f.backward(dx, dgo))
+        assert labels.get("kernel_bank_reorder", 0) == 0 and np.array_equal(bits(net_f.gradInput.float()), bits(gi_u))
+    finally:
+        assert lib.thgpu_conv_set_mode(before) == 0
+
+
+def test_twin_view_is_refused_when_the_buffer_is_not_the_prepared_one(gt):
+    """THGPU_GRADOUTPUT_IN_TWIN is only honoured for the buffer thgpu_SpatialConvolutionMM_gradOutputTwin prepared:
+    handed a layer whose fgradInput was never prepared (or has been resized since), the entry point makes the padded copy
+    itself and the result is right."""
+    import ctypes
+    lib = gt._lib.lib
+    before = lib.thgpu_conv_get_mode()
+    assert lib.thgpu_conv_set_mode(2) == 0
+    try:
+        rng = rng_for(195)
+        conv = gt.nn.SpatialConvolutionMM(64, 64, 3, 3, 1, 1, 1, rng=rng).gpu()
+        x, go = uniform(rng, (2, 64, 12, 10)), uniform(rng, (2, 64, 12, 10))
+        dx, dgo = dev(gt, x), dev(gt, go)
+        conv.forward(dx)
+        ref = conv.updateGradInput(dx, dgo).float().copy()
+        fresh = gt.nn.SpatialConvolutionMM(64, 64, 3, 3, 1, 1, 1, rng=rng).gpu()
+        fresh.weight.copy(conv.weight)
+        fresh.forward(dx)
+        wrote = ctypes.c_int(7)
+        labels = kernel_labels(gt, lambda: gt._lib.check_status(lib.thgpu_SpatialConvolutionMM_updateGradInputTwin(
+            dx._p, dgo._p, fresh.weight._p, fresh.finput._p, fresh.fgradInput._p, fresh.gradInput._p,
+            3, 3, 1, 1, 1, 1, 8, 0.0, None, ctypes.byref(wrote))))
+        assert wrote.value == 0 and any(k.startswith("pad_planes") for k in labels), labels
+        assert np.array_equal(bits(fresh.gradInput.float()), bits(ref))
+        # the view: sizes of gradOutput, rows inside planes of (H + 2) x (W + 2), borders zero after preparation
+        twin = fresh._gradOutputTwin(dx)
+        assert twin is not None and tuple(twin.size()) == (2, 64, 12, 10) and tuple(twin.stride()) == (64 * 14 * 12, 14 * 12, 12, 1)
+        # on the column route no view is handed out
+        assert lib.thgpu_conv_set_mode(0) == 0
+        assert fresh._gradOutputTwin(dx) is None
+    finally:
+        assert lib.thgpu_conv_set_mode(before) == 0
