@@ -63,8 +63,40 @@ local function link(producer, consumer)
    consumer.linkedProducer = producer
 end
 
+-- Backward inside a fused container: the module whose gradInput is a convolution's gradOutput (gradConsumer) also
+-- stores it in the padded layout that convolution's gradInput product gathers from, through the view
+-- SpatialConvolutionMM_gradOutputTwin hands out, and the convolution is told so -- only here, where nothing can touch
+-- either copy in between.  The loop is nn.Sequential:updateGradInput's (mcw_nn/Sequential.lua:45-57).
+local function fused_updateGradInput(self, input, gradOutput)
+   local mods = self.modules
+   local current = gradOutput
+   local ready_for = nil              -- the convolution whose fgradInput already holds `current` in padded form
+   for i = #mods, 1, -1 do
+      local m = mods[i]
+      local m_input = i > 1 and mods[i - 1].output or input
+      local consumer = m.gradConsumer and mods[m.gradConsumer]
+      local twin = nil
+      if consumer then
+         local c_input = m.gradConsumer > 1 and mods[m.gradConsumer - 1].output or input
+         consumer.gradOutputTwin = consumer.gradOutputTwin or c_input.new()
+         twin = c_input.nn.SpatialConvolutionMM_gradOutputTwin(consumer, c_input)
+      end
+      m.twinTarget = twin
+      m.gradOutputInTwin = (ready_for == m) or nil
+      m.wroteTwin = nil
+      current = m:updateGradInput(m_input, current)
+      local passes_on = threshold(m) and m.fusedBackward
+      if twin and m.wroteTwin then ready_for = consumer elseif not passes_on then ready_for = nil end
+      m.twinTarget, m.gradOutputInTwin = nil, nil
+   end
+   self.gradInput = current
+   return current
+end
+
 function gpunn.unfuse(net)
+   net.updateGradInput = nil           -- back to the class method
    for _, m in ipairs(net.modules) do
+      m.gradConsumer, m.twinTarget, m.gradOutputInTwin, m.wroteTwin = nil, nil, nil, nil
       if m.modules then gpunn.unfuse(m) end
       if m.linkedConsumer then
          m.linkedConsumer, m.updateOutput = nil, nil
@@ -110,5 +142,20 @@ function gpunn.fuse(net)
          if mods[j] and isa(mods[j], 'nn.SpatialConvolutionMM') then link(m, mods[j]) end
       end
    end
+   -- backward: the module whose gradInput reaches a convolution's updateGradInput unchanged
+   local any = false
+   for i, m in ipairs(mods) do
+      if isa(m, 'nn.SpatialConvolutionMM') and m.gradInput then
+         local j = i + 1
+         if mods[j] and threshold(mods[j]) and mods[j].fusedBackward then j = j + 1 end
+         local p = mods[j]
+         if p and (isa(p, 'nn.SpatialConvolutionMM') or isa(p, 'nn.SpatialMaxPooling'))
+            and (j == i + 1 or p.inputThreshold ~= nil) then
+            p.gradConsumer = i
+            any = true
+         end
+      end
+   end
+   if any then net.updateGradInput = fused_updateGradInput end
    return net
 end

@@ -17,6 +17,10 @@
 //                     is zeroed where the input is not above it
 //   inputInPaddedBuffer   set by gpunn.fuse(net) while the layer's input is a view into a zero-bordered buffer that
 //                     the layer in front writes (lua/fuse.lua): the gathered convolution reads it there
+//   twinTarget, gradOutputInTwin   set by the fused container's updateGradInput (lua/fuse.lua) for one call: a view to
+//                     store a second copy of gradInput through, and the statement that gradOutput already lies in this
+//                     layer's fgradInput; the call leaves wroteTwin (boolean) behind
+//   gradOutputTwin    a torch.GPUTensor the module keeps for SpatialConvolutionMM_gradOutputTwin to turn into that view
 extern "C" {
 #include <lua.h>
 #include <lauxlib.h>
@@ -32,6 +36,23 @@ int fail(lua_State *L, int rc) { return rc ? luaL_error(L, "%s", thgpu_last_erro
 
 THGPUTensor *field(lua_State *L, const char *name) {
     return static_cast<THGPUTensor *>(luaT_getfieldcheckudata(L, 1, name, kTensor));
+}
+// An optional tensor field: NULL when absent (or false).
+THGPUTensor *opt_field(lua_State *L, const char *name) {
+    lua_getfield(L, 1, name);
+    THGPUTensor *t = lua_toboolean(L, -1) ? static_cast<THGPUTensor *>(luaT_toudata(L, -1, kTensor)) : NULL;
+    lua_pop(L, 1);
+    return t;
+}
+bool flag_field(lua_State *L, const char *name) {
+    lua_getfield(L, 1, name);
+    const bool on = lua_toboolean(L, -1) != 0;
+    lua_pop(L, 1);
+    return on;
+}
+void set_flag_field(lua_State *L, const char *name, bool value) {
+    lua_pushboolean(L, value ? 1 : 0);
+    lua_setfield(L, 1, name);
 }
 THGPUTensor *arg(lua_State *L, int idx) { return static_cast<THGPUTensor *>(luaT_checkudata(L, idx, kTensor)); }
 
@@ -110,8 +131,19 @@ int conv_updateGradInput(lua_State *L) {
     THGPUTensor *finput = field(L, "finput");
     THGPUTensor *fgradInput = field(L, "fgradInput");
     THGPUTensor *gradInput = field(L, "gradInput");
+    THGPUTensor *twin = opt_field(L, "twinTarget");
+    const bool delivered = flag_field(L, "gradOutputInTwin");
     int rc;
-    if (has_field(L, "inputThreshold")) {
+    if (twin || delivered) {
+        const int flags = (has_field(L, "inputThreshold") ? THGPU_FUSE_INPUT_MASK : 0) |
+                          (delivered ? THGPU_GRADOUTPUT_IN_TWIN : 0);
+        const float threshold = static_cast<float>(opt_number(L, "inputThreshold", 0));
+        int wrote = 0;
+        rc = thgpu_SpatialConvolutionMM_updateGradInputTwin(input, gradOutput, weight, finput, fgradInput, gradInput,
+                                                            f.kW, f.kH, f.dW, f.dH, f.padW, f.padH, flags, threshold,
+                                                            twin, &wrote);
+        set_flag_field(L, "wroteTwin", wrote != 0);
+    } else if (has_field(L, "inputThreshold")) {
         const float threshold = static_cast<float>(opt_number(L, "inputThreshold", 0));
         rc = thgpu_SpatialConvolutionMM_updateGradInputFused(input, gradOutput, weight, finput, fgradInput, gradInput,
                                                              f.kW, f.kH, f.dW, f.dH, f.padW, f.padH,
@@ -122,6 +154,24 @@ int conv_updateGradInput(lua_State *L) {
     }
     fail(L, rc);
     return returning(L, "gradInput");
+}
+// input.nn.SpatialConvolutionMM_gradOutputTwin(self, input): the view through which the producer of this layer's
+// gradOutput may store it in padded form (self.gradOutputTwin, returned), or nil when the layer's gradInput does not
+// take the gathered route.
+int conv_gradOutputTwin(lua_State *L) {
+    THGPUTensor *input = arg(L, 2);
+    const ConvFields f = conv_fields(L);
+    THGPUTensor *weight = field(L, "weight");
+    THGPUTensor *fgradInput = field(L, "fgradInput");
+    THGPUTensor *twin = field(L, "gradOutputTwin");
+    int available = 0;
+    fail(L, thgpu_SpatialConvolutionMM_gradOutputTwin(input, weight, fgradInput, twin, f.kW, f.kH, f.dW, f.dH, f.padW,
+                                                      f.padH, &available));
+    if (!available) {
+        lua_pushnil(L);
+        return 1;
+    }
+    return returning(L, "gradOutputTwin");
 }
 int conv_accGradParameters(lua_State *L) {
     THGPUTensor *input = arg(L, 2);
@@ -154,8 +204,16 @@ int pool_updateGradInput(lua_State *L) {
     const PoolFields f = pool_fields(L);
     THGPUTensor *gradInput = field(L, "gradInput");
     THGPUTensor *indices = field(L, "indices");
+    THGPUTensor *twin = opt_field(L, "twinTarget");
     int rc;
-    if (has_field(L, "inputThreshold")) {
+    if (twin) {
+        const float threshold = static_cast<float>(opt_number(L, "inputThreshold", 0));
+        int wrote = 0;
+        rc = thgpu_SpatialMaxPooling_updateGradInputTwin(input, gradOutput, gradInput, indices, f.kW, f.kH, f.dW, f.dH,
+                                                         has_field(L, "inputThreshold") ? THGPU_FUSE_INPUT_MASK : 0,
+                                                         threshold, twin, &wrote);
+        set_flag_field(L, "wroteTwin", wrote != 0);
+    } else if (has_field(L, "inputThreshold")) {
         const float threshold = static_cast<float>(opt_number(L, "inputThreshold", 0));
         rc = thgpu_SpatialMaxPooling_updateGradInputMasked(input, gradOutput, gradInput, indices, f.kW, f.kH, f.dW, f.dH,
                                                            threshold);
@@ -265,6 +323,7 @@ const struct luaL_Reg kOps[] = {
     {"SpatialConvolutionMM_updateOutput", conv_updateOutput},
     {"SpatialConvolutionMM_updateGradInput", conv_updateGradInput},
     {"SpatialConvolutionMM_accGradParameters", conv_accGradParameters},
+    {"SpatialConvolutionMM_gradOutputTwin", conv_gradOutputTwin},
     {"SpatialMaxPooling_updateOutput", pool_updateOutput},
     {"SpatialMaxPooling_updateGradInput", pool_updateGradInput},
     {"Threshold_updateOutput", thr_updateOutput},

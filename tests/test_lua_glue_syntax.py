@@ -93,7 +93,7 @@ def test_glue_registers_both_entry_points_and_every_operator_name():
     # operators return a named field pushed explicitly, never "whatever is on top of the stack"
     bodies = re.findall(r"\nint (\w+)\(lua_State \*L\) \{(.*?)\n\}", nn_glue, flags=re.S)
     ops = [(n, b) for n, b in bodies if re.match(r"(conv|pool|thr|avg|sub|lsm|nll)_", n)]
-    assert len(ops) == 16
+    assert len(ops) == 17
     for name, body in ops:
         last = body.strip().splitlines()[-1].strip()
         assert last == "return 0;" or last.startswith('return returning(L, "'), (name, last)
