@@ -112,3 +112,58 @@ def check_layers(gt, name, net, layers, B, x, go, outs, gins, grads, mode):
                 _, ind_ref = oracle.maxpool_updateOutput(ins[i], l[2], l[1], l[4], l[3])
                 assert np.array_equal(bits(m.indices.float()), bits(ind_ref)), (name, i)
         del dx, dgo, out, gi
+
+
+def test_full_size_alexnet_fused_layerwise(gt):
+    """The benchmark's configuration -- the AlexNet-style stack at batch 128 after Sequential.fuse(), route chosen per
+    layer -- against the oracle, layer by layer on the oracle's inputs: a convolution's output is compared after the
+    ReLU it applies itself, a layer behind a ReLU returns the gradient already masked with it.  (Modules called one by
+    one take dense tensors; the padded buffers and delivered gradients that the container adds when it runs the whole
+    stack are held to bit-identity with the unfused stack at the same size in tests/test_gpu_fusion.py.)"""
+    stacks = gt.stacks
+    name = "alexnet"
+    cfg = stacks.STACKS[name]
+    B, layers = cfg["batch"], cfg["layers"]
+    x, go, outs, gins, grads = oracle_run(stacks, name)
+    lib = gt._lib.lib
+    before = lib.thgpu_conv_get_mode()
+    assert lib.thgpu_conv_set_mode(1) == 0
+    try:
+        net = stacks.build(name, seed_base=4000).gpu().fuse()
+        ins = [x] + outs[:-1]
+        gouts = gins[1:] + [go]
+        n = len(layers)
+        for i, (l, m) in enumerate(zip(layers, net.modules)):
+            if l[0] == "relu":
+                assert m.fusedForward and (m.fusedBackward or i == n - 1 or layers[i + 1][0] == "relu"), i
+                continue
+            print("alexnet fused layer %d %s" % (i, l), flush=True)
+            relu_behind = i + 1 < n and layers[i + 1][0] == "relu" and l[0] == "conv"
+            relu_front = i > 0 and layers[i - 1][0] == "relu"
+            dx = dev(gt, ins[i])
+            # the gradient that reaches this module is the same as in the unfused stack: where a ReLU follows, its
+            # backward has been applied by the module behind it
+            dgo = dev(gt, gouts[i])
+            want_out = outs[i + 1] if relu_behind else outs[i]
+            want_gi = gins[i - 1] if relu_front else gins[i]   # masked with the ReLU in front
+            m.zeroGradParameters()
+            out = m.forward(dx).float()
+            gi = m.backward(dx, dgo).float()
+            if l[0] == "conv":
+                assert (m.fusedThreshold is not None) == relu_behind and (m.inputThreshold is not None) == relu_front, i
+                _, cin, cout, kW, kH, dW, dH, pW, pH = l
+                K, N = cin * kH * kW, outs[i].shape[2] * outs[i].shape[3]
+                tag = "alexnet b%d fused layer%d " % (B, i)
+                check_close(tag + "output", out, want_out, K)
+                assert np.array_equal(out == 0, want_out == 0) or not relu_behind or \
+                    np.mean((out == 0) != (want_out == 0)) < 1e-4          # the threshold bites in the same places
+                check_close(tag + "gradInput", gi, want_gi, cout * kH * kW)
+                check_close(tag + "gradWeight", m.gradWeight.float(), grads[i][0], B * N)
+                check_close(tag + "gradBias", m.gradBias.float(), grads[i][1], B * N)
+            else:
+                assert (m.inputThreshold is not None) == relu_front, i
+                assert np.array_equal(bits(out), bits(want_out)), i
+                assert np.array_equal(bits(gi), bits(want_gi)), i
+            del dx, dgo, out, gi
+    finally:
+        assert lib.thgpu_conv_set_mode(before) == 0

@@ -42,6 +42,40 @@ def test_im2col_arange_is_self_describing_and_pads_with_positive_zero():
     assert zeros.size > 0 and not np.any(np.signbit(zeros))
 
 
+@pytest.mark.parametrize("k,pad", [(3, 0), (3, 1), (3, 2), (5, 2), (5, 4), (4, 3), (2, 1), (3, 4), (1, 2)])
+def test_unfold_edges_against_padding_by_hand(k, pad):
+    """The left / right and top / bottom edge handling of the unfold (lpad / rpad in
+    mcw_nn/generic/SpatialConvolutionMM.c:35-37,81-85), pinned independently of any index formula: pad the image by
+    hand with numpy, then column row (c, kh, kw) is the padded plane shifted by (kh, kw) and cut to the output size.
+    Paddings from 0 through k-1 and above (a whole tap row or column outside the image); fold is held to the adjoint
+    identity on the same geometries, with integer data so that every sum is exact."""
+    rng = rng_for(40 + 7 * k + pad)
+    B, C, H, W = 2, 2, 6, 7
+    Ho, Wo = H + 2 * pad - k + 1, W + 2 * pad - k + 1
+    if Ho < 1 or Wo < 1:
+        pytest.skip("kernel larger than the padded image")
+    im = rng.integers(-4, 5, (B, C, H, W)).astype(np.float32)
+    padded = np.pad(im, [(0, 0), (0, 0), (pad, pad), (pad, pad)])
+    col = oracle.im2col(im, k, k, pad, pad, 1, 1)
+    assert col.shape == (B, C * k * k, Ho * Wo)
+    for c in range(C):
+        for kh in range(k):
+            for kw in range(k):
+                want = padded[:, c, kh:kh + Ho, kw:kw + Wo].reshape(B, Ho * Wo)
+                assert np.array_equal(col[:, (c * k + kh) * k + kw], want), (c, kh, kw)
+    assert not np.any(np.signbit(col[col == 0]))          # padding is +0.0f
+    y = rng.integers(-4, 5, col.shape).astype(np.float32)
+    back = oracle.col2im(y, C, H, W, k, k, pad, pad, 1, 1)
+    assert float(np.sum(col.astype(np.float64) * y)) == float(np.sum(im.astype(np.float64) * back))
+    # fold by hand: every column row added back at its shift, cropped to the image
+    acc = np.zeros_like(padded, dtype=np.float64)
+    for c in range(C):
+        for kh in range(k):
+            for kw in range(k):
+                acc[:, c, kh:kh + Ho, kw:kw + Wo] += y[:, (c * k + kh) * k + kw].reshape(B, Ho, Wo)
+    assert np.array_equal(back, acc[:, :, pad:pad + H, pad:pad + W].astype(np.float32))
+
+
 @pytest.mark.parametrize("geo", GEOMS)
 def test_col2im_equals_ordered_bruteforce_bit_exact(geo):
     C, H, W, kH, kW, pH, pW, sH, sW = geo
