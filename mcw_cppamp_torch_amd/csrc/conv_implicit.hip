@@ -93,6 +93,17 @@ __global__ __launch_bounds__(256) void tap_table_kernel(int *__restrict__ t, int
     t[idx] = c * plane + kh * pitch + kw;
 }
 
+// The tap table padded to `count` entries: the entries beyond the taps repeat tap 0 (any valid offset would do: they
+// address the scratch columns of a product run wider than its result, GemmProblem::j_store).
+__global__ __launch_bounds__(256) void tap_table_padded_kernel(int *__restrict__ t, int planes, int kH, int kW, int plane,
+                                                               int pitch, int count) {
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= count) return;
+    const int k = idx < planes * kH * kW ? idx : 0;
+    const int kw = k % kW, kh = (k / kW) % kH, c = k / (kW * kH);
+    t[idx] = c * plane + kh * pitch + kw;
+}
+
 // t[(y, x)] = y*row_step + x*col_step
 __global__ __launch_bounds__(256) void pixel_table_kernel(int *__restrict__ t, int Hn, int Wn, int row_step,
                                                           int col_step) {
@@ -126,6 +137,8 @@ const int *table(int kind, int a, int b, int c, int d, int e, long count) {
     const unsigned blocks = (unsigned)((count + 255) / 256);
     if (kind == 0)
         hipLaunchKernelGGL(tap_table_kernel, dim3(blocks), dim3(256), 0, s, t, a, b, c, d, e);
+    else if (kind == 2)
+        hipLaunchKernelGGL(tap_table_padded_kernel, dim3(blocks), dim3(256), 0, s, t, a, b, c, d, e, (int)count);
     else
         hipLaunchKernelGGL(pixel_table_kernel, dim3(blocks), dim3(256), 0, s, t, a, b, c, d);
     if (check_launch("conv offset table")) {
@@ -152,6 +165,10 @@ int trim_tables() {
 const int *tap_table(int planes, int kH, int kW, int plane, int pitch) {
     return table(0, planes, kH, kW, plane, pitch, (long)planes * kH * kW);
 }
+const int *tap_table_padded(int planes, int kH, int kW, int plane, int pitch, int count) {
+    // (the padded length is a function of the taps, so the key of kind 2 need not hold it)
+    return table(2, planes, kH, kW, plane, pitch, count);
+}
 const int *pixel_table(int Hn, int Wn, int row_step, int col_step) {
     return table(1, Hn, Wn, row_step, col_step, 0, (long)Hn * Wn);
 }
@@ -163,6 +180,7 @@ int g_mode = -1;
 // The three products as GEMM problems, without pointers and tables (those are filled in by the launchers; a
 // problem with `gathered` set is enough for the planner to say whether a tiled kernel takes it).
 const int kNoTable = 0;  // stands in for a table where only the planner looks at the problem
+constexpr int kNarrowestTile = 64;  // columns of the narrowest GEMM tile
 
 GemmProblem forward_problem(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
     const int Hp = H + 2 * pH, Wp = W + 2 * pW;
@@ -201,6 +219,10 @@ GemmProblem gradweight_problem(long B, int C, int H, int W, int M, int kH, int k
     p.M = M;
     p.J = K;
     p.N = K;
+    if (K < kNarrowestTile) {  // fewer taps than the narrowest tile has columns: run it that wide, store K of them
+        p.J = p.N = kNarrowestTile;
+        p.j_store = K;
+    }
     p.R = (int)N;
     p.nb = (int)B;
     p.beta = 1.0f;
@@ -360,11 +382,13 @@ void conv_set_mode(int mode) { g_mode = mode; }
 // Shapes the gathered GEMMs take: the padded batch must stay within 32-bit byte offsets and a tile of the fast
 // kernel must take both products that share finput (the GEMM's own planner answers that: M, J >= 64, R >= 16,
 // offsets of operands and output below 2^30 floats, a tile the tuning switches allow).
+// Forward and gradWeight share finput (the padded input), so a layer takes both or neither.  K >= 16 is the GEMM's
+// shortest reduction (forward); a gradWeight product with fewer than 64 taps runs 64 columns wide (gradweight_problem).
 static bool forward_fits(long B, int C, int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW) {
     const long Hp = H + 2L * pH, Wp = W + 2L * pW;
     const long Ho = (Hp - kH) / sH + 1, Wo = (Wp - kW) / sW + 1;
     const long K = (long)C * kH * kW, N = Ho * Wo;
-    if (!(M >= 64 && K >= 64 && N >= 16 && B * N >= 64 && B * N < (1L << 31) && B * C * Hp * Wp < kMaxExtent)) return false;
+    if (!(M >= 64 && K >= 16 && N >= 16 && B * N >= 64 && B * N < (1L << 31) && B * C * Hp * Wp < kMaxExtent)) return false;
     return gemm_tiled_fits(forward_problem(B, C, H, W, M, kH, kW, pH, pW, sH, sW)) &&
            gemm_tiled_fits(gradweight_problem(B, C, H, W, M, kH, kW, pH, pW, sH, sW));
 }
@@ -529,7 +553,7 @@ int conv_implicit_gradweight(const float *padded, const float *gradOutput, float
     p.A = gradOutput;
     p.B = padded;
     p.rowtab = pixel_table(Ho, Wo, sH * Wp, sW);
-    p.coltab = tap_table(C, kH, kW, Hp * Wp, Wp);
+    p.coltab = p.j_store > 0 ? tap_table_padded(C, kH, kW, Hp * Wp, Wp, p.J) : tap_table(C, kH, kW, Hp * Wp, Wp);
     if (!p.rowtab || !p.coltab) return 1;
     p.C = gradWeight;
     p.alpha = scale;

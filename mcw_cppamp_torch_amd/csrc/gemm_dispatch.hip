@@ -45,7 +45,8 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(const RowSumJob rs, c
                                                            float mask_threshold, int c_pitch, int mask_pitch,
                                                            long mask_sC, long mask_bsC, FastDiv divCW,
                                                            float *__restrict__ C2, long c2_sC, long c2_bsC, int c2_pitch,
-                                                           const unsigned side_first_block, const WeightJob side) {
+                                                           const unsigned side_first_block, const WeightJob side,
+                                                           const unsigned j_store) {
     // workgroups behind the reduction's carry a job of the next layer's (side_jobs.h)
     if (blockIdx.x >= side_first_block) {
         reorder_weight(side, (blockIdx.x - side_first_block) * 256u + threadIdx.x);
@@ -86,6 +87,7 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(const RowSumJob rs, c
     }
     unsigned i, j;
     divJ.divmod(idx, i, j);
+    if (j >= j_store) return;  // a scratch column of a product run wider than its result (GemmProblem::j_store)
     long coff = j, moff = j, toff = 0;
     if (N != J || c_pitch || mask_pitch || C2) {
         unsigned im, n, y, x;
@@ -215,10 +217,15 @@ GemmPlan plan_gemm(const GemmProblem &p, int steps_total) {
         if (c.a_rc_only && !p.a_rc) continue;
         if (c.rows_used > 0 && !(p.scatter && layout == 4 && p.M == c.bm && p.scat_rows <= c.rows_used)) continue;
         const long tiles = cdiv(p.M, c.bm) * cdiv(p.J, c.bn);
-        int max_split = (int)(steps_total / 8 > 0 ? (steps_total / 8 < 256 ? steps_total / 8 : 256) : 1);
+        // (a product run wider than its result has one narrow tile per row block: it may split further to fill the GPU)
+        const int split_cap = p.j_store > 0 ? 1024 : 256;
+        int max_split = (int)(steps_total / 8 > 0 ? (steps_total / 8 < split_cap ? steps_total / 8 : split_cap) : 1);
         if (p.scatter) max_split = 1;  // the scattered store has no partial-sum form
-        for (int ns = 1; ns <= max_split; ++ns) {
-            if (fsplit > 0 && ns != (fsplit < max_split ? fsplit : max_split)) continue;
+        const int min_split = p.j_store > 0 ? 2 : 1;  // scratch columns never reach C unsplit
+        int want = fsplit > 0 ? (fsplit < max_split ? fsplit : max_split) : 0;
+        if (want > 0 && want < min_split) want = min_split;
+        for (int ns = min_split; ns <= max_split; ++ns) {
+            if (want > 0 && ns != want) continue;
             if (tiles * ns > 8L * cus * c.resident && ns > 1 && fsplit <= 0) break;
             if (ns > 1 && p.ws_fixed && (long)ns * p.M * p.J > p.ws_fixed_floats) break;  // partial sums must fit
             const int sps = (int)cdiv(steps_total, ns);
@@ -292,6 +299,8 @@ int gemm_launch(const GemmProblem &p) {
     g.mask_sC = p.mask_sC ? p.mask_sC : p.sC;
     g.mask_bsC = p.mask_bsC ? p.mask_bsC : p.bsC;
     g.divCW = FastDiv((uint32_t)g.c_w);
+    if (p.j_store > 0 && (!red || p.j_store > p.J || p.sC < p.j_store || p.C2 || p.scatter))
+        return fail("gemm: scratch columns need reduction batching and a row pitch of C that holds the stored ones");
     if (p.C2) {
         if (red || p.scatter || p.c_w <= 0 || g.N % p.c_w != 0 || p.c2_pitch < p.c_w || p.c2_sC <= 0 || p.c2_bsC <= 0)
             return fail("gemm: a second copy of the result needs column batching, a plane width and the copy's strides");
@@ -370,6 +379,8 @@ int gemm_launch(const GemmProblem &p) {
     const int lb = p.b_rc ? LD_RC_VEC : gather ? LD_XC_GATHER : LD_XC_SCALAR;
     if (gather && !best) return fail("gemm: a gathered B needs a shape the tiled kernel takes (M, J >= 64, R >= 16)");
     if (p.C2 && !best) return fail("gemm: a second copy of the result needs a shape the tiled kernel takes");
+    if (p.j_store > 0 && (!best || g.nsplit < 2))
+        return fail("gemm: scratch columns need a tiled kernel and a split reduction");
 
     int rc;
     {
@@ -415,7 +426,7 @@ int gemm_launch(const GemmProblem &p) {
                                p.M, p.J, g.N, p.sC, p.bsC, FastDiv((uint32_t)p.J), g.divN, g.nsplit, p.alpha,
                                p.beta, g.act, g.act_threshold, g.act_value, g.mask, g.mask_threshold, g.c_pitch,
                                g.mask_pitch, g.mask_sC, g.mask_bsC, g.divCW, g.C2, g.c2_sC, g.c2_bsC, g.c2_pitch,
-                               side_first, side);
+                               side_first, side, (unsigned)(p.j_store > 0 ? p.j_store : p.J));
         }
         if (check_launch("gemm_split_reduce")) return 1;
     }

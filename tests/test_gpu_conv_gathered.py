@@ -78,6 +78,12 @@ GATHERED = [
     (16, 3, 224, 224, 64, 11, 11, 2, 2, 4, 4),         # first benchmark configuration, full size
     (2, 48, 12, 12, 64, 3, 3, 1, 1, 1, 1),             # C < 64: forward gathered, gradInput by columns
     (2, 64, 12, 12, 48, 3, 3, 1, 1, 1, 1),             # M < 64: forward by columns, gradInput gathered
+    # fewer than 64 taps: the gradWeight product runs 64 columns wide and stores K of them
+    (4, 3, 40, 36, 64, 3, 3, 1, 1, 1, 1),              # VGG-style first layer, K = 27
+    (3, 1, 33, 35, 128, 5, 5, 2, 2, 1, 1),             # one input plane, K = 25, two row tiles
+    (5, 3, 31, 29, 70, 4, 4, 1, 1, 2, 2),              # K = 48, stride 2, rows ragged against the tile
+    (2, 3, 64, 48, 128, 7, 3, 3, 1, 2, 1),             # K = 63: the non-square edge case with three input planes
+    (2, 2, 30, 30, 64, 3, 3, 0, 0, 1, 1),              # K = 18, unpadded: gathered from the dense input in place
 ]
 
 
@@ -95,9 +101,9 @@ def test_gathered_conv_fwd_bwd_parity(gt, gathered_route, cfg):
     out_ref, go, gi_ref, gw_ref, gb_ref = reference(x, w, b, rng, geo, scale, gw0, gb0)
     got = run_conv(gt, x, w, b, go, geo, scale, gw0, gb0)
     N = out_ref.shape[2] * out_ref.shape[3]
-    if M >= 64 and K >= 64 and (pH, pW) == (0, 0):
+    if M >= 64 and K >= 16 and (pH, pW) == (0, 0):
         assert got["finput"].size <= 1            # an unpadded dense input is gathered from where it lies: no copy
-    elif M >= 64 and K >= 64:
+    elif M >= 64 and K >= 16:
         assert np.array_equal(bits(got["finput"]), bits(padded(x, pH, pW)))   # the padded input, not columns
     else:
         assert got["finput"].shape == (B, K, N)
@@ -520,3 +526,55 @@ def test_strided_gradinput_short_row_kernel_integer_exact(gt, gathered_route, sw
     assert np.array_equal(gi, gi_ref)
     host = big.float()
     assert np.all(host[:guard] == 7.5) and np.all(host[guard + n:] == 7.5)
+
+
+@pytest.mark.parametrize("split", [None, 2, 7])
+@pytest.mark.parametrize("cfg", [(4, 3, 40, 36, 64, 3, 3, 1, 1, 1, 1), (3, 1, 33, 35, 128, 5, 5, 2, 2, 1, 1),
+                                 (5, 3, 31, 29, 70, 4, 4, 1, 1, 2, 2), (2, 3, 64, 48, 128, 7, 3, 3, 1, 2, 1)])
+def test_narrow_gradweight_runs_wide_and_stores_its_own_columns_integer_exact(gt, gathered_route, switches, cfg, split):
+    """A layer with fewer than 64 taps (K = C*kH*kW: a first layer with 3x3 or 5x5 kernels) has a gradWeight product
+    narrower than the narrowest GEMM tile.  It runs 64 columns wide on a padded tap table and the split reduction's
+    final pass stores the first K columns only: on integer data every result equals the oracle's bit for bit, gradBias
+    (summed on the side by the same product) included, and what lies around gradWeight in memory is untouched."""
+    if split is not None:
+        switches("gemm_split", split)
+    B, C, H, W, M, kH, kW, pH, pW, sH, sW = cfg
+    geo = (kH, kW, pH, pW, sH, sW)
+    K = C * kH * kW
+    rng = rng_for(48)
+    ints = lambda shape: rng.integers(-3, 4, shape).astype(np.float32)  # noqa: E731
+    x, w, b = ints((B, C, H, W)), ints((M, K)), ints((M,))
+    gw0, gb0 = ints((M, K)), ints((M,))
+    out_ref, finput_ref = oracle.conv_updateOutput(x, w, b, *geo)
+    go = ints(out_ref.shape)
+    gi_ref, _ = oracle.conv_updateGradInput(go, w, x.shape, *geo)
+    gw_ref, gb_ref = gw0.copy(), gb0.copy()
+    oracle.conv_accGradParameters(go, finput_ref, gw_ref, gb_ref, 2.0)
+    # gradWeight as a window of a larger buffer: guard rows before and behind it
+    m = gt.nn.SpatialConvolutionMM(C, M, kW, kH, sW, sH, 0, padW=pW, padH=pH)
+    m._assign("weight", w)
+    m._assign("bias", b)
+    m.gpu()
+    big = dev(gt, np.full((M + 2, K), 9.0, np.float32))
+    m.gradWeight = big.narrow(0, 1, M)
+    m.gradWeight.copy(gw0)
+    m.gradBias.copy(gb0)
+    dx, dgo = dev(gt, x), dev(gt, go)
+    gt.gputorch.prof_reset()
+    gt.gputorch.prof_enable(True)
+    try:
+        out = m.forward(dx).float()
+        gi = m.updateGradInput(dx, dgo).float()
+        m.accGradParameters(dx, dgo, 2.0)
+        gt.gputorch.synchronize()
+        labels = list(gt.gputorch.prof_report())
+    finally:
+        gt.gputorch.prof_enable(False)
+        gt.gputorch.prof_reset()
+    assert np.array_equal(out, out_ref) and np.array_equal(gi, gi_ref)
+    got = big.float()
+    assert np.array_equal(got[1:-1], gw_ref) and np.all(got[0] == 9.0) and np.all(got[-1] == 9.0)
+    assert np.array_equal(m.gradBias.float(), gb_ref)
+    gw_label = [k for k in labels if k.startswith("gemm_conv_gradweight")]
+    assert len(gw_label) == 1 and "J=64 " in gw_label[0] and "tile=64x64" in gw_label[0] and "split=1 " not in gw_label[0] + " ", labels
+    assert not any(k.startswith(("im2col", "gradbias")) for k in labels), labels      # no columns, no separate bias sum

@@ -201,14 +201,14 @@ def test_padded_buffer_claims_are_checked_and_a_column_route_producer_can_feed_a
     assert lib.thgpu_SpatialConvolutionMM_updateOutputFused(x._p, conv.weight._p, conv.bias._p, conv.finput._p,
                                                             conv.fgradInput._p, conv.output._p, 3, 3, 1, 1, 1, 1, 8, 0.0, 0.0) != 0
     assert lib.thgpu_conv_gathers(2, 64, 9, 9, 64, 3, 3, 1, 1, 1, 1) == (1 if lib.thgpu_conv_get_mode() != 0 else 0)
-    assert lib.thgpu_conv_gathers(2, 3, 9, 9, 64, 3, 3, 1, 1, 1, 1) == 0      # K = 27: no tile
-    # mode 1: a producer whose products no tiled kernel takes (K = 27) stays on columns, its 64-plane consumer gathers
+    assert lib.thgpu_conv_gathers(2, 1, 9, 9, 64, 3, 3, 1, 1, 1, 1) == 0      # K = 9: below the shortest reduction
+    # mode 1: a producer whose products no tiled kernel takes (K = 9) stays on columns, its 64-plane consumer gathers
     # from the producer's padded output
     before = lib.thgpu_conv_get_mode()
     assert lib.thgpu_conv_set_mode(1) == 0
     try:
-        spec = [("conv", 3, 64, 3, 1, 1), ("relu",), ("conv", 64, 64, 3, 1, 1), ("relu",), ("pool", 2, 2)]
-        xx = uniform(rng_for(97), (2, 3, 12, 14))
+        spec = [("conv", 1, 64, 3, 1, 1), ("relu",), ("conv", 64, 64, 3, 1, 1), ("relu",), ("pool", 2, 2)]
+        xx = uniform(rng_for(97), (2, 1, 12, 14))
         net_u, out_u, gi_u, outs_u, grads_u, go = run(gt, spec, xx, 98, False)
         net_f, out_f, gi_f, outs_f, grads_f, _ = run(gt, spec, xx, 98, True, go)
         assert net_f.modules[0].finput.dim() == 3 and net_f.modules[0].output._zero_border == (1, 1)
