@@ -41,10 +41,11 @@ int col2im_launch(const float *col, long B, int C, int H, int W, int kH, int kW,
 // out_plane / out_pitch: floats between the output's planes and rows when it is not densely packed (0: dense).
 int maxpool_fwd_launch(const float *in, long planes, int H, int W, int kH, int kW, int dH, int dW, float *out,
                        float *indices, long out_plane = 0, int out_pitch = 0);
-// *wrote_twin (when twin.base is set) says whether the kernel that ran also stored the second copy.
+// *wrote_twin (when twin.base is set) says whether the kernel that ran also stored the second copy.  twin_gaps: the
+// floats between the rows of the second copy are known to hold zeros and may be stored (as zeros) along with the rows.
 int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int H, int W, int Ho, int Wo, int kH,
                        int kW, int dH, int dW, float *gin, InputMask mask = InputMask(), TwinOutput twin = TwinOutput(),
-                       bool *wrote_twin = nullptr);
+                       bool *wrote_twin = nullptr, bool twin_gaps = false);
 int threshold_fwd_launch(const float *in, float *out, long n, float th, float val);
 int threshold_bwd_launch(const float *in, const float *gout, float *gin, long n, float th);
 int gradbias_launch(const float *gout, float *gbias, long B, int M, long N, float scale);

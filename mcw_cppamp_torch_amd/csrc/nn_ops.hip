@@ -174,6 +174,20 @@ bool twin_output(const THGPUTensor *twin, const THGPUTensor *like, TwinOutput &o
     return true;
 }
 
+// Whether `twin` is the view thgpu_SpatialConvolutionMM_gradOutputTwin hands out into a buffer that is on record as
+// zero-bordered: then the floats between its rows are zeros that a producer may store again along with the rows.
+bool twin_rows_in_zero_border(const THGPUTensor *twin, const TwinOutput &out) {
+    const int o = twin->nDimension == 4 ? 1 : 0;
+    for (const auto &kv : g_zero_bordered) {
+        const TwinGeom &t = kv.second;
+        if (kv.first + (long)t.top * t.Wq + t.left == out.base && t.Wq == out.pitch && (long)t.Hq * t.Wq == out.plane &&
+            twin->size[o] == t.M && twin->size[o + 1] == t.Ho && twin->size[o + 2] == t.Wo &&
+            (o ? twin->size[0] : 1) == t.B)
+            return true;
+    }
+    return false;
+}
+
 int conv_update_output(THGPUTensor *input, THGPUTensor *weight, THGPUTensor *bias, THGPUTensor *finput,
                        THGPUTensor *fgradInput, THGPUTensor *output, int kW, int kH, int dW, int dH, int padW,
                        int padH, OutputThreshold act, bool input_in_padded_buffer) {
@@ -651,7 +665,7 @@ static int pool_update_grad_input(THGPUTensor *input, THGPUTensor *gradOutput, T
         if (twin && !twin_output(twin, gradInput, second)) second = TwinOutput();
         bool wrote = false;
         rc = maxpool_bwd_launch(dptr(go), dptr(indices), B * C, H, W, Ho, Wo, kH, kW, dH, dW, dptr(gradInput), mask,
-                                second, &wrote);
+                                second, &wrote, second.base && twin_rows_in_zero_border(twin, second));
         if (wrote_twin) *wrote_twin = !rc && wrote ? 1 : 0;
     }
     if (in) THGPUTensor_free(in);

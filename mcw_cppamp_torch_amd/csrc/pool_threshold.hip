@@ -558,6 +558,189 @@ __global__ __launch_bounds__(256) void maxpool_bwd_cell_kernel(const float *__re
     }
 }
 
+// The staged kernel: the cell kernel's arithmetic with the tile kernel's memory streams, the default for the window
+// shapes of the benchmark stacks.  Counters showed what holds the cell kernel back: its stores -- 8 bytes per lane,
+// rows of W floats that start anywhere -- reach the L2 as requests of 29 bytes on average, 2.2 times as many as the
+// data needs, and the request rate, not the byte rate, is what saturates.  Here a workgroup owns a contiguous range
+// of pixels (a group of small planes, or a strip of rows of a large one), its lanes compute the range's cells exactly
+// as the cell kernel does (every load requested up front, no zero-fill, no scatter phases), park the results in LDS,
+// and after ONE barrier the range leaves as one contiguous stream of full-width requests, the mask (requested first,
+// as a contiguous stream too) applied on the way.  A second copy (TwinOutput) leaves the same way, row gaps included
+// when they are known to hold zeros, so that it is a contiguous stream as well.
+constexpr int kStagedPixelsPerLane = 16;  // a workgroup stages up to 4096 pixels (16 KB of LDS)
+constexpr int kStagedCellsPerLane = 4;    // ... computed as up to 1024 cells
+
+struct PoolStagedPlan {
+    int G;       // planes per workgroup (more than one only when a strip is the whole plane)
+    int PR;      // pixel rows per strip (a multiple of the row stride unless the strip is the whole plane)
+    int strips;  // strips per plane
+    int Xc;      // cells per cell row
+    FastDiv divStrips, divXc, divPlaneCells, divTwinPitch;
+};
+
+template <int KH, int KW, int DH, int DW>
+__global__ __launch_bounds__(256) void maxpool_bwd_staged_kernel(const float *__restrict__ gout,
+                                                                 const float *__restrict__ indy,
+                                                                 const float *__restrict__ indx,
+                                                                 float *__restrict__ gin, const PoolGeom g,
+                                                                 const PoolStagedPlan p, unsigned planes,
+                                                                 const InputMask mask, const TwinOutput twin,
+                                                                 const bool twin_gaps, const unsigned pool_blocks,
+                                                                 const WeightJob side) {
+    extern __shared__ float px[];  // [np][nh][W]: the range's gradInput
+    if (blockIdx.x >= pool_blocks) {  // workgroups behind the pooling's carry a job of the next layer's (side_jobs.h)
+        reorder_weight(side, (blockIdx.x - pool_blocks) * 256u + threadIdx.x);
+        return;
+    }
+    constexpr int TH = (KH + DH - 1) / DH, TW = (KW + DW - 1) / DW;
+    constexpr int PXL = kStagedPixelsPerLane, CI = kStagedCellsPerLane;
+    const int tid = threadIdx.x;
+    unsigned grp, strip;
+    p.divStrips.divmod(blockIdx.x, grp, strip);
+    const unsigned plane0 = grp * (unsigned)p.G;
+    const int np = (int)(planes - plane0 < (unsigned)p.G ? planes - plane0 : (unsigned)p.G);
+    const int h0 = (int)strip * p.PR;
+    const int nh = g.H - h0 < p.PR ? g.H - h0 : p.PR;
+    const int npix = np * nh * g.W;
+    const long base = (long)plane0 * g.H * g.W + (long)h0 * g.W;  // (h0 = 0 when planes are grouped)
+
+    // ---- the mask of the range: requested first, used last ---------------------------------------------------------
+    float mv[PXL];
+    if (mask.in) {
+        const float *m = mask.in + base;
+#pragma unroll
+        for (int u = 0; u < PXL; ++u) {
+            const int e = tid + u * 256;
+            mv[u] = e < npix ? m[e] : 0.0f;
+        }
+    }
+
+    // ---- the range's cells: all window requests of a lane's cells go out before the first is used -------------------
+    const int yc0 = h0 / DH;                       // strips start on a cell row
+    const int nyc = (nh + DH - 1) / DH;
+    const int per_plane = nyc * p.Xc;
+    const int ncell = np * per_plane;
+    float wg[CI][TH][TW], wy[CI][TH][TW], wx[CI][TH][TW];
+    bool win[CI][TH][TW];
+    int cell_px[CI], cell_hl[CI], cell_w0[CI];  // LDS offset of the cell's first pixel, its row in the range, its column
+#pragma unroll
+    for (int ci = 0; ci < CI; ++ci) {
+        const int c = tid + ci * 256;
+        const bool live = c < ncell;
+        unsigned pl = 0, rem = (unsigned)(live ? c : 0), yl, x;
+        if (p.G > 1) p.divPlaneCells.divmod(rem, pl, rem);  // grouped planes are whole: Yc*Xc cells each
+        p.divXc.divmod(rem, yl, x);
+        const int y = yc0 + (int)yl;
+        cell_hl[ci] = live ? (int)yl * DH : nh;              // (a dead cell owns no row of the range)
+        cell_w0[ci] = (int)x * DW;
+        cell_px[ci] = ((int)pl * nh + (int)yl * DH) * g.W + (int)x * DW;
+        const long obase = (long)(plane0 + pl) * g.Ho * g.Wo;
+#pragma unroll
+        for (int a = 0; a < TH; ++a)
+#pragma unroll
+            for (int b = 0; b < TW; ++b) {
+                const int i = y - a, j = (int)x - b;
+                win[ci][a][b] = live && i >= 0 && i < g.Ho && j >= 0 && j < g.Wo;
+                const int ic = i < 0 ? 0 : i < g.Ho ? i : g.Ho - 1, jc = j < 0 ? 0 : j < g.Wo ? j : g.Wo - 1;
+                const long o = obase + (long)ic * g.Wo + jc;
+                wg[ci][a][b] = gout[o];
+                wy[ci][a][b] = indy[o];
+                wx[ci][a][b] = indx[o];
+            }
+    }
+#pragma unroll
+    for (int ci = 0; ci < CI; ++ci) {
+        float acc[DH][DW];
+#pragma unroll
+        for (int ph = 0; ph < DH; ++ph)
+#pragma unroll
+            for (int pw = 0; pw < DW; ++pw) acc[ph][pw] = 0.0f;
+        // windows in (i, j) ascending order: the float addition order of the CPU module's scatter
+#pragma unroll
+        for (int a = TH - 1; a >= 0; --a)
+#pragma unroll
+            for (int b = TW - 1; b >= 0; --b) {
+                const int ky = win[ci][a][b] ? (int)wy[ci][a][b] - 1 - a * DH : -1, kx = (int)wx[ci][a][b] - 1 - b * DW;
+#pragma unroll
+                for (int ph = 0; ph < DH; ++ph)
+#pragma unroll
+                    for (int pw = 0; pw < DW; ++pw) {
+                        if (ph + a * DH >= KH || pw + b * DW >= KW) continue;
+                        acc[ph][pw] += (ky == ph && kx == pw) ? wg[ci][a][b] : 0.0f;
+                    }
+            }
+#pragma unroll
+        for (int ph = 0; ph < DH; ++ph)
+#pragma unroll
+            for (int pw = 0; pw < DW; ++pw)
+                if (cell_hl[ci] + ph < nh && cell_w0[ci] + pw < g.W) px[cell_px[ci] + ph * g.W + pw] = acc[ph][pw];
+    }
+    __syncthreads();
+
+    // ---- the range leaves as one contiguous stream -------------------------------------------------------------------
+    float *dst = gin + base;
+#pragma unroll
+    for (int u = 0; u < PXL; ++u) {
+        const int e = tid + u * 256;
+        if (e < npix) {
+            float v = px[e];
+            if (mask.in) {
+                v = mv[u] > mask.threshold ? v : 0.0f;
+                if (twin.base) px[e] = v;  // the second copy takes the masked values
+            }
+            dst[e] = v;
+        }
+    }
+    if (!twin.base) return;
+    if (mask.in) __syncthreads();
+    // The second copy: per plane the rows lie twin.pitch apart; with twin_gaps the floats between one row's end and
+    // the next row's start (zeros by the buffer's contract) are stored too, which makes the plane's rows one run.
+    const bool more_rows = h0 + nh < g.H;  // the strip's last row is followed by another row of the plane
+    const int run = twin_gaps ? (more_rows ? nh * twin.pitch : (nh - 1) * twin.pitch + g.W) : nh * twin.pitch;
+    for (int pl = 0; pl < np; ++pl) {
+        float *t = twin.base + (long)(plane0 + pl) * twin.plane + (long)h0 * twin.pitch;
+        const float *src = px + pl * nh * g.W;
+        for (int e = tid; e < run; e += 256) {
+            unsigned hl, xq;
+            p.divTwinPitch.divmod((unsigned)e, hl, xq);
+            if ((int)xq < g.W) t[e] = src[(int)hl * g.W + (int)xq];
+            else if (twin_gaps) t[e] = 0.0f;
+        }
+    }
+}
+
+// Shape of the staged kernel's launch; false when one cell row of a plane does not fit a workgroup.
+bool plan_pool_staged(const PoolGeom &g, long planes, int dH, int dW, int twin_pitch, PoolStagedPlan &p) {
+    long max_pix = 256L * kStagedPixelsPerLane;
+    const long max_cells = 256L * kStagedCellsPerLane;
+    const int want = tuning().pool_bwd_pixels;  // (a tuning aid: a smaller workgroup share)
+    if (want >= 256 && want < max_pix) max_pix = want;
+    const long Yc = (g.H + dH - 1) / dH, Xc = (g.W + dW - 1) / dW;
+    p.Xc = (int)Xc;
+    if ((long)dH * g.W > max_pix || Xc > max_cells) return false;
+    if ((long)g.H * g.W <= max_pix && Yc * Xc <= max_cells) {
+        long G = max_pix / ((long)g.H * g.W);
+        if (G > max_cells / (Yc * Xc)) G = max_cells / (Yc * Xc);
+        if (G > planes) G = planes;
+        p.G = (int)(G < 1 ? 1 : G);
+        p.PR = g.H;
+    } else {
+        p.G = 1;
+        long cell_rows = max_pix / ((long)dH * g.W);  // cell rows per strip
+        if (cell_rows > max_cells / Xc) cell_rows = max_cells / Xc;
+        if (cell_rows < 1) return false;
+        const long strips = (Yc + cell_rows - 1) / cell_rows;
+        cell_rows = (Yc + strips - 1) / strips;  // even strips
+        p.PR = (int)(cell_rows * dH);
+    }
+    p.strips = (g.H + p.PR - 1) / p.PR;
+    p.divStrips = FastDiv((uint32_t)p.strips);
+    p.divXc = FastDiv((uint32_t)Xc);
+    p.divPlaneCells = FastDiv((uint32_t)(Yc * Xc));
+    p.divTwinPitch = FastDiv((uint32_t)(twin_pitch > 0 ? twin_pitch : 1));
+    return true;
+}
+
 // The direct kernel, for geometries the tile kernel's plan does not take.  Every pixel visits the windows
 // covering it in (i ascending, j ascending) order.
 __global__ __launch_bounds__(256) void maxpool_bwd_direct_kernel(const float *__restrict__ gout,
@@ -800,6 +983,18 @@ long pool_plan_selftest() {
                             }
                             if (!ok) ++bad;
                         }
+                        PoolStagedPlan sp;
+                        if (plan_pool_staged(g, planes, d, dw, W + 3, sp)) {
+                            const long Yc = (H + d - 1) / d, Xc = (W + dw - 1) / dw;
+                            const long cell_rows = sp.G > 1 || sp.PR == H ? Yc : sp.PR / d;
+                            const bool ok = sp.G >= 1 && sp.G <= planes && sp.PR >= 1 && sp.PR <= H &&
+                                            (sp.G == 1 || sp.PR == H) && (sp.PR == H || sp.PR % d == 0) &&
+                                            (long)sp.G * sp.PR * W <= 256L * kStagedPixelsPerLane &&
+                                            (long)sp.G * cell_rows * Xc <= 256L * kStagedCellsPerLane &&
+                                            (long)sp.strips * sp.PR >= H && (long)(sp.strips - 1) * sp.PR < H &&
+                                            sp.Xc == Xc;
+                            if (!ok) ++bad;
+                        }
                         PoolFwdPlan f;
                         if (plan_pool_fwd(g, planes, f)) {
                             const long rows = f.G > 1 ? H : (long)(f.SR - 1) * d + k;
@@ -818,7 +1013,8 @@ long pool_plan_selftest() {
 }
 
 int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int H, int W, int Ho, int Wo, int kH,
-                       int kW, int dH, int dW, float *gin, InputMask mask, TwinOutput twin, bool *wrote_twin) {
+                       int kW, int dH, int dW, float *gin, InputMask mask, TwinOutput twin, bool *wrote_twin,
+                       bool twin_gaps) {
     if (wrote_twin) *wrote_twin = false;
     hipStream_t s = stream();
     if (!s) return 1;
@@ -840,6 +1036,41 @@ int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int
     // The cell kernel takes the window shapes it is compiled for; the pool_bwd_tile and pool_bwd_direct switches force
     // the LDS tile kernel and the direct kernel (testing and tuning aids).
     const bool cell_shape = (kH == 3 && kW == 3 && dH == 2 && dW == 2) || (kH == 2 && kW == 2 && dH == 2 && dW == 2);
+    // Staged or cell kernel: a launch of a few microseconds is over before the staged kernel's chain of requests,
+    // barrier and write-out has paid for itself (measured cross-over: 13x13 planes at batch 128, 5.5 M pixels, run
+    // 14 us on the cell kernel and 17.5 us staged; from some 20 M pixels on the staged kernel is ahead, by a third at
+    // sizes that stream from memory).  pool_bwd_pixels > 0 pins the staged kernel.
+    const bool small_launch = total < 12L * 1000 * 1000 && tuning().pool_bwd_pixels == 0;
+    PoolStagedPlan sp;
+    if (cell_shape && !tuning().pool_bwd_direct && !tuning().pool_bwd_tile && !tuning().pool_bwd_cell && !small_launch &&
+        Ho > 0 && Wo > 0 && plan_pool_staged(g, planes, dH, dW, twin.base ? twin.pitch : 0, sp)) {
+        const long blocks = ((planes + sp.G - 1) / sp.G) * sp.strips;
+        if (blocks < (1L << 30)) {
+            WeightJob side = {};
+            unsigned side_blocks = 0;
+            if (twin.base) {  // the second copy is part of the launch's traffic
+                bytes += 4.0 * (double)total;
+                if (wrote_twin) *wrote_twin = true;
+                // ... and whoever reads that copy next may have a kernel bank to re-order: this launch carries it
+                if (take_bank_job(side)) {
+                    side_blocks = (side.count + 255u) / 256u;
+                    bytes += 4.0 * (side.count + (double)side.M * side.C * side.kH * side.kW);
+                }
+            }
+            {
+                LaunchScope scope(pool_label("maxpool_bwd", g, planes), 0.0, bytes);
+                const dim3 grid((unsigned)blocks + side_blocks), block(256);
+                const size_t lds = sizeof(float) * (size_t)sp.G * sp.PR * W;
+#define THGPU_POOL_BWD_STAGED(KH_, KW_, DH_, DW_)                                                                     \
+    hipLaunchKernelGGL((maxpool_bwd_staged_kernel<KH_, KW_, DH_, DW_>), grid, block, lds, s, gout, indices,           \
+                       indices + ototal, gin, g, sp, (unsigned)planes, mask, twin, twin_gaps, (unsigned)blocks, side)
+                if (kH == 3) THGPU_POOL_BWD_STAGED(3, 3, 2, 2);
+                else THGPU_POOL_BWD_STAGED(2, 2, 2, 2);
+#undef THGPU_POOL_BWD_STAGED
+            }
+            return check_launch("maxpool_bwd");
+        }
+    }
     if (cell_shape && !tuning().pool_bwd_direct && !tuning().pool_bwd_tile && Ho > 0 && Wo > 0) {
         const long Yc = (H + dH - 1) / dH, Xc = (W + dW - 1) / dW;
         const long cells = planes * Yc * Xc;

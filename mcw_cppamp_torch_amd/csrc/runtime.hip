@@ -61,6 +61,10 @@ static int tuning_set(const char *name, const char *value) {
         g_tuning.pool_bwd_direct = v[0] == '1';
     } else if (!std::strcmp(name, "pool_bwd_tile")) {
         g_tuning.pool_bwd_tile = v[0] == '1';
+    } else if (!std::strcmp(name, "pool_bwd_cell")) {
+        g_tuning.pool_bwd_cell = v[0] == '1';
+    } else if (!std::strcmp(name, "pool_bwd_pixels")) {
+        g_tuning.pool_bwd_pixels = std::atoi(v);
     } else if (!std::strcmp(name, "gradbias_separate")) {
         g_tuning.gradbias_separate = v[0] == '1';
     } else {
@@ -77,7 +81,8 @@ const Tuning &tuning() {
             {"THGPU_IM2COL_KERNEL", "im2col_kernel"},   {"THGPU_IM2COL_PLAN", "im2col_plan"},
             {"THGPU_COL2IM_GENERIC", "col2im_generic"}, {"THGPU_POOL_FWD_WAVE", "pool_fwd_wave"},
             {"THGPU_POOL_BWD_DIRECT", "pool_bwd_direct"}, {"THGPU_GRADBIAS_SEPARATE", "gradbias_separate"},
-            {"THGPU_POOL_BWD_TILE", "pool_bwd_tile"}};
+            {"THGPU_POOL_BWD_TILE", "pool_bwd_tile"}, {"THGPU_POOL_BWD_CELL", "pool_bwd_cell"},
+            {"THGPU_POOL_BWD_PIXELS", "pool_bwd_pixels"}};
         for (auto &e : kEnv)
             if (const char *v = std::getenv(e[0])) (void)tuning_set(e[1], v);
     }

@@ -152,11 +152,13 @@ def test_every_kernel_that_stores_a_masked_gradient_or_a_thresholded_output(gt, 
         assert lib.thgpu_conv_set_mode(before) == 0
 
 
-@pytest.mark.parametrize("kernel", ["auto", "tile", "direct"])
+@pytest.mark.parametrize("kernel", ["auto", "tile", "direct", "cell", "staged", "staged_small_share"])
 @pytest.mark.parametrize("pool", [(3, 2), (2, 2), (3, 1)])
 def test_masked_pooling_backward(gt, pool, kernel, switches):
     switches("pool_bwd_direct", "1" if kernel == "direct" else None)
     switches("pool_bwd_tile", "1" if kernel == "tile" else None)
+    switches("pool_bwd_cell", "1" if kernel == "cell" else None)
+    switches("pool_bwd_pixels", {"staged": "4096", "staged_small_share": "300"}.get(kernel))
     spec = [("conv", 3, 8, 3, 1, 1), ("relu",), ("pool",) + pool]
     x = uniform(rng_for(94), (3, 3, 29, 31))
     _, out_u, gi_u, _, grads_u, go = run(gt, spec, x, 95, False)
@@ -240,8 +242,9 @@ TWIN_SPEC = [("conv", 3, 64, 5, 2, 2), ("relu",), ("pool", 3, 2), ("conv", 64, 1
              ("conv", 128, 64, 3, 1, 1), ("relu",), ("pool", 2, 2), ("conv", 64, 64, 5, 1, 2), ("relu",), ("pool", 3, 2)]
 
 
-@pytest.mark.parametrize("forced", [{}, {"gemm_split": "3"}, {"gemm_split": "1"}, {"pool_bwd_tile": "1"}],
-                         ids=["auto", "split", "unsplit", "pool_tile"])
+@pytest.mark.parametrize("forced", [{}, {"gemm_split": "3"}, {"gemm_split": "1"}, {"pool_bwd_tile": "1"},
+                                    {"pool_bwd_cell": "1"}, {"pool_bwd_pixels": "4096"}, {"pool_bwd_pixels": "500"}],
+                         ids=["auto", "split", "unsplit", "pool_tile", "pool_cell", "pool_staged", "pool_staged_strips"])
 def test_gradients_written_into_the_next_products_padded_buffer(gt, forced, switches):
     """In a fused Sequential on the gathered route every producer of a convolution's gradOutput (max-pooling backward,
     a unit-stride convolution's gradInput product through its epilogue or its split reduction) also stores it in that

@@ -307,14 +307,18 @@ POOLS = [(2, 3, 7, 7, 3, 3, 2, 2), (3, 2, 9, 8, 2, 2, 2, 2), (2, 2, 10, 11, 3, 2
          (3, 2, 40, 64, 3, 3, 1, 2), (2, 2, 33, 33, 2, 2, 1, 1), (1, 1, 64, 64, 64, 64, 1, 1)]
 
 
-@pytest.fixture(params=["auto", "direct", "tile"])
+@pytest.fixture(params=["auto", "direct", "tile", "cell", "staged", "staged_small_share"])
 def pool_bwd_kernel(request, switches):
-    """Runs a test with the library's own forward and backward kernel choice (direct forward; cell backward where a
-    window shape has one, else the LDS tile kernel), then with the wavefront-level tile forward and the direct backward
-    kernel forced, then with the LDS tile backward kernel forced."""
+    """Runs a test with the library's own forward and backward kernel choice (direct forward; for 3x3 / 2x2 windows at
+    stride 2 the cell backward kernel on small launches and the staged one on large, else the LDS tile kernel), then
+    with the wavefront-level tile forward and the direct backward kernel forced, then with each of the LDS tile, cell
+    and staged backward kernels forced (the staged one with its full workgroup share and with a small one, so that
+    strips of rows and ragged last groups occur on small planes too)."""
     switches("pool_fwd_wave", "1" if request.param == "direct" else None)
     switches("pool_bwd_direct", "1" if request.param == "direct" else None)
     switches("pool_bwd_tile", "1" if request.param == "tile" else None)
+    switches("pool_bwd_cell", "1" if request.param == "cell" else None)
+    switches("pool_bwd_pixels", {"staged": "4096", "staged_small_share": "300"}.get(request.param))
     return request.param
 
 
