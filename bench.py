@@ -425,6 +425,7 @@ def summarise(args):
     bench.py --summarise traffic FETCH.csv WRITE.csv BENCH.json STEPS  (two --pmc runs' _counter_collection.csv)
     bench.py --summarise mfma COUNTERS.csv                             (one --pmc run with the SQ_* counters)
     bench.py --summarise hbm-pmc COUNTERS.csv KERNEL_TRACE.csv         (one --pmc run around --workload hbm_sweep)
+    bench.py --summarise requests REQ.csv FETCH.csv WRITE.csv REQ_KERNEL_TRACE.csv   (three --pmc runs around hbm_sweep)
     BENCH.json is the line an ordinary run of the same configuration printed; STEPS the steps the profiled runs made
     (warm-up included).  Writes the summary to stdout; `header` lines (the commands) come from --summary-header."""
     kind, files = args.summarise[0], args.summarise[1:]
@@ -485,6 +486,9 @@ def summarise(args):
                                                                     ("%.2f" % ((fe + wr) / al)) if al else "-"))
         g = fam["gemm"]
         per = (g[1] + g[2]) / g[0]
+        if "fill" in fam:
+            out.append("(fill: the profiled run's first step also writes the zero borders of the padded buffers, once per buffer; a later "
+                       "step only zeroes gradWeight / gradBias, the algorithmic figure.)")
         out += ["", "All kernels: %.1f MiB per step." % total,
                 "GEMM family: %.1f MiB per step over %d launches = %.1f MiB (%.4g bytes) per launch on average."
                 % ((g[1] + g[2]) / steps, g[0] / steps, per, per * 1048576),
@@ -543,8 +547,47 @@ def summarise(args):
         out.append("waves/SIMD = 4 * SQ_WAVE_CYCLES / (launch duration * 2.4 GHz * 1024 SIMDs), at most 8; life = mean residence of "
                    "a wavefront; waiting = SQ_WAIT_ANY / SQ_WAVE_CYCLES (any wait, barriers included); on mem = SQ_WAIT_INST_ANY / "
                    "SQ_WAVE_CYCLES; VALU / LDS / VMEM = instructions per wavefront.")
+    elif kind == "requests":
+        # Three --pmc runs around `bench.py --workload hbm_sweep` (TCP_TCC_READ_REQ_sum TCP_TCC_WRITE_REQ_sum; FETCH_SIZE;
+        # WRITE_SIZE), each with --kernel-trace: how many requests a kernel sends from the vector caches to the L2 and
+        # how many bytes each carries on average -- the request rate, not the byte rate, is what a kernel with short or
+        # misaligned runs saturates.
+        def load(path):
+            d = collections.OrderedDict()
+            for r in csv.DictReader(open(path)):
+                e = d.setdefault(int(r["Dispatch_Id"]), {"name": r["Kernel_Name"], "grid": int(r["Grid_Size"]), "ns": 0})
+                e[r["Counter_Name"]] = float(r["Counter_Value"])
+            return d
+        req, fetch, write = load(files[0]), load(files[1]), load(files[2])
+        for r in csv.DictReader(open(files[3])):             # durations: the kernel trace of the request-counter run
+            if int(r["Dispatch_Id"]) in req:
+                req[int(r["Dispatch_Id"])]["ns"] = int(r["End_Timestamp"]) - int(r["Start_Timestamp"])
+        agg = collections.OrderedDict()
+        for k, e in req.items():
+            fam = _family(e["name"])
+            if fam is None or fam == "gemm" or k not in fetch or k not in write:
+                continue
+            a = agg.setdefault((fam, _short(e["name"])[:34], e["grid"]), collections.defaultdict(float))
+            a["n"] += 1
+            a["ns"] += e["ns"]
+            a["rd"] += e.get("TCP_TCC_READ_REQ_sum", 0.0)
+            a["wr"] += e.get("TCP_TCC_WRITE_REQ_sum", 0.0)
+            a["fetch"] += fetch[k].get("FETCH_SIZE", 0.0) * FETCH_SCALE * 1024
+            a["write"] += write[k].get("WRITE_SIZE", 0.0) * WRITE_SCALE * 1024
+        out.append("%-34s %10s %8s %9s %10s %10s %9s %9s %8s %8s" % (
+            "kernel", "threads", "launches", "us/launch", "read req", "write req", "fetch MiB", "write MiB", "B/rd req",
+            "B/wr req"))
+        for (fam, name, grid), a in agg.items():
+            n = a["n"]
+            out.append("%-34s %10d %8d %9.1f %10.0f %10.0f %9.1f %9.1f %8.0f %8.0f" % (
+                name, grid, n, a["ns"] / n / 1e3, a["rd"] / n, a["wr"] / n, a["fetch"] / n / 1048576, a["write"] / n / 1048576,
+                a["fetch"] / max(a["rd"], 1), a["write"] / max(a["wr"], 1)))
+        out.append("read / write req = TCP_TCC_READ_REQ_sum / TCP_TCC_WRITE_REQ_sum per launch; fetch / write MiB = FETCH_SIZE x %.1f, "
+                   "WRITE_SIZE x %.1f (memory-side traffic); B/req = memory-side bytes per L2 request of that direction (reads "
+                   "served by the L2 lower it, a full request carries 64 bytes of a store or 128 of a load)."
+                   % (FETCH_SCALE, WRITE_SCALE))
     else:
-        sys.exit("--summarise kernel-trace | traffic | mfma | hbm-pmc")
+        sys.exit("--summarise kernel-trace | traffic | mfma | hbm-pmc | requests")
     print("\n".join(out))
 
 

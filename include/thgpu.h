@@ -470,8 +470,9 @@ int thgpu_SpatialConvolutionMM_accGradParametersFused(THGPUTensor *input, THGPUT
  *      (and nothing is touched) when the layer's gradInput does not take the gathered route.
  *   2. the producer's updateGradInput -- thgpu_SpatialMaxPooling_updateGradInputTwin or
  *      thgpu_SpatialConvolutionMM_updateGradInputTwin with that `twin` -- stores every value of its gradInput a second
- *      time through the view; *wrote_twin says whether the kernel that ran could (the max-pooling cell kernel and the
- *      unit-stride gathered gradInput product can; otherwise only the dense result is written).
+ *      time through the view; *wrote_twin says whether the kernel that ran could (the max-pooling kernels for 3x3 and 2x2
+ *      windows at stride 2 and the unit-stride gathered gradInput product can; otherwise only the dense result is
+ *      written).
  *   3. the layer's thgpu_SpatialConvolutionMM_updateGradInputTwin with THGPU_GRADOUTPUT_IN_TWIN, called with that
  *      dense gradInput as gradOutput before anything else touches either tensor: no padded copy is made.  The flag
  *      is the caller's word for the contents; it is ignored (the copy is made) unless fgradInput is still the buffer
