@@ -568,16 +568,38 @@ __global__ __launch_bounds__(256) void maxpool_bwd_cell_kernel(const float *__re
 // as a contiguous stream too) applied on the way.  A second copy (TwinOutput) leaves the same way, row gaps included
 // when they are known to hold zeros, so that it is a contiguous stream as well.
 constexpr int kStagedPixelsPerLane = 16;  // a workgroup stages up to 4096 pixels (16 KB of LDS)
-constexpr int kStagedCellsPerLane = 4;    // ... computed as up to 1024 cells
+constexpr int kStagedCellsPerLane = 4;    // ... computed as up to 4 passes of 256 / Xc cell rows
 
 struct PoolStagedPlan {
-    int G;       // planes per workgroup (more than one only when a strip is the whole plane)
-    int PR;      // pixel rows per strip (a multiple of the row stride unless the strip is the whole plane)
-    int strips;  // strips per plane
-    int Xc;      // cells per cell row
-    FastDiv divStrips, divXc, divPlaneCells, divTwinPitch;
+    int G;         // planes per workgroup (more than one only when a strip is the whole plane)
+    int PR;        // pixel rows per strip (a multiple of the row stride unless the strip is the whole plane)
+    int strips;    // strips per plane
+    int Xc;        // cells per cell row
+    int pass_rows; // cell rows a workgroup's 256 lanes cover at once: 256 / Xc
+    int twin_step_rows, twin_step_cols;  // 256 = twin_step_rows * (row pitch of the second copy) + twin_step_cols
+    FastDiv divStrips, divXc, divYc, divTwinPitch;
 };
 
+// A float at a byte offset from a wavefront-uniform base: the address is scalar base + 32-bit lane offset, one
+// instruction's worth of address arithmetic instead of a 64-bit multiply-add per access.
+__device__ __forceinline__ float pool_ld(const float *base, unsigned byte_off) {
+    return *reinterpret_cast<const float *>(reinterpret_cast<const char *>(base) + byte_off);
+}
+__device__ __forceinline__ void pool_st(float *base, unsigned byte_off, float v) {
+    *reinterpret_cast<float *>(reinterpret_cast<char *>(base) + byte_off) = v;
+}
+// Quotient and remainder of a number below 2^24 (a lane or cell index within a workgroup's range): the remainder
+// through the full-rate 24-bit multiply.
+__device__ __forceinline__ void pool_divmod24(const FastDiv &d, unsigned n, unsigned &q, unsigned &r) {
+    q = d.div(n);
+    r = n - __umul24(q, d.d);
+}
+
+// The instruction count per pixel is what bounds this kernel once its streams are contiguous, so the indexing is
+// arranged to be cheap: a lane keeps ONE cell column x for all its cells (cell row r0 + ci * pass_rows of the range),
+// so column clamps and validity are computed once; every array is addressed as a uniform per-workgroup base plus a
+// 32-bit byte offset; and a window's saved argmax is compared as one number, wy * 1024 + wx (both small integers
+// held in floats, so the sum is exact), against the constant that names the pixel.
 template <int KH, int KW, int DH, int DW>
 __global__ __launch_bounds__(256) void maxpool_bwd_staged_kernel(const float *__restrict__ gout,
                                                                  const float *__restrict__ indy,
@@ -594,15 +616,22 @@ __global__ __launch_bounds__(256) void maxpool_bwd_staged_kernel(const float *__
     }
     constexpr int TH = (KH + DH - 1) / DH, TW = (KW + DW - 1) / DW;
     constexpr int PXL = kStagedPixelsPerLane, CI = kStagedCellsPerLane;
-    const int tid = threadIdx.x;
+    const unsigned tid = threadIdx.x;
     unsigned grp, strip;
     p.divStrips.divmod(blockIdx.x, grp, strip);
     const unsigned plane0 = grp * (unsigned)p.G;
     const int np = (int)(planes - plane0 < (unsigned)p.G ? planes - plane0 : (unsigned)p.G);
     const int h0 = (int)strip * p.PR;
     const int nh = g.H - h0 < p.PR ? g.H - h0 : p.PR;
-    const int npix = np * nh * g.W;
+    const unsigned npix = (unsigned)(np * nh * g.W);
     const long base = (long)plane0 * g.H * g.W + (long)h0 * g.W;  // (h0 = 0 when planes are grouped)
+
+    // The write-out's lanes are shifted so that every wavefront store of 64 consecutive floats starts on a 64-byte
+    // line of gradInput: a store leaves the vector cache in 64-byte requests, and a run that starts mid-line costs five
+    // requests instead of four (the range starts wherever its plane does).  Lane t takes the floats t - shift + 256 u;
+    // the plan leaves room for the up to 15 lanes that fall in front of the range.
+    float *dst = gin + base;
+    const unsigned shift = (unsigned)((reinterpret_cast<uintptr_t>(dst) >> 2) & 15u);
 
     // ---- the mask of the range: requested first, used last ---------------------------------------------------------
     float mv[PXL];
@@ -610,43 +639,62 @@ __global__ __launch_bounds__(256) void maxpool_bwd_staged_kernel(const float *__
         const float *m = mask.in + base;
 #pragma unroll
         for (int u = 0; u < PXL; ++u) {
-            const int e = tid + u * 256;
-            mv[u] = e < npix ? m[e] : 0.0f;
+            const unsigned e = tid + u * 256u - shift;  // (wraps to a huge number in front of the range)
+            mv[u] = pool_ld(m, (e < npix ? e : 0u) * 4u);
         }
     }
 
     // ---- the range's cells: all window requests of a lane's cells go out before the first is used -------------------
-    const int yc0 = h0 / DH;                       // strips start on a cell row
+    const long wbase = (long)plane0 * g.Ho * g.Wo;  // the group's first window
+    const float *gb = gout + wbase, *yb = indy + wbase, *xb = indx + wbase;
+    const int yc0 = h0 / DH;  // strips start on a cell row
     const int nyc = (nh + DH - 1) / DH;
-    const int per_plane = nyc * p.Xc;
-    const int ncell = np * per_plane;
-    float wg[CI][TH][TW], wy[CI][TH][TW], wx[CI][TH][TW];
-    bool win[CI][TH][TW];
-    int cell_px[CI], cell_hl[CI], cell_w0[CI];  // LDS offset of the cell's first pixel, its row in the range, its column
+    const unsigned nrows = (unsigned)(np * nyc);  // cell rows of the range
+    unsigned r0, x;
+    pool_divmod24(p.divXc, tid, r0, x);
+    const bool lane_live = r0 < (unsigned)p.pass_rows;  // (the last 256 mod Xc lanes have no column of their own)
+    // the lane's column: which of its TW window columns exist, where they are, which of its DW pixel columns exist
+    bool cv[TW], pv[DW];
+    unsigned jb[TW];  // byte offset of the window column within a row of windows
+#pragma unroll
+    for (int b = 0; b < TW; ++b) {
+        const int j = (int)x - b;
+        cv[b] = j >= 0 && j < g.Wo;
+        jb[b] = (unsigned)(j < 0 ? 0 : j < g.Wo ? j : g.Wo - 1) * 4u;
+    }
+#pragma unroll
+    for (int pw = 0; pw < DW; ++pw) pv[pw] = (int)x * DW + pw < g.W;
+    float wg[CI][TH][TW], code[CI][TH][TW];
+    bool win[CI][TH][TW], rowlive[CI];
+    int cell_hl[CI];        // the cell's first row in the range
+    unsigned cell_px[CI];   // LDS offset of the cell's first pixel
 #pragma unroll
     for (int ci = 0; ci < CI; ++ci) {
-        const int c = tid + ci * 256;
-        const bool live = c < ncell;
-        unsigned pl = 0, rem = (unsigned)(live ? c : 0), yl, x;
-        if (p.G > 1) p.divPlaneCells.divmod(rem, pl, rem);  // grouped planes are whole: Yc*Xc cells each
-        p.divXc.divmod(rem, yl, x);
+        const unsigned r = r0 + (unsigned)(ci * p.pass_rows);
+        rowlive[ci] = lane_live && r < nrows;
+        const unsigned rr = rowlive[ci] ? r : 0u;
+        unsigned pl = 0, yl = rr;
+        if (p.G > 1) pool_divmod24(p.divYc, rr, pl, yl);  // grouped planes are whole: Yc cell rows each
         const int y = yc0 + (int)yl;
-        cell_hl[ci] = live ? (int)yl * DH : nh;              // (a dead cell owns no row of the range)
-        cell_w0[ci] = (int)x * DW;
-        cell_px[ci] = ((int)pl * nh + (int)yl * DH) * g.W + (int)x * DW;
-        const long obase = (long)(plane0 + pl) * g.Ho * g.Wo;
+        cell_hl[ci] = (int)yl * DH;
+        // (every product here is of numbers far below 2^24: the full-rate 24-bit multiply)
+        cell_px[ci] = __umul24(__umul24(pl, (unsigned)nh) + yl * DH, (unsigned)g.W) + x * DW;
 #pragma unroll
-        for (int a = 0; a < TH; ++a)
+        for (int a = 0; a < TH; ++a) {
+            const int i = y - a;
+            const bool rv = rowlive[ci] && i >= 0 && i < g.Ho;
+            const unsigned iclamp = (unsigned)(i < 0 ? 0 : i < g.Ho ? i : g.Ho - 1);
+            const unsigned ib = __umul24(__umul24(pl, (unsigned)g.Ho) + iclamp, (unsigned)g.Wo * 4u);
 #pragma unroll
             for (int b = 0; b < TW; ++b) {
-                const int i = y - a, j = (int)x - b;
-                win[ci][a][b] = live && i >= 0 && i < g.Ho && j >= 0 && j < g.Wo;
-                const int ic = i < 0 ? 0 : i < g.Ho ? i : g.Ho - 1, jc = j < 0 ? 0 : j < g.Wo ? j : g.Wo - 1;
-                const long o = obase + (long)ic * g.Wo + jc;
-                wg[ci][a][b] = gout[o];
-                wy[ci][a][b] = indy[o];
-                wx[ci][a][b] = indx[o];
+                // every load unconditional, from an index clamped into the group's windows; what a clamped index
+                // fetched is discarded through `win`
+                const unsigned o = ib + jb[b];
+                win[ci][a][b] = rv && cv[b];
+                wg[ci][a][b] = pool_ld(gb, o);
+                code[ci][a][b] = __fmaf_rn(pool_ld(yb, o), 1024.0f, pool_ld(xb, o));
             }
+        }
     }
 #pragma unroll
     for (int ci = 0; ci < CI; ++ci) {
@@ -660,84 +708,109 @@ __global__ __launch_bounds__(256) void maxpool_bwd_staged_kernel(const float *__
         for (int a = TH - 1; a >= 0; --a)
 #pragma unroll
             for (int b = TW - 1; b >= 0; --b) {
-                const int ky = win[ci][a][b] ? (int)wy[ci][a][b] - 1 - a * DH : -1, kx = (int)wx[ci][a][b] - 1 - b * DW;
+                const float c = win[ci][a][b] ? code[ci][a][b] : 0.0f;  // (a saved argmax is 1-based: never 0)
 #pragma unroll
                 for (int ph = 0; ph < DH; ++ph)
 #pragma unroll
                     for (int pw = 0; pw < DW; ++pw) {
+                        // taps beyond the window ((ph + a*DH, pw + b*DW) outside KH x KW) are never saved
                         if (ph + a * DH >= KH || pw + b * DW >= KW) continue;
-                        acc[ph][pw] += (ky == ph && kx == pw) ? wg[ci][a][b] : 0.0f;
+                        const float hit = (float)((ph + a * DH + 1) * 1024 + pw + b * DW + 1);
+                        acc[ph][pw] += c == hit ? wg[ci][a][b] : 0.0f;
                     }
             }
 #pragma unroll
         for (int ph = 0; ph < DH; ++ph)
 #pragma unroll
             for (int pw = 0; pw < DW; ++pw)
-                if (cell_hl[ci] + ph < nh && cell_w0[ci] + pw < g.W) px[cell_px[ci] + ph * g.W + pw] = acc[ph][pw];
+                if (rowlive[ci] && cell_hl[ci] + ph < nh && pv[pw]) px[cell_px[ci] + ph * g.W + pw] = acc[ph][pw];
     }
     __syncthreads();
 
     // ---- the range leaves as one contiguous stream -------------------------------------------------------------------
-    float *dst = gin + base;
+    float v[PXL];
+#pragma unroll
+    for (int u = 0; u < PXL; ++u) {  // all LDS reads first (from a clamped index: no branch, no wait in between)
+        const unsigned e = tid + u * 256u - shift;
+        v[u] = px[e < npix ? e : 0u];
+    }
+    if (mask.in) {
+#pragma unroll
+        for (int u = 0; u < PXL; ++u) v[u] = mv[u] > mask.threshold ? v[u] : 0.0f;
+        if (twin.base) {  // the second copy takes the masked values
+#pragma unroll
+            for (int u = 0; u < PXL; ++u) {
+                const unsigned e = tid + u * 256u - shift;
+                if (e < npix) px[e] = v[u];
+            }
+        }
+    }
 #pragma unroll
     for (int u = 0; u < PXL; ++u) {
-        const int e = tid + u * 256;
-        if (e < npix) {
-            float v = px[e];
-            if (mask.in) {
-                v = mv[u] > mask.threshold ? v : 0.0f;
-                if (twin.base) px[e] = v;  // the second copy takes the masked values
-            }
-            dst[e] = v;
-        }
+        const unsigned e = tid + u * 256u - shift;
+        if (e < npix) pool_st(dst, e * 4u, v[u]);
     }
     if (!twin.base) return;
     if (mask.in) __syncthreads();
     // The second copy: per plane the rows lie twin.pitch apart; with twin_gaps the floats between one row's end and
     // the next row's start (zeros by the buffer's contract) are stored too, which makes the plane's rows one run.
+    // A lane walks the run in steps of 256 floats and keeps (row, column) by carrying, without a division per float.
     const bool more_rows = h0 + nh < g.H;  // the strip's last row is followed by another row of the plane
-    const int run = twin_gaps ? (more_rows ? nh * twin.pitch : (nh - 1) * twin.pitch + g.W) : nh * twin.pitch;
+    const unsigned run = (unsigned)(twin_gaps && !more_rows ? (nh - 1) * twin.pitch + g.W : nh * twin.pitch);
+    unsigned hl0, xq0;
+    pool_divmod24(p.divTwinPitch, tid, hl0, xq0);
     for (int pl = 0; pl < np; ++pl) {
         float *t = twin.base + (long)(plane0 + pl) * twin.plane + (long)h0 * twin.pitch;
         const float *src = px + pl * nh * g.W;
-        for (int e = tid; e < run; e += 256) {
-            unsigned hl, xq;
-            p.divTwinPitch.divmod((unsigned)e, hl, xq);
-            if ((int)xq < g.W) t[e] = src[(int)hl * g.W + (int)xq];
-            else if (twin_gaps) t[e] = 0.0f;
+        unsigned xq = xq0, srow = __umul24(hl0, (unsigned)g.W);  // column in the padded row, LDS offset of the source row
+        for (unsigned e = tid; e < run; e += 256u) {
+            if (xq < (unsigned)g.W) pool_st(t, e * 4u, src[srow + xq]);
+            else if (twin_gaps) pool_st(t, e * 4u, 0.0f);
+            xq += (unsigned)p.twin_step_cols;
+            srow += (unsigned)(p.twin_step_rows * g.W);
+            if (xq >= (unsigned)twin.pitch) {
+                xq -= (unsigned)twin.pitch;
+                srow += (unsigned)g.W;
+            }
         }
     }
 }
 
-// Shape of the staged kernel's launch; false when one cell row of a plane does not fit a workgroup.
+// Shape of the staged kernel's launch; false when a cell row of a plane does not fit a workgroup's lanes or its LDS.
 bool plan_pool_staged(const PoolGeom &g, long planes, int dH, int dW, int twin_pitch, PoolStagedPlan &p) {
-    long max_pix = 256L * kStagedPixelsPerLane;
-    const long max_cells = 256L * kStagedCellsPerLane;
+    long max_pix = 256L * kStagedPixelsPerLane - 16;  // (up to 15 lanes of the write-out fall in front of the range)
     const int want = tuning().pool_bwd_pixels;  // (a tuning aid: a smaller workgroup share)
     if (want >= 256 && want < max_pix) max_pix = want;
     const long Yc = (g.H + dH - 1) / dH, Xc = (g.W + dW - 1) / dW;
     p.Xc = (int)Xc;
-    if ((long)dH * g.W > max_pix || Xc > max_cells) return false;
-    if ((long)g.H * g.W <= max_pix && Yc * Xc <= max_cells) {
+    if ((long)dH * g.W > max_pix || Xc > 256) return false;
+    p.pass_rows = (int)(256 / Xc);
+    const long max_rows = (long)kStagedCellsPerLane * p.pass_rows;  // cell rows per workgroup
+    if ((long)g.H * g.W <= max_pix && Yc <= max_rows) {
         long G = max_pix / ((long)g.H * g.W);
-        if (G > max_cells / (Yc * Xc)) G = max_cells / (Yc * Xc);
+        if (G > max_rows / Yc) G = max_rows / Yc;
         if (G > planes) G = planes;
         p.G = (int)(G < 1 ? 1 : G);
         p.PR = g.H;
     } else {
         p.G = 1;
         long cell_rows = max_pix / ((long)dH * g.W);  // cell rows per strip
-        if (cell_rows > max_cells / Xc) cell_rows = max_cells / Xc;
+        if (cell_rows > max_rows) cell_rows = max_rows;
         if (cell_rows < 1) return false;
         const long strips = (Yc + cell_rows - 1) / cell_rows;
         cell_rows = (Yc + strips - 1) / strips;  // even strips
         p.PR = (int)(cell_rows * dH);
     }
+    // the kernel addresses a group's windows by 32-bit byte offsets built with 24-bit multiplies
+    if ((long)p.G * g.Ho >= (1L << 24) || (long)p.G * g.Ho * g.Wo >= (1L << 29)) return false;
     p.strips = (g.H + p.PR - 1) / p.PR;
     p.divStrips = FastDiv((uint32_t)p.strips);
     p.divXc = FastDiv((uint32_t)Xc);
-    p.divPlaneCells = FastDiv((uint32_t)(Yc * Xc));
-    p.divTwinPitch = FastDiv((uint32_t)(twin_pitch > 0 ? twin_pitch : 1));
+    p.divYc = FastDiv((uint32_t)Yc);
+    const int pitch = twin_pitch > 0 ? twin_pitch : 1;
+    p.divTwinPitch = FastDiv((uint32_t)pitch);
+    p.twin_step_rows = 256 / pitch;
+    p.twin_step_cols = 256 % pitch;
     return true;
 }
 
@@ -989,8 +1062,9 @@ long pool_plan_selftest() {
                             const long cell_rows = sp.G > 1 || sp.PR == H ? Yc : sp.PR / d;
                             const bool ok = sp.G >= 1 && sp.G <= planes && sp.PR >= 1 && sp.PR <= H &&
                                             (sp.G == 1 || sp.PR == H) && (sp.PR == H || sp.PR % d == 0) &&
-                                            (long)sp.G * sp.PR * W <= 256L * kStagedPixelsPerLane &&
-                                            (long)sp.G * cell_rows * Xc <= 256L * kStagedCellsPerLane &&
+                                            (long)sp.G * sp.PR * W <= 256L * kStagedPixelsPerLane - 16 &&
+                                            Xc <= 256 && sp.pass_rows == 256 / Xc &&
+                                            (long)sp.G * cell_rows <= (long)kStagedCellsPerLane * sp.pass_rows &&
                                             (long)sp.strips * sp.PR >= H && (long)(sp.strips - 1) * sp.PR < H &&
                                             sp.Xc == Xc;
                             if (!ok) ++bad;
@@ -1077,7 +1151,7 @@ int maxpool_bwd_launch(const float *gout, const float *indices, long planes, int
         if (cells < (1L << 31)) {
             WeightJob side = {};
             unsigned side_blocks = 0;
-            if (twin.base) {  // only this kernel keeps a second copy; it is part of the launch's traffic
+            if (twin.base) {  // the second copy is part of the launch's traffic
                 bytes += 4.0 * (double)total;
                 if (wrote_twin) *wrote_twin = true;
                 // ... and whoever reads that copy next may have a kernel bank to re-order: this launch carries it
