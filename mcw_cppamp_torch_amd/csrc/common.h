@@ -67,7 +67,7 @@ float *static_scratch(size_t *floats);
 
 // Testing and tuning switches.  Filled from the environment once, when the library initialises
 // (THGPU_GEMM_TILE, THGPU_GEMM_SPLIT, THGPU_IM2COL_KERNEL, THGPU_IM2COL_PLAN, THGPU_COL2IM_GENERIC,
-// THGPU_POOL_FWD_WAVE, THGPU_POOL_BWD_DIRECT, THGPU_POOL_BWD_TILE, THGPU_POOL_BWD_CELL), and changed afterwards only through thgpu_debug_set: no launch reads the
+// THGPU_POOL_FWD_WAVE, THGPU_POOL_BWD_DIRECT, THGPU_POOL_BWD_TILE, THGPU_POOL_BWD_CELL, THGPU_CONV_NARROW_OFF), and changed afterwards only through thgpu_debug_set: no launch reads the
 // environment.
 struct Tuning {
     char gemm_tile[16] = "";      // a tile configuration by name; "" leaves the choice to the cost model
@@ -81,6 +81,7 @@ struct Tuning {
     bool pool_bwd_cell = false;   // the cell backward kernel (no LDS) where the staged kernel would run
     int pool_bwd_pixels = 0;      // pixels a workgroup of the staged backward kernel takes; 0 leaves it to the planner
     bool gradbias_separate = false;  // the two-stage bias-gradient sum even where the gradWeight product could do it
+    bool conv_narrow_off = false;    // the tiled GEMM kernels where the kernels for layers with a handful of taps would run
 };
 const Tuning &tuning();
 

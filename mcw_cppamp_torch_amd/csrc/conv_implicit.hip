@@ -527,6 +527,9 @@ int conv_implicit_forward(const float *padded, const float *weight, const float 
     p.rowtab = tap_table(C, kH, kW, Hp * Wp, Wp);
     p.coltab = pixel_table(Ho, Wo, sH * Wp, sW);
     if (!p.rowtab || !p.coltab) return 1;
+    if (conv_narrow_forward_fits(B, M, (long)C * kH * kW, Wo, (long)Ho * Wo, sW, out))
+        return conv_narrow_forward(padded, (long)C * Hp * Wp, weight, bias, output, B, M, C * kH * kW, Ho, Wo, sH * Wp,
+                                   p.rowtab, act);
     p.C = output;
     p.bias = bias;
     p.act = act.on;

@@ -71,6 +71,12 @@ struct OutputThreshold {
 int conv_implicit_forward(const float *padded, const float *weight, const float *bias, float *output, long B, int C,
                           int H, int W, int M, int kH, int kW, int pH, int pW, int sH, int sW,
                           OutputThreshold act = OutputThreshold(), OutputLayout out = OutputLayout());
+// Forward of a layer with at most 32 taps and 64 output planes without the tiled GEMM (conv_narrow.hip): whether the
+// shape is taken, and the launch (padded images image_stride floats apart; output position (y, x) reads from
+// y * row_step + x on; the gathered route's tap table).
+bool conv_narrow_forward_fits(long B, int M, long K, int Wo, long N, int col_step, OutputLayout out);
+int conv_narrow_forward(const float *padded, long image_stride, const float *weight, const float *bias, float *output,
+                        long B, int M, int K, int Ho, int Wo, int row_step, const int *rowtab, OutputThreshold act);
 // gradBias (may be null) receives scale * the sums of gradOutput over images and positions when the product can
 // compute them on the side; *bias_done says whether it did.
 int conv_implicit_gradweight(const float *padded, const float *gradOutput, float *gradWeight, long B, int C, int H,

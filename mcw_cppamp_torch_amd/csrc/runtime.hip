@@ -67,6 +67,8 @@ static int tuning_set(const char *name, const char *value) {
         g_tuning.pool_bwd_pixels = std::atoi(v);
     } else if (!std::strcmp(name, "gradbias_separate")) {
         g_tuning.gradbias_separate = v[0] == '1';
+    } else if (!std::strcmp(name, "conv_narrow_off")) {
+        g_tuning.conv_narrow_off = v[0] == '1';
     } else {
         return fail("thgpu_debug_set: unknown switch '%s'", name);
     }
@@ -82,7 +84,7 @@ const Tuning &tuning() {
             {"THGPU_COL2IM_GENERIC", "col2im_generic"}, {"THGPU_POOL_FWD_WAVE", "pool_fwd_wave"},
             {"THGPU_POOL_BWD_DIRECT", "pool_bwd_direct"}, {"THGPU_GRADBIAS_SEPARATE", "gradbias_separate"},
             {"THGPU_POOL_BWD_TILE", "pool_bwd_tile"}, {"THGPU_POOL_BWD_CELL", "pool_bwd_cell"},
-            {"THGPU_POOL_BWD_PIXELS", "pool_bwd_pixels"}};
+            {"THGPU_POOL_BWD_PIXELS", "pool_bwd_pixels"}, {"THGPU_CONV_NARROW_OFF", "conv_narrow_off"}};
         for (auto &e : kEnv)
             if (const char *v = std::getenv(e[0])) (void)tuning_set(e[1], v);
     }

@@ -578,3 +578,94 @@ def test_narrow_gradweight_runs_wide_and_stores_its_own_columns_integer_exact(gt
     gw_label = [k for k in labels if k.startswith("gemm_conv_gradweight")]
     assert len(gw_label) == 1 and "J=64 " in gw_label[0] and "tile=64x64" in gw_label[0] and "split=1 " not in gw_label[0] + " ", labels
     assert not any(k.startswith(("im2col", "gradbias")) for k in labels), labels      # no columns, no separate bias sum
+
+
+NARROW_FORWARD = [  # B, C, H, W, kH, kW, pH, pW, sH, sW: 64 output planes, at most 32 taps, unit column stride,
+    # Wo a multiple of 4, Ho*Wo a multiple of 128
+    (3, 3, 16, 16, 3, 3, 1, 1, 1, 1),     # K = 27: the first layer of a VGG-style stack, small
+    (2, 1, 19, 35, 4, 4, 0, 0, 1, 1),     # K = 16, unpadded: the input is read in place
+    (2, 2, 31, 16, 3, 3, 1, 1, 2, 1),     # K = 18, strided along the rows
+    (2, 2, 15, 17, 4, 4, 2, 1, 1, 1),     # K = 32: every step full
+    (3, 1, 16, 16, 5, 5, 2, 2, 1, 1),     # K = 25: an odd count (the last step holds one tap)
+    (1, 3, 32, 33, 3, 2, 1, 0, 1, 1),     # K = 18, a non-square kernel, one image
+    (2, 3, 31, 24, 3, 3, 1, 1, 2, 1),     # K = 27, rows of 24 positions: a group of 128 spans rows
+]
+
+
+@pytest.mark.parametrize("relu", [False, True], ids=["plain", "relu"])
+@pytest.mark.parametrize("cfg", NARROW_FORWARD)
+def test_layers_with_a_handful_of_taps_run_the_narrow_forward_kernel_integer_exact(gt, gathered_route, switches, cfg, relu):
+    """A layer with at most 32 taps and 64 output planes (the first layer of a VGG-style stack) computes its forward
+    pass with weights held in registers and no tiled GEMM (conv_narrow.hip).  On integer data the result equals the
+    oracle's bit for bit, with the bias added and, inside a fused stack, the ReLU applied on the way out; the timing
+    label shows which kernel ran; with the conv_narrow_off switch the tiled kernel gives the same values; memory around
+    the output is untouched."""
+    B, C, H, W, kH, kW, pH, pW, sH, sW = cfg
+    M, K = 64, C * kH * kW
+    geo = (kH, kW, pH, pW, sH, sW)
+    rng = rng_for(77 + K + H)
+    ints = lambda shape: rng.integers(-3, 4, shape).astype(np.float32)  # noqa: E731
+    x, w, b = ints((B, C, H, W)), ints((M, K)), ints((M,))
+    ref, _ = oracle.conv_updateOutput(x, w, b, *geo)
+    assert (ref.shape[2] * ref.shape[3]) % 128 == 0 and ref.shape[3] % 4 == 0 and sW == 1
+    if relu:
+        ref = oracle.threshold_updateOutput(ref)
+
+    def run():
+        conv = gt.nn.SpatialConvolutionMM(C, M, kW, kH, sW, sH, 0, padW=pW, padH=pH)
+        conv._assign("weight", w)
+        conv._assign("bias", b)
+        net = gt.nn.Sequential().add(conv)
+        if relu:
+            net.add(gt.nn.ReLU())
+        net.gpu()
+        if relu:
+            net.fuse()
+        # the output as a window of a larger buffer: guard planes before and behind it
+        big = dev(gt, np.full((B + 2,) + ref.shape[1:], 9.0, np.float32))
+        conv.output = big.narrow(0, 1, B)
+        gt.gputorch.prof_reset()
+        gt.gputorch.prof_enable(True)
+        try:
+            out = net.forward(dev(gt, x)).float()
+            gt.gputorch.synchronize()
+            labels = list(gt.gputorch.prof_report())
+        finally:
+            gt.gputorch.prof_enable(False)
+            gt.gputorch.prof_reset()
+        guard = big.float()
+        assert np.all(guard[0] == 9.0) and np.all(guard[-1] == 9.0)
+        return out, labels
+
+    out, labels = run()
+    assert np.array_equal(out, ref)
+    assert any(k.startswith("conv_narrow_fwd") for k in labels) and not any(k.startswith("gemm_conv_fwd") for k in labels), labels
+    switches("conv_narrow_off", "1")
+    tiled, labels = run()
+    assert np.array_equal(tiled, ref)
+    assert any(k.startswith("gemm_conv_fwd") for k in labels) and not any(k.startswith("conv_narrow") for k in labels), labels
+
+
+def test_narrow_forward_kernel_on_real_values_at_the_first_layer_of_the_vgg_stack(gt, gathered_route):
+    """3 -> 64 planes, 3x3, padding 1, on 224x224 images (batch 4): within 1e-4*sqrt(27) of the oracle, norm-wise and
+    element-wise."""
+    B, C, H, W, M = 4, 3, 224, 224, 64
+    rng = rng_for(781)
+    x = uniform(rng, (B, C, H, W))
+    w = uniform(rng, (M, 27)) / np.float32(np.sqrt(27))
+    b = uniform(rng, (M,))
+    ref, _ = oracle.conv_updateOutput(x, w, b, 3, 3, 1, 1, 1, 1)
+    conv = gt.nn.SpatialConvolutionMM(C, M, 3, 3, 1, 1, 1)
+    conv._assign("weight", w)
+    conv._assign("bias", b)
+    conv.gpu()
+    gt.gputorch.prof_reset()
+    gt.gputorch.prof_enable(True)
+    try:
+        out = conv.forward(dev(gt, x)).float()
+        labels = list(gt.gputorch.prof_report())
+    finally:
+        gt.gputorch.prof_enable(False)
+        gt.gputorch.prof_reset()
+    assert any(k.startswith("conv_narrow_fwd") for k in labels), labels
+    check_close("vgg first layer, narrow forward kernel", out, ref, 27)
