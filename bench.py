@@ -410,7 +410,9 @@ FAMILIES = [("gemm_fast", "gemm"), ("gemm_generic", "gemm"), ("im2col", "im2col"
             ("maxpool_bwd", "maxpool_bwd"), ("maxpool_fwd", "maxpool_fwd"), ("threshold_fwd", "threshold_fwd"),
             ("threshold_bwd", "threshold_bwd"), ("split_reduce", "gemm_split_reduce"),
             ("gradbias_partial", "gradbias"), ("gradbias_final", "gradbias_final"), ("fill_kernel", "fill"),
-            ("pad_planes", "pad_planes"), ("conv_narrow_forward", "conv_narrow_fwd")]
+            ("pad_planes", "pad_planes"), ("conv_narrow_forward", "conv_narrow_fwd"),
+            ("conv_narrow_gradweight_finish", "conv_narrow_gradweight_finish"),
+            ("conv_narrow_gradweight", "conv_narrow_gradweight")]
 
 
 def _family(kernel_name):

@@ -552,6 +552,13 @@ int conv_implicit_gradweight(const float *padded, const float *gradOutput, float
     const int Hp = H + 2 * pH, Wp = W + 2 * pW;
     const int Ho = (Hp - kH) / sH + 1, Wo = (Wp - kW) / sW + 1;
     if (trim_tables()) return 1;
+    if (conv_narrow_gradweight_fits(B, M, (long)C * kH * kW, Wo, (long)Ho * Wo, sW)) {
+        const int *taps = tap_table(C, kH, kW, Hp * Wp, Wp);
+        if (!taps) return 1;
+        if (bias_done) *bias_done = gradBias != nullptr;
+        return conv_narrow_gradweight(padded, (long)C * Hp * Wp, gradOutput, gradWeight, gradBias, B, M, C * kH * kW, Ho,
+                                      Wo, sH * Wp, taps, scale);
+    }
     GemmProblem p = gradweight_problem(B, C, H, W, M, kH, kW, pH, pW, sH, sW);
     p.A = gradOutput;
     p.B = padded;

@@ -148,6 +148,127 @@ __global__ __launch_bounds__(256, 2) void conv_narrow_forward_kernel(const Narro
     }
 }
 
+// ---- gradWeight of the same layers ----------------------------------------------------------------------------------
+// gradWeight[m][k] += scale * sum over images and positions n of gradOutput[m][n] * P[tap(k) + pixel(n)]: 64 x K results
+// from a reduction over every output position of the batch.  As a tiled GEMM it runs 64 columns wide for K taps, split
+// a thousand ways.  Here the work is what it is -- reading gradOutput once -- and the results never leave the
+// registers until the end: a wavefront owns a 64 x 32 block of accumulators (rows m, columns k) for the whole launch
+// and walks blocks of 32 positions; lane (i, h) fetches four consecutive positions of row i of gradOutput with one
+// 16-byte load (positions 4h .. 4h+3 of every eight: the first operand of four MFMA steps), lane (j, h) the same four
+// positions of the padded image at tap j (the second operand), so both operands pair the same positions.  The lanes
+// also add up what they fetch of gradOutput: the row sums are the bias gradient.  Every wavefront leaves its 64 x 32
+// partial sums and 64 x 2 partial row sums in the workspace, and a second small launch adds them in wavefront order
+// (a fixed order: results do not depend on timing) into gradWeight and gradBias.
+struct NarrowGradGeom {
+    const float *P;      // zero-padded images, image_stride floats apart
+    const float *go;     // gradOutput [B][64][N]
+    float *partial;      // [waves][64 * 32 + 64 * 2]
+    const int *rowtab;   // [K]
+    int K, N;
+    int row_step;
+    FastDiv divWo;
+    long image_stride;
+    unsigned blocks;     // B * N / 32
+    FastDiv divBlocksPerImage;
+};
+
+constexpr int kNarrowPartial = 64 * 32 + 64 * 2;
+
+__global__ __launch_bounds__(256) void conv_narrow_gradweight_kernel(const NarrowGradGeom g) {
+    const int lane = threadIdx.x & 63, col = lane & 31, half = lane >> 5;
+    const unsigned wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 4u + (threadIdx.x >> 6));
+    const unsigned waves = gridDim.x * 4u;
+    const unsigned tap = (unsigned)g.rowtab[col < g.K ? col : 0] * 4u;  // (columns beyond K: any valid tap; never stored)
+    // row `col` (+32) of gradOutput, positions 4*half on: byte offset within an image's gradOutput
+    const unsigned go_lane = ((unsigned)col * (unsigned)g.N + 4u * (unsigned)half) * 4u;
+
+    float4u av[2][4], bv[4];
+    auto request = [&](unsigned blk) {
+        unsigned img, bi;
+        g.divBlocksPerImage.divmod(blk, img, bi);
+        const char *rows = reinterpret_cast<const char *>(g.go + (long)img * 64 * g.N + (long)bi * 32);
+        const char *image = reinterpret_cast<const char *>(g.P + (long)img * g.image_stride);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {  // eight positions at a time: this half's four
+            av[0][c] = *reinterpret_cast<const float4u *>(rows + (go_lane + (unsigned)c * 32u));
+            av[1][c] = *reinterpret_cast<const float4u *>(rows + (go_lane + (unsigned)c * 32u + 32u * (unsigned)g.N * 4u));
+            unsigned y, x;
+            g.divWo.divmod(bi * 32u + (unsigned)c * 8u + 4u * (unsigned)half, y, x);  // (Wo is a multiple of 4: one row)
+            bv[c] = *reinterpret_cast<const float4u *>(image + ((y * (unsigned)g.row_step + x) * 4u + tap));
+        }
+    };
+
+    float16v acc[2];
+    float rowsum[2] = {0.0f, 0.0f};
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[rb][v] = 0.0f;
+    unsigned blk = wave;
+    if (blk < g.blocks) request(blk);
+    while (blk < g.blocks) {
+        float4u a[2][4], b[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            a[0][c] = av[0][c];
+            a[1][c] = av[1][c];
+            b[c] = bv[c];
+        }
+        const unsigned next = blk + waves;
+        if (next < g.blocks) request(next);  // the next block's operands are on their way during this block's MFMAs
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb) {
+                acc[rb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rb][c].x, b[c].x, acc[rb], 0, 0, 0);
+                acc[rb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rb][c].y, b[c].y, acc[rb], 0, 0, 0);
+                acc[rb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rb][c].z, b[c].z, acc[rb], 0, 0, 0);
+                acc[rb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rb][c].w, b[c].w, acc[rb], 0, 0, 0);
+                rowsum[rb] += (a[rb][c].x + a[rb][c].y) + (a[rb][c].z + a[rb][c].w);
+            }
+        }
+        blk = next;
+    }
+    // accumulator register v of lane (j, h): row 8*(v/4) + 4*h + v%4 (+32), column j
+    float *out = g.partial + (long)wave * kNarrowPartial;
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) out[(rb * 32 + 8 * (v / 4) + 4 * half + (v % 4)) * 32 + col] = acc[rb][v];
+        out[64 * 32 + (rb * 32 + col) * 2 + half] = rowsum[rb];
+    }
+}
+
+// gradWeight[m][k] += scale * (sum over wavefronts of partial[w][m][k]), gradBias[m] += scale * (sum of the row sums):
+// one wavefront per result, lanes striding the wavefronts' partial sums, then a butterfly over the lanes -- a fixed
+// order of additions.
+__global__ __launch_bounds__(256) void conv_narrow_gradweight_finish_kernel(const float *__restrict__ partial,
+                                                                            unsigned waves, int K, float scale,
+                                                                            float *__restrict__ gradWeight,
+                                                                            float *__restrict__ gradBias) {
+    const unsigned lane = threadIdx.x & 63u;
+    const unsigned result = blockIdx.x * 4u + (threadIdx.x >> 6);  // 64*K weight results, then 64 bias results
+    const unsigned nweights = 64u * (unsigned)K;
+    if (result >= nweights + (gradBias ? 64u : 0u)) return;
+    float sum = 0.0f;
+    if (result < nweights) {
+        const unsigned m = result / (unsigned)K, k = result % (unsigned)K;
+        for (unsigned w = lane; w < waves; w += 64u) sum += partial[(long)w * kNarrowPartial + m * 32u + k];
+    } else {
+        const unsigned m = result - nweights;
+        for (unsigned w = lane; w < waves; w += 64u) {
+            const float *p = partial + (long)w * kNarrowPartial + 64 * 32 + m * 2u;
+            sum += p[0] + p[1];
+        }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) sum += __shfl_xor(sum, off);
+    if (lane == 0) {
+        if (result < nweights) gradWeight[result] += scale * sum;
+        else gradBias[result - nweights] += scale * sum;
+    }
+}
+
 }  // namespace
 
 bool conv_narrow_forward_fits(long B, int M, long K, int Wo, long N, int col_step, OutputLayout out) {
@@ -215,6 +336,66 @@ int conv_narrow_forward(const float *padded, long image_stride, const float *wei
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), 0, s, g);
     }
     return check_launch("conv_narrow_forward");
+}
+
+bool conv_narrow_gradweight_fits(long B, int M, long K, int Wo, long N, int col_step) {
+    if (tuning().conv_narrow_off || tuning().gemm_tile[0] || tuning().gemm_split > 0) return false;
+    // 64 planes, at most 32 taps, unit column stride, rows of a multiple of 4 positions, planes of a multiple of 32
+    // positions, 32-bit byte offsets within an image's gradOutput
+    return M == 64 && K >= 1 && K <= 32 && col_step == 1 && Wo % 4 == 0 && N >= 32 && N % 32 == 0 &&
+           64L * N * 4 < (1L << 31) && B * (N / 32) < (1L << 31) && B >= 1;
+}
+
+int conv_narrow_gradweight(const float *padded, long image_stride, const float *gradOutput, float *gradWeight,
+                           float *gradBias, long B, int M, int K, int Ho, int Wo, int row_step, const int *rowtab,
+                           float scale) {
+    hipStream_t s = stream();
+    if (!s) return 1;
+    if (!padded || !gradOutput || !gradWeight || !rowtab) return fail("conv_narrow_gradweight: null operand");
+    const int N = Ho * Wo;
+    NarrowGradGeom g;
+    g.P = padded;
+    g.go = gradOutput;
+    g.rowtab = rowtab;
+    g.K = K;
+    g.N = N;
+    g.row_step = row_step;
+    g.divWo = FastDiv((uint32_t)Wo);
+    g.image_stride = image_stride;
+    g.blocks = (unsigned)(B * (N / 32));
+    g.divBlocksPerImage = FastDiv((uint32_t)(N / 32));
+    // ONE workgroup per CU (a wavefront per SIMD, the next block's operands always in flight).  More resident
+    // wavefronts are slower here, measured: 0.186 ms with one workgroup per CU, 0.236 with two, 0.245 with three on
+    // 64 x 3 x 224 x 224 -- every wavefront reads 64 rows of gradOutput at once, 200 KB apart, and the more of them are
+    // in flight the further apart in time the requests to one DRAM page arrive.
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        THGPU_HIP_TRY(hipGetDevice(&dev));
+        THGPU_HIP_TRY(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
+        cus = n > 0 ? n : 256;
+    }
+    unsigned grid = (unsigned)cus;
+    const unsigned need = (g.blocks + 3u) / 4u;
+    if (grid > need) grid = need;
+    const unsigned waves = grid * 4u;
+    g.partial = workspace((size_t)waves * kNarrowPartial * sizeof(float));
+    if (!g.partial) return 1;
+    {
+        const double bytes = 4.0 * ((double)B * M * N + (double)B * image_stride + (double)waves * kNarrowPartial);
+        const char *label = prof_enabled() ? prof_label("conv_narrow_gradweight M=%d J=%d R=%ld", M, K, B * (long)N)
+                                           : "conv_narrow_gradweight";
+        LaunchScope scope(label, 2.0 * M * (double)K * (double)B * N, bytes);  // (the layer's flops; bound by its loads)
+        hipLaunchKernelGGL(conv_narrow_gradweight_kernel, dim3(grid), dim3(256), 0, s, g);
+    }
+    if (check_launch("conv_narrow_gradweight")) return 1;
+    {
+        const unsigned results = 64u * (unsigned)K + (gradBias ? 64u : 0u);
+        LaunchScope scope("conv_narrow_gradweight_finish", 0.0, 4.0 * ((double)waves * kNarrowPartial + 2.0 * results));
+        hipLaunchKernelGGL(conv_narrow_gradweight_finish_kernel, dim3((results + 3u) / 4u), dim3(256), 0, s, g.partial, waves,
+                           K, scale, gradWeight, gradBias);
+    }
+    return check_launch("conv_narrow_gradweight_finish");
 }
 
 }  // namespace thgpu

@@ -299,8 +299,9 @@ int gemm_launch(const GemmProblem &p) {
     g.mask_sC = p.mask_sC ? p.mask_sC : p.sC;
     g.mask_bsC = p.mask_bsC ? p.mask_bsC : p.bsC;
     g.divCW = FastDiv((uint32_t)g.c_w);
-    if (p.j_store > 0 && (!red || p.j_store > p.J || p.sC < p.j_store || p.C2 || p.scatter))
-        return fail("gemm: scratch columns need reduction batching and a row pitch of C that holds the stored ones");
+    // (reduction batching or one image: either way every column of the product is a column of C or scratch)
+    if (p.j_store > 0 && (p.N != p.J || p.j_store > p.J || p.sC < p.j_store || p.C2 || p.scatter))
+        return fail("gemm: scratch columns need an unbatched column index and a row pitch of C that holds the stored ones");
     if (p.C2) {
         if (red || p.scatter || p.c_w <= 0 || g.N % p.c_w != 0 || p.c2_pitch < p.c_w || p.c2_sC <= 0 || p.c2_bsC <= 0)
             return fail("gemm: a second copy of the result needs column batching, a plane width and the copy's strides");

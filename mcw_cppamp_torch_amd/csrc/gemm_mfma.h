@@ -79,8 +79,8 @@ struct GemmProblem {
     // when it is false the caller computes the sums itself.
     float *rowsum = nullptr;
     bool *rowsum_done = nullptr;
-    // Reduction batching only: the product is computed J columns wide but only the first j_store of them exist in C
-    // (rows of C are sC >= j_store floats apart); the rest are scratch.  This is how a product with fewer columns than
+    // Products whose columns are not batched over images (N == J: gradWeight): computed J columns wide, but only the
+    // first j_store of them exist in C (rows of C are sC >= j_store floats apart); the rest are scratch.  This is how a product with fewer columns than
     // the narrowest tile runs on the tiled kernels: its column table is padded with entries that repeat a valid one.
     // The reduction is always split (the partial sums are J wide, the final pass stores j_store).  0: all J columns.
     int j_store = 0;

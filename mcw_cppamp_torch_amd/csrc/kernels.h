@@ -77,6 +77,12 @@ int conv_implicit_forward(const float *padded, const float *weight, const float 
 bool conv_narrow_forward_fits(long B, int M, long K, int Wo, long N, int col_step, OutputLayout out);
 int conv_narrow_forward(const float *padded, long image_stride, const float *weight, const float *bias, float *output,
                         long B, int M, int K, int Ho, int Wo, int row_step, const int *rowtab, OutputThreshold act);
+// ... and its gradWeight (+= scale * sums over the batch) with gradBias (+= scale * row sums of gradOutput; may be
+// null), gradOutput dense [B][64][Ho*Wo].
+bool conv_narrow_gradweight_fits(long B, int M, long K, int Wo, long N, int col_step);
+int conv_narrow_gradweight(const float *padded, long image_stride, const float *gradOutput, float *gradWeight,
+                           float *gradBias, long B, int M, int K, int Ho, int Wo, int row_step, const int *rowtab,
+                           float scale);
 // gradBias (may be null) receives scale * the sums of gradOutput over images and positions when the product can
 // compute them on the side; *bias_done says whether it did.
 int conv_implicit_gradweight(const float *padded, const float *gradOutput, float *gradWeight, long B, int C, int H,

@@ -530,12 +530,14 @@ def test_strided_gradinput_short_row_kernel_integer_exact(gt, gathered_route, sw
 
 @pytest.mark.parametrize("split", [None, 2, 7])
 @pytest.mark.parametrize("cfg", [(4, 3, 40, 36, 64, 3, 3, 1, 1, 1, 1), (3, 1, 33, 35, 128, 5, 5, 2, 2, 1, 1),
-                                 (5, 3, 31, 29, 70, 4, 4, 1, 1, 2, 2), (2, 3, 64, 48, 128, 7, 3, 3, 1, 2, 1)])
+                                 (5, 3, 31, 29, 70, 4, 4, 1, 1, 2, 2), (2, 3, 64, 48, 128, 7, 3, 3, 1, 2, 1),
+                                 (1, 3, 40, 36, 64, 3, 3, 1, 1, 1, 1)])     # (the last: one image, no batched reduction)
 def test_narrow_gradweight_runs_wide_and_stores_its_own_columns_integer_exact(gt, gathered_route, switches, cfg, split):
     """A layer with fewer than 64 taps (K = C*kH*kW: a first layer with 3x3 or 5x5 kernels) has a gradWeight product
     narrower than the narrowest GEMM tile.  It runs 64 columns wide on a padded tap table and the split reduction's
     final pass stores the first K columns only: on integer data every result equals the oracle's bit for bit, gradBias
     (summed on the side by the same product) included, and what lies around gradWeight in memory is untouched."""
+    switches("conv_narrow_off", "1")      # (this test is about the tiled product; conv_narrow.hip has its own below)
     if split is not None:
         switches("gemm_split", split)
     B, C, H, W, M, kH, kW, pH, pW, sH, sW = cfg
@@ -577,7 +579,8 @@ def test_narrow_gradweight_runs_wide_and_stores_its_own_columns_integer_exact(gt
     assert np.array_equal(m.gradBias.float(), gb_ref)
     gw_label = [k for k in labels if k.startswith("gemm_conv_gradweight")]
     assert len(gw_label) == 1 and "J=64 " in gw_label[0] and "tile=64x64" in gw_label[0] and "split=1 " not in gw_label[0] + " ", labels
-    assert not any(k.startswith(("im2col", "gradbias")) for k in labels), labels      # no columns, no separate bias sum
+    # no columns; no separate bias sum either where the reduction runs over a batch (one image: the two-stage sum)
+    assert not any(k.startswith(("im2col",) + (("gradbias",) if B > 1 else ())) for k in labels), labels
 
 
 NARROW_FORWARD = [  # B, C, H, W, kH, kW, pH, pW, sH, sW: 64 output planes, at most 32 taps, unit column stride,
@@ -669,3 +672,81 @@ def test_narrow_forward_kernel_on_real_values_at_the_first_layer_of_the_vgg_stac
         gt.gputorch.prof_reset()
     assert any(k.startswith("conv_narrow_fwd") for k in labels), labels
     check_close("vgg first layer, narrow forward kernel", out, ref, 27)
+
+
+NARROW_GRADWEIGHT = NARROW_FORWARD + [
+    (4, 3, 40, 36, 3, 3, 1, 1, 1, 1),     # Ho*Wo = 1440: a multiple of 32 that is none of 128
+    (130, 1, 5, 9, 4, 4, 1, 1, 1, 1),     # 32 positions per image, 130 images: one block per image
+]
+
+
+@pytest.mark.parametrize("cfg", NARROW_GRADWEIGHT)
+def test_layers_with_a_handful_of_taps_run_the_narrow_gradweight_kernels_integer_exact(gt, gathered_route, switches, cfg):
+    """gradWeight and gradBias of a layer with at most 32 taps and 64 output planes: partial sums per wavefront in
+    registers, added up by a second launch (conv_narrow.hip).  On integer data both equal the oracle's bit for bit,
+    accumulated onto what the tensors held, scaled; memory around gradWeight is untouched; two runs give identical
+    bits; the timing labels show which kernels ran and that no tiled product, im2col or separate bias sum did."""
+    B, C, H, W, kH, kW, pH, pW, sH, sW = cfg
+    M, K = 64, C * kH * kW
+    geo = (kH, kW, pH, pW, sH, sW)
+    rng = rng_for(177 + K + H)
+    ints = lambda shape: rng.integers(-3, 4, shape).astype(np.float32)  # noqa: E731
+    x, w, b = ints((B, C, H, W)), ints((M, K)), ints((M,))
+    gw0, gb0 = ints((M, K)), ints((M,))
+    out_ref, finput_ref = oracle.conv_updateOutput(x, w, b, *geo)
+    go = ints(out_ref.shape)
+    gw_ref, gb_ref = gw0.copy(), gb0.copy()
+    oracle.conv_accGradParameters(go, finput_ref, gw_ref, gb_ref, 2.0)
+    results = []
+    for _ in range(2):
+        m = gt.nn.SpatialConvolutionMM(C, M, kW, kH, sW, sH, 0, padW=pW, padH=pH)
+        m._assign("weight", w)
+        m._assign("bias", b)
+        m.gpu()
+        big = dev(gt, np.full((M + 2, K), 9.0, np.float32))
+        m.gradWeight = big.narrow(0, 1, M)
+        m.gradWeight.copy(gw0)
+        m.gradBias.copy(gb0)
+        dx, dgo = dev(gt, x), dev(gt, go)
+        gt.gputorch.prof_reset()
+        gt.gputorch.prof_enable(True)
+        try:
+            m.accGradParameters(dx, dgo, 2.0)          # (without a forward pass: the padded input is rebuilt)
+            gt.gputorch.synchronize()
+            labels = list(gt.gputorch.prof_report())
+        finally:
+            gt.gputorch.prof_enable(False)
+            gt.gputorch.prof_reset()
+        got = big.float()
+        assert np.array_equal(got[1:-1], gw_ref) and np.all(got[0] == 9.0) and np.all(got[-1] == 9.0)
+        assert np.array_equal(m.gradBias.float(), gb_ref)
+        assert any(k.startswith("conv_narrow_gradweight ") for k in labels) and "conv_narrow_gradweight_finish" in labels, labels
+        assert not any(k.startswith(("gemm_", "im2col", "gradbias")) for k in labels), labels
+        results.append((got.copy(), m.gradBias.float()))
+    assert np.array_equal(results[0][0], results[1][0]) and np.array_equal(results[0][1], results[1][1])
+
+
+def test_narrow_gradweight_kernels_on_real_values_at_the_first_layer_of_the_vgg_stack(gt, gathered_route):
+    """3 -> 64 planes, 3x3, padding 1, on 224x224 images (batch 4): gradWeight and gradBias within 1e-4*sqrt(B*N) of the
+    oracle, norm-wise and element-wise."""
+    B, C, H, W, M = 4, 3, 224, 224, 64
+    rng = rng_for(782)
+    x = uniform(rng, (B, C, H, W))
+    w = uniform(rng, (M, 27)) / np.float32(np.sqrt(27))
+    b = uniform(rng, (M,))
+    out_ref, finput_ref = oracle.conv_updateOutput(x, w, b, 3, 3, 1, 1, 1, 1)
+    go = uniform(rng, out_ref.shape)
+    gw_ref, gb_ref = np.zeros((M, 27), np.float32), np.zeros((M,), np.float32)
+    oracle.use_blas(True)
+    try:
+        oracle.conv_accGradParameters(go, finput_ref, gw_ref, gb_ref, 1.0)
+    finally:
+        oracle.use_blas(False)
+    conv = gt.nn.SpatialConvolutionMM(C, M, 3, 3, 1, 1, 1)
+    conv._assign("weight", w)
+    conv._assign("bias", b)
+    conv.gpu()
+    conv.zeroGradParameters()
+    conv.accGradParameters(dev(gt, x), dev(gt, go), 1.0)
+    check_close("vgg first layer gradWeight, narrow kernels", conv.gradWeight.float(), gw_ref, B * H * W)
+    check_close("vgg first layer gradBias, narrow kernels", conv.gradBias.float(), gb_ref, B * H * W)
