@@ -111,10 +111,13 @@ int thgpu_init(void);
 
 /* Testing and tuning switches (no counterpart in the reference).  name: gemm_tile (a tile configuration such
  * as "128x128"), gemm_split (a reduction split count), im2col_kernel (unit | strip | direct), im2col_plan
- * ("v,PL,TG"), col2im_generic ("1"), pool_fwd_wave ("1"), pool_bwd_direct ("1"), pool_bwd_tile ("1"), pool_bwd_cell ("1"), pool_bwd_pixels (pixels per workgroup of the staged
- * max-pool backward kernel, which it also pins), gradbias_separate ("1"); value NULL or "" restores the
- * library's own choice.  The environment variables THGPU_GEMM_TILE, THGPU_GEMM_SPLIT, THGPU_IM2COL_KERNEL,
- * THGPU_IM2COL_PLAN, THGPU_COL2IM_GENERIC, THGPU_POOL_FWD_WAVE, THGPU_POOL_BWD_DIRECT, THGPU_POOL_BWD_TILE, THGPU_POOL_BWD_CELL, THGPU_POOL_BWD_PIXELS and THGPU_GRADBIAS_SEPARATE give the initial values and are read once, when the library
+ * ("v,PL,TG"), col2im_generic ("1"), pool_fwd_wave ("1"), pool_bwd_direct ("1"), pool_bwd_tile ("1"),
+ * pool_bwd_cell ("1"), pool_bwd_pixels (pixels per workgroup of the staged max-pool backward kernel, which it also
+ * pins), gradbias_separate ("1"), conv_narrow_off ("1": the tiled GEMM kernels where the kernels for layers with at
+ * most 32 taps would run); value NULL or "" restores the library's own choice.  The environment variables
+ * THGPU_GEMM_TILE, THGPU_GEMM_SPLIT, THGPU_IM2COL_KERNEL, THGPU_IM2COL_PLAN, THGPU_COL2IM_GENERIC,
+ * THGPU_POOL_FWD_WAVE, THGPU_POOL_BWD_DIRECT, THGPU_POOL_BWD_TILE, THGPU_POOL_BWD_CELL, THGPU_POOL_BWD_PIXELS,
+ * THGPU_GRADBIAS_SEPARATE and THGPU_CONV_NARROW_OFF give the initial values and are read once, when the library
  * initialises; no operator call reads the environment. */
 int thgpu_debug_set(const char *name, const char *value);
 
