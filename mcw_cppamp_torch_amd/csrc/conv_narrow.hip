@@ -319,14 +319,7 @@ int conv_narrow_forward(const float *padded, long image_stride, const float *wei
     // ONE workgroup per CU (measured on 64 x 3 x 224 x 224: 0.184 ms; two per CU, which the registers allow, 0.193;
     // every wavefront writes 64 planes at once, and more of them in flight spread the requests to one DRAM page
     // further apart in time).
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        THGPU_HIP_TRY(hipGetDevice(&dev));
-        THGPU_HIP_TRY(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
-        cus = n > 0 ? n : 256;
-    }
-    unsigned grid = (unsigned)cus;
+    unsigned grid = (unsigned)num_cus();
     const unsigned need = (g.groups + 3u) / 4u;
     if (grid > need) grid = need;
     {
@@ -368,14 +361,7 @@ int conv_narrow_gradweight(const float *padded, long image_stride, const float *
     // wavefronts are slower here, measured: 0.186 ms with one workgroup per CU, 0.236 with two, 0.245 with three on
     // 64 x 3 x 224 x 224 -- every wavefront reads 64 rows of gradOutput at once, 200 KB apart, and the more of them are
     // in flight the further apart in time the requests to one DRAM page arrive.
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        THGPU_HIP_TRY(hipGetDevice(&dev));
-        THGPU_HIP_TRY(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
-        cus = n > 0 ? n : 256;
-    }
-    unsigned grid = (unsigned)cus;
+    unsigned grid = (unsigned)num_cus();
     const unsigned need = (g.blocks + 3u) / 4u;
     if (grid > need) grid = need;
     const unsigned waves = grid * 4u;
