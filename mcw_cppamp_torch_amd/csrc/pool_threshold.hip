@@ -559,9 +559,9 @@ __global__ __launch_bounds__(256) void maxpool_bwd_cell_kernel(const float *__re
 }
 
 // The staged kernel: the cell kernel's arithmetic with the tile kernel's memory streams, the default for the window
-// shapes of the benchmark stacks.  Counters showed what holds the cell kernel back: its stores -- 8 bytes per lane,
-// rows of W floats that start anywhere -- reach the L2 as requests of 29 bytes on average, 2.2 times as many as the
-// data needs, and the request rate, not the byte rate, is what saturates.  Here a workgroup owns a contiguous range
+// shapes of the benchmark stacks.  The cell kernel's stores -- 8 bytes per lane, rows of W floats that start
+// anywhere -- reach the L2 as requests of 29 bytes on average, 2.2 times as many as the data needs (counters), and
+// on launches large enough to stream from memory that costs it 10 - 20 %.  Here a workgroup owns a contiguous range
 // of pixels (a group of small planes, or a strip of rows of a large one), its lanes compute the range's cells exactly
 // as the cell kernel does (every load requested up front, no zero-fill, no scatter phases), park the results in LDS,
 // and after ONE barrier the range leaves as one contiguous stream of full-width requests, the mask (requested first,
