@@ -750,3 +750,55 @@ def test_narrow_gradweight_kernels_on_real_values_at_the_first_layer_of_the_vgg_
     conv.accGradParameters(dev(gt, x), dev(gt, go), 1.0)
     check_close("vgg first layer gradWeight, narrow kernels", conv.gradWeight.float(), gw_ref, B * H * W)
     check_close("vgg first layer gradBias, narrow kernels", conv.gradBias.float(), gb_ref, B * H * W)
+
+
+def narrow_draws(count):
+    """Seeded random layers with 64 output planes and 16 .. 32 taps; about a third of them have the shape the kernels of
+    conv_narrow.hip take (unit column stride, Wo a multiple of 4, Ho*Wo a multiple of 32 or 128), the rest run the tiled
+    products for layers with fewer than 64 taps."""
+    rng = rng_for(4242)
+    out = []
+    while len(out) < count:
+        it = len(out)
+        C, kH, kW = int(rng.integers(1, 5)), int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        if not 16 <= C * kH * kW <= 32:
+            continue
+        pH, pW = int(rng.integers(0, kH)), int(rng.integers(0, kW))
+        sH, sW = int(rng.integers(1, 3)), int(rng.choice([1, 1, 1, 2]))
+        Wo = int(rng.integers(1, 12)) * (4 if it % 5 else 3)
+        Ho = int(rng.integers(1, 40))
+        if it % 3 == 0:
+            Ho = max(1, (128 // int(np.gcd(128, Wo))) * int(rng.integers(1, 3)))   # Ho*Wo a multiple of 128
+        H, W = (Ho - 1) * sH + kH - 2 * pH, (Wo - 1) * sW + kW - 2 * pW
+        if H < 1 or W < 1:
+            continue
+        B = 1 if it % 4 == 0 else int(rng.integers(2, 4))
+        out.append((B, C, H, W, kH, kW, pH, pW, sH, sW))
+    return out
+
+
+@pytest.mark.parametrize("cfg", narrow_draws(48))
+def test_random_layers_with_a_handful_of_taps_integer_exact(gt, gathered_route, cfg):
+    """Forward and accGradParameters of 48 seeded random layers with 16 .. 32 taps and 64 output planes (a quarter of
+    them single images) on integer data: output, gradWeight and gradBias bit for bit against the oracle, whichever
+    kernels the library picks for the shape."""
+    B, C, H, W, kH, kW, pH, pW, sH, sW = cfg
+    K = C * kH * kW
+    geo = (kH, kW, pH, pW, sH, sW)
+    rng = rng_for(9000 + 31 * H + W + K)
+    ints = lambda shape: rng.integers(-3, 4, shape).astype(np.float32)  # noqa: E731
+    x, w, b = ints((B, C, H, W)), ints((64, K)), ints((64,))
+    ref, finput_ref = oracle.conv_updateOutput(x, w, b, *geo)
+    go, gw, gb = ints(ref.shape), ints((64, K)), ints((64,))
+    m = gt.nn.SpatialConvolutionMM(C, 64, kW, kH, sW, sH, 0, padW=pW, padH=pH)
+    m._assign("weight", w)
+    m._assign("bias", b)
+    m.gpu()
+    m.gradWeight.copy(gw)
+    m.gradBias.copy(gb)
+    dx = dev(gt, x)
+    out = m.forward(dx).float()
+    assert out.shape == ref.shape and np.array_equal(out, ref)
+    oracle.conv_accGradParameters(go, finput_ref, gw, gb, 3.0)
+    m.accGradParameters(dx, dev(gt, go), 3.0)
+    assert np.array_equal(m.gradWeight.float(), gw) and np.array_equal(m.gradBias.float(), gb)
